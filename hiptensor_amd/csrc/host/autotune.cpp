@@ -1,0 +1,140 @@
+// Measured selection for HIPTENSOR_ALGO_DEFAULT_PATIENT: runs the cost model's leading
+// candidates on scratch tensors and keeps the fastest.
+//
+// The reference's bruteForceModel (library/src/contraction/contraction_selection.cpp:
+// 44-195) times every registered kernel once; it sizes its scratch by the product of
+// extents, which under-allocates padded layouts.  Here only the top few candidates run,
+// scratch is sized by the span each tensor really covers, and each candidate gets one
+// warm-up and three timed launches.
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include <hip/hip_runtime_api.h>
+
+#include "handle.hpp"
+
+namespace hipta
+{
+    size_t time_choices(const Handle& h, const GemmView& v, const std::vector<Choice>& ranked, size_t top, std::string& trace)
+    {
+        (void)h;
+        const size_t n = std::min(top, ranked.size());
+        if(n <= 1)
+            return 0;
+        const size_t eb    = (size_t)v.elem_bytes;
+        const size_t spanX = (size_t)(v.swapped ? v.spanB : v.spanA) * eb;
+        const size_t spanY = (size_t)(v.swapped ? v.spanA : v.spanB) * eb;
+        const size_t spanD = (size_t)v.spanD * eb;
+        const size_t spanC = (size_t)v.spanC * eb;
+        uint64_t     ws    = 0;
+        for(size_t i = 0; i < n; i++)
+            ws = std::max<uint64_t>(ws, ranked[i].ws_bytes);
+
+        // tables
+        const std::vector<int32_t>* tabs[8] = {&v.xp, &v.xk, &v.yq, &v.yk, &v.cp, &v.cq, &v.dp, &v.dq};
+        size_t                      total = 0, offs[8];
+        for(int i = 0; i < 8; i++)
+        {
+            offs[i] = total;
+            total += (tabs[i]->size() + 63) / 64 * 64;
+        }
+        std::vector<int32_t> host(total, 0);
+        for(int i = 0; i < 8; i++)
+            std::copy(tabs[i]->begin(), tabs[i]->end(), host.begin() + (long)offs[i]);
+
+        void *dX = nullptr, *dY = nullptr, *dC = nullptr, *dD = nullptr, *dW = nullptr, *dT = nullptr;
+        auto  release = [&]() {
+            for(void* p : {dX, dY, dC, dD, dW, dT})
+                if(p)
+                    (void)hipFree(p);
+        };
+        bool ok = hipMalloc(&dX, std::max<size_t>(spanX, 16)) == hipSuccess
+                  && hipMalloc(&dY, std::max<size_t>(spanY, 16)) == hipSuccess
+                  && hipMalloc(&dD, std::max<size_t>(spanD, 16)) == hipSuccess
+                  && hipMalloc(&dT, total * sizeof(int32_t)) == hipSuccess
+                  && (!v.bilinear || hipMalloc(&dC, std::max<size_t>(spanC, 16)) == hipSuccess)
+                  && (ws == 0 || hipMalloc(&dW, ws) == hipSuccess);
+        if(ok)
+            ok = hipMemset(dX, 0, std::max<size_t>(spanX, 16)) == hipSuccess
+                 && hipMemset(dY, 0, std::max<size_t>(spanY, 16)) == hipSuccess
+                 && (!v.bilinear || hipMemset(dC, 0, std::max<size_t>(spanC, 16)) == hipSuccess)
+                 && hipMemcpy(dT, host.data(), total * sizeof(int32_t), hipMemcpyHostToDevice) == hipSuccess;
+        if(!ok)
+        {
+            release();
+            (void)hipGetLastError();
+            return 0;
+        }
+        const int32_t*  base = (const int32_t*)dT;
+        hiptk_problem_t p{};
+        p.cls     = v.cls;
+        p.op      = v.bilinear ? HIPTK_OP_BILINEAR : HIPTK_OP_SCALE;
+        p.P       = v.P;
+        p.Q       = v.Q;
+        p.K       = v.K;
+        p.x_kfast = v.x_kfast;
+        p.y_kfast = v.y_kfast;
+        p.x_vec   = v.x_vec;
+        p.y_vec   = v.y_vec;
+        p.cd_vec  = v.cd_vec;
+        p.xp      = base + offs[0];
+        p.xk      = base + offs[1];
+        p.yq      = base + offs[2];
+        p.yk      = base + offs[3];
+        p.cp      = v.bilinear ? base + offs[4] : nullptr;
+        p.cq      = v.bilinear ? base + offs[5] : nullptr;
+        p.dp      = base + offs[6];
+        p.dq      = base + offs[7];
+
+        alignas(16) double one[2]  = {0, 0};
+        alignas(16) float  onef[2] = {1.f, 0.f};
+        one[0]                     = 1.0;
+        const bool  dbl    = v.cls == HIPTK_F64 || v.cls == HIPTK_F64_AS_F32 || v.cls == HIPTK_C64;
+        const void* scalar = dbl ? (const void*)one : (const void*)onef;
+
+        hipEvent_t e0, e1;
+        if(hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
+        {
+            release();
+            return 0;
+        }
+        size_t best   = 0;
+        float  bestMs = 1e30f;
+        char   line[160];
+        for(size_t i = 0; i < n; i++)
+        {
+            p.tile_id = ranked[i].sol->tile_id;
+            p.split_k = ranked[i].split_k;
+            int  herr = 0;
+            bool good = hiptk_contract(&p, scalar, scalar, dX, dY, dC, dD, dW, ws, nullptr, &herr) == HIPTK_OK;
+            (void)hipEventRecord(e0, nullptr);
+            for(int r = 0; r < 3 && good; r++)
+                good = hiptk_contract(&p, scalar, scalar, dX, dY, dC, dD, dW, ws, nullptr, &herr) == HIPTK_OK;
+            (void)hipEventRecord(e1, nullptr);
+            (void)hipEventSynchronize(e1);
+            float ms = 0.f;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            ms /= 3.f;
+            snprintf(line,
+                     sizeof(line),
+                     "%sKernelName: %s splitK: %d measured: %0.3f us estimate: %0.3f us",
+                     trace.empty() ? "" : "; ",
+                     ranked[i].sol->name.c_str(),
+                     ranked[i].split_k,
+                     good ? ms * 1e3 : -1.0,
+                     ranked[i].est_us);
+            trace += line;
+            if(good && ms < bestMs)
+            {
+                bestMs = ms;
+                best   = i;
+            }
+        }
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+        release();
+        return best;
+    }
+}

@@ -1,0 +1,426 @@
+#include "planner.hpp"
+
+#include <algorithm>
+#include <cstdio>
+
+#include "hiptk_kernels.h"
+
+namespace hipta
+{
+    namespace
+    {
+        // hipDataType values (hip/library_types.h)
+        enum
+        {
+            DT_R32F  = 0,
+            DT_R64F  = 1,
+            DT_R16F  = 2,
+            DT_C32F  = 4,
+            DT_C64F  = 5,
+            DT_R16BF = 14
+        };
+        // hiptensorComputeType_t values
+        enum
+        {
+            CT_16F  = 1,
+            CT_32F  = 4,
+            CT_64F  = 16,
+            CT_16BF = 1024,
+            CT_C32F = 2048,
+            CT_C64F = 4096
+        };
+
+        int find_mode(const std::vector<int32_t>& modes, int32_t m)
+        {
+            for(size_t i = 0; i < modes.size(); i++)
+                if(modes[i] == m)
+                    return (int)i;
+            return -1;
+        }
+
+        bool has_repeats(const std::vector<int32_t>& modes)
+        {
+            for(size_t i = 0; i < modes.size(); i++)
+                for(size_t j = i + 1; j < modes.size(); j++)
+                    if(modes[i] == modes[j])
+                        return true;
+            return false;
+        }
+
+        enum Group
+        {
+            GP,
+            GQ,
+            GK
+        };
+
+        // Merge dims i and i+1 (i is faster) when every tensor that carries them steps
+        // through both with one stride.
+        void fuse(std::vector<Dim>& d, Group g, bool bilinear)
+        {
+            size_t i = 0;
+            while(i + 1 < d.size())
+            {
+                const Dim& a = d[i];
+                const Dim& b = d[i + 1];
+                bool       ok;
+                if(g == GK)
+                    ok = b.sx == a.sx * a.len && b.sy == a.sy * a.len;
+                else
+                {
+                    ok = (g == GP ? b.sx == a.sx * a.len : b.sy == a.sy * a.len)
+                         && b.sd == a.sd * a.len && (!bilinear || b.sc == a.sc * a.len);
+                }
+                if(ok)
+                {
+                    d[i].len *= b.len;
+                    d.erase(d.begin() + (long)i + 1);
+                }
+                else
+                    i++;
+            }
+        }
+
+        int64_t extent(const std::vector<Dim>& d)
+        {
+            int64_t e = 1;
+            for(const Dim& x : d)
+                e *= x.len;
+            return e;
+        }
+
+        template <typename Get>
+        bool make_table(const std::vector<Dim>& d, int64_t n, size_t padded, Get get, std::vector<int32_t>& out, int64_t& maxoff)
+        {
+            out.assign(padded, 0);
+            std::vector<int64_t> idx(d.size(), 0);
+            int64_t              off = 0;
+            maxoff                   = 0;
+            for(int64_t i = 0; i < n; i++)
+            {
+                if(off > 0x7FFFFFFFll)
+                    return false;
+                out[(size_t)i] = (int32_t)off;
+                maxoff         = std::max(maxoff, off);
+                // odometer increment, fastest dim first
+                for(size_t k = 0; k < d.size(); k++)
+                {
+                    off += get(d[k]);
+                    if(++idx[k] < d[k].len)
+                        break;
+                    off -= get(d[k]) * d[k].len;
+                    idx[k] = 0;
+                }
+            }
+            return true;
+        }
+
+        // Widest power-of-two vector (<= maxv elements) that stays inside the leading
+        // dim's contiguous run and keeps every vector start aligned.
+        int vector_width(int64_t lead_len, const std::vector<int64_t>& other_strides, uint32_t align_bytes, int elem_bytes, int maxv)
+        {
+            for(int v = maxv; v > 1; v /= 2)
+            {
+                if(lead_len % v != 0)
+                    continue;
+                if((uint32_t)(v * elem_bytes) > align_bytes)
+                    continue;
+                bool ok = true;
+                for(int64_t s : other_strides)
+                    if(s % v != 0)
+                        ok = false;
+                if(ok)
+                    return v;
+            }
+            return 1;
+        }
+    }
+
+    int64_t span_elems(const std::vector<int64_t>& len, const std::vector<int64_t>& stride)
+    {
+        int64_t e = 1;
+        for(size_t i = 0; i < len.size(); i++)
+        {
+            if(len[i] <= 0)
+                return 0;
+            e += (len[i] - 1) * (i < stride.size() ? stride[i] : 0);
+        }
+        return e;
+    }
+
+    int kernel_class(int typeA, int typeB, int typeC, int typeD, bool bilinear, int compute)
+    {
+        if(typeA != typeB || typeA != typeD || (bilinear && typeC != typeA))
+            return -1;
+        switch(typeA)
+        {
+        case DT_R16F: return compute == CT_32F ? HIPTK_F16 : -1;
+        case DT_R16BF: return compute == CT_32F ? HIPTK_BF16 : -1;
+        case DT_R32F:
+            if(compute == CT_32F)
+                return HIPTK_F32;
+            if(compute == CT_16F)
+                return HIPTK_F32_AS_F16;
+            if(compute == CT_16BF)
+                return HIPTK_F32_AS_BF16;
+            return -1;
+        case DT_R64F:
+            if(compute == CT_64F)
+                return HIPTK_F64;
+            if(compute == CT_32F)
+                return HIPTK_F64_AS_F32;
+            return -1;
+        case DT_C32F: return compute == CT_C32F ? HIPTK_C32 : -1;
+        case DT_C64F: return compute == CT_C64F ? HIPTK_C64 : -1;
+        default: return -1;
+        }
+    }
+
+    int class_elem_bytes(int cls)
+    {
+        switch(cls)
+        {
+        case HIPTK_F16:
+        case HIPTK_BF16: return 2;
+        case HIPTK_F32:
+        case HIPTK_F32_AS_F16:
+        case HIPTK_F32_AS_BF16: return 4;
+        case HIPTK_F64:
+        case HIPTK_F64_AS_F32:
+        case HIPTK_C32: return 8;
+        case HIPTK_C64: return 16;
+        default: return 0;
+        }
+    }
+
+    int class_max_vec(int cls)
+    {
+        const int b = class_elem_bytes(cls);
+        return b ? 16 / b : 1;
+    }
+
+    PlanStatus build_view(const ProblemIn& in, GemmView& v, std::string& why)
+    {
+        v          = GemmView();
+        v.bilinear = in.bilinear;
+        v.cls      = kernel_class(in.A.dtype, in.B.dtype, in.C.dtype, in.D.dtype, in.bilinear, in.compute);
+        if(v.cls < 0)
+        {
+            why = "no kernel class for this combination of data types and compute type";
+            return PlanStatus::UNSUPPORTED_TYPES;
+        }
+        v.elem_bytes = class_elem_bytes(v.cls);
+
+        const TensorIn &A = in.A, &B = in.B, &C = in.C, &D = in.D;
+        if(A.len.size() != A.mode.size() || A.len.size() != A.stride.size()
+           || B.len.size() != B.mode.size() || B.len.size() != B.stride.size()
+           || D.len.size() != D.mode.size() || D.len.size() != D.stride.size()
+           || (in.bilinear && (C.len.size() != D.len.size() || C.stride.size() != D.len.size())))
+        {
+            why = "rank of a tensor descriptor does not match its mode list";
+            return PlanStatus::INVALID;
+        }
+        if(has_repeats(A.mode) || has_repeats(B.mode) || has_repeats(D.mode))
+        {
+            why = "a mode label appears twice in one tensor";
+            return PlanStatus::UNSUPPORTED_SHAPE;
+        }
+        for(const TensorIn* t : {&A, &B, &D})
+            for(int64_t l : t->len)
+                if(l <= 0)
+                {
+                    why = "a mode has extent 0";
+                    return PlanStatus::UNSUPPORTED_SHAPE;
+                }
+
+        // ---- classify modes: M = D and A, N = D and B, K = A and B ----
+        struct Raw
+        {
+            int64_t len, sa, sb, sc, sd;
+        };
+        std::vector<Raw> M, N, K;
+        for(size_t i = 0; i < D.mode.size(); i++)
+        {
+            const int ia = find_mode(A.mode, D.mode[i]);
+            const int ib = find_mode(B.mode, D.mode[i]);
+            if(ia >= 0 && ib >= 0)
+            {
+                why = "a mode appears in A, B and D (batch modes are not part of this path)";
+                return PlanStatus::UNSUPPORTED_SHAPE;
+            }
+            if(ia < 0 && ib < 0)
+            {
+                why = "a mode of D appears in neither A nor B";
+                return PlanStatus::INVALID;
+            }
+            const int64_t len = ia >= 0 ? A.len[(size_t)ia] : B.len[(size_t)ib];
+            if(len != D.len[i] || (in.bilinear && C.len[i] != D.len[i]))
+            {
+                why = "extent of an output mode differs between tensors";
+                return PlanStatus::INVALID;
+            }
+            Raw r{len, 0, 0, in.bilinear ? C.stride[i] : 0, D.stride[i]};
+            if(ia >= 0)
+            {
+                r.sa = A.stride[(size_t)ia];
+                M.push_back(r);
+            }
+            else
+            {
+                r.sb = B.stride[(size_t)ib];
+                N.push_back(r);
+            }
+        }
+        for(size_t i = 0; i < A.mode.size(); i++)
+        {
+            const int ib = find_mode(B.mode, A.mode[i]);
+            if(ib < 0 || find_mode(D.mode, A.mode[i]) >= 0)
+                continue; // modes held by A alone are read at index 0, as the reference does
+            if(A.len[i] != B.len[(size_t)ib])
+            {
+                why = "extent of a contracted mode differs between A and B";
+                return PlanStatus::INVALID;
+            }
+            K.push_back(Raw{A.len[i], A.stride[i], B.stride[(size_t)ib], 0, 0});
+        }
+
+        // ---- orientation: q must be the index D is contiguous in ----
+        auto min_sd = [](const std::vector<Raw>& g) {
+            int64_t best = INT64_MAX;
+            for(const Raw& r : g)
+                if(r.len > 1)
+                    best = std::min(best, r.sd);
+            return best;
+        };
+        v.swapped = min_sd(M) < min_sd(N);
+
+        const std::vector<Raw>& Pg = v.swapped ? N : M;
+        const std::vector<Raw>& Qg = v.swapped ? M : N;
+        for(const Raw& r : Pg)
+            if(r.len > 1)
+                v.pdims.push_back(Dim{r.len, v.swapped ? r.sb : r.sa, 0, r.sc, r.sd});
+        for(const Raw& r : Qg)
+            if(r.len > 1)
+                v.qdims.push_back(Dim{r.len, 0, v.swapped ? r.sa : r.sb, r.sc, r.sd});
+        for(const Raw& r : K)
+            if(r.len > 1)
+                v.kdims.push_back(Dim{r.len, v.swapped ? r.sb : r.sa, v.swapped ? r.sa : r.sb, 0, 0});
+
+        // ---- order (fastest first) and fuse ----
+        std::stable_sort(v.qdims.begin(), v.qdims.end(), [](const Dim& a, const Dim& b) {
+            return a.sd != b.sd ? a.sd < b.sd : a.sy < b.sy;
+        });
+        std::stable_sort(v.pdims.begin(), v.pdims.end(), [](const Dim& a, const Dim& b) {
+            return a.sx != b.sx ? a.sx < b.sx : a.sd < b.sd;
+        });
+        {
+            // K order follows the operand that is contiguous along a K mode; X wins a tie.
+            bool x_has = false, y_has = false;
+            for(const Dim& d : v.kdims)
+            {
+                x_has |= d.sx == 1;
+                y_has |= d.sy == 1;
+            }
+            const bool by_y = !x_has && y_has;
+            std::stable_sort(v.kdims.begin(), v.kdims.end(), [by_y](const Dim& a, const Dim& b) {
+                const int64_t ka = by_y ? a.sy : a.sx, kb = by_y ? b.sy : b.sx;
+                return ka != kb ? ka < kb : (by_y ? a.sx < b.sx : a.sy < b.sy);
+            });
+        }
+        fuse(v.pdims, GP, in.bilinear);
+        fuse(v.qdims, GQ, in.bilinear);
+        fuse(v.kdims, GK, in.bilinear);
+        v.P = extent(v.pdims);
+        v.Q = extent(v.qdims);
+        v.K = extent(v.kdims);
+        if(v.P > 0x7FFFFF00ll || v.Q > 0x7FFFFF00ll || v.K > 0x7FFFFF00ll)
+        {
+            why = "a folded extent exceeds 2^31";
+            return PlanStatus::UNSUPPORTED_SHAPE;
+        }
+
+        // ---- gather direction and vector width per operand ----
+        const int maxv = class_max_vec(v.cls);
+        const TensorIn& Xt = v.swapped ? B : A;
+        const TensorIn& Yt = v.swapped ? A : B;
+        auto strides_except = [](const std::vector<Dim>& a, const std::vector<Dim>& b, bool use_x, const Dim* skip) {
+            std::vector<int64_t> s;
+            for(const std::vector<Dim>* g : {&a, &b})
+                for(const Dim& d : *g)
+                    if(&d != skip)
+                        s.push_back(use_x ? d.sx : d.sy);
+            return s;
+        };
+        auto pick = [&](bool use_x, const std::vector<Dim>& rows, uint32_t align, int& kfast, int& vec) {
+            int vk = 1, vr = 1;
+            if(!v.kdims.empty() && (use_x ? v.kdims[0].sx : v.kdims[0].sy) == 1)
+                vk = vector_width(v.kdims[0].len, strides_except(rows, v.kdims, use_x, &v.kdims[0]), align, v.elem_bytes, maxv);
+            if(!rows.empty() && (use_x ? rows[0].sx : rows[0].sy) == 1)
+                vr = vector_width(rows[0].len, strides_except(rows, v.kdims, use_x, &rows[0]), align, v.elem_bytes, maxv);
+            // the kernels are instantiated for full-width vectors and for scalars
+            if(vk < maxv)
+                vk = 1;
+            if(vr < maxv)
+                vr = 1;
+            if(vr > vk)
+            {
+                kfast = 0;
+                vec   = vr;
+            }
+            else
+            {
+                kfast = 1;
+                vec   = vk;
+            }
+        };
+        pick(true, v.pdims, Xt.align, v.x_kfast, v.x_vec);
+        pick(false, v.qdims, Yt.align, v.y_kfast, v.y_vec);
+        v.cd_vec = 1;
+        if(!v.qdims.empty() && v.qdims[0].sd == 1 && (!in.bilinear || v.qdims[0].sc == 1))
+        {
+            std::vector<int64_t> others;
+            for(const std::vector<Dim>* g : {&v.pdims, &v.qdims})
+                for(const Dim& d : *g)
+                    if(&d != &v.qdims[0])
+                    {
+                        others.push_back(d.sd);
+                        if(in.bilinear)
+                            others.push_back(d.sc);
+                    }
+            uint32_t al = D.align;
+            if(in.bilinear)
+                al = std::min(al, C.align);
+            v.cd_vec = vector_width(v.qdims[0].len, others, al, v.elem_bytes, maxv);
+        }
+
+        // ---- offset tables ----
+        auto pad256 = [](int64_t n) { return (size_t)((n + 255) / 256 * 256); };
+        int64_t mxp, mxk, myq, myk, mcp, mcq, mdp, mdq;
+        bool    ok = true;
+        ok &= make_table(v.pdims, v.P, pad256(v.P), [](const Dim& d) { return d.sx; }, v.xp, mxp);
+        ok &= make_table(v.kdims, v.K, pad256(v.K) + 256, [](const Dim& d) { return d.sx; }, v.xk, mxk);
+        ok &= make_table(v.qdims, v.Q, pad256(v.Q), [](const Dim& d) { return d.sy; }, v.yq, myq);
+        ok &= make_table(v.kdims, v.K, pad256(v.K) + 256, [](const Dim& d) { return d.sy; }, v.yk, myk);
+        ok &= make_table(v.pdims, v.P, pad256(v.P), [](const Dim& d) { return d.sd; }, v.dp, mdp);
+        ok &= make_table(v.qdims, v.Q, pad256(v.Q), [](const Dim& d) { return d.sd; }, v.dq, mdq);
+        if(in.bilinear)
+        {
+            ok &= make_table(v.pdims, v.P, pad256(v.P), [](const Dim& d) { return d.sc; }, v.cp, mcp);
+            ok &= make_table(v.qdims, v.Q, pad256(v.Q), [](const Dim& d) { return d.sc; }, v.cq, mcq);
+        }
+        else
+            mcp = mcq = 0;
+        const int64_t lim = 0x7FFFFFFFll;
+        if(!ok || mxp + mxk > lim || myq + myk > lim || mcp + mcq > lim || mdp + mdq > lim)
+        {
+            why = "a tensor spans more than 2^31 elements";
+            return PlanStatus::UNSUPPORTED_SHAPE;
+        }
+
+        v.spanA = span_elems(A.len, A.stride);
+        v.spanB = span_elems(B.len, B.stride);
+        v.spanD = span_elems(D.len, D.stride);
+        v.spanC = in.bilinear ? span_elems(C.len, C.stride) : 0;
+        return PlanStatus::OK;
+    }
+}

@@ -1,0 +1,174 @@
+#include "solution.hpp"
+
+#include <algorithm>
+#include <cmath>
+
+namespace hipta
+{
+    static uint64_t mix(uint64_t h, uint64_t v)
+    {
+        // 64-bit variant of the boost-style combine the reference uses for its solution
+        // ids (library/src/include/hash.hpp:50-58)
+        return h ^ (v + 0x9e3779b97f4a7c15ull + (h << 6) + (h >> 2));
+    }
+
+    SolutionRegistry::SolutionRegistry()
+    {
+        for(int cls = 0; cls < HIPTK_NUM_CLASSES; cls++)
+        {
+            const int n = hiptk_tile_count(cls);
+            for(int t = 0; t < n; t++)
+            {
+                hiptk_tile_info_t ti;
+                if(hiptk_tile_info(cls, t, &ti) != HIPTK_OK)
+                    continue;
+                Solution s;
+                s.cls       = cls;
+                s.tile_id   = t;
+                s.bp        = ti.bp;
+                s.bq        = ti.bq;
+                s.bk        = ti.bk;
+                s.threads   = ti.threads;
+                s.lds_bytes = ti.lds_bytes;
+                s.name      = ti.name;
+                uint64_t h  = 0x68697074656e73ull;
+                for(uint64_t x : {(uint64_t)cls, (uint64_t)t, (uint64_t)ti.bp, (uint64_t)ti.bq, (uint64_t)ti.bk})
+                    h = mix(h, x);
+                s.uid = h;
+                mAll.push_back(s);
+            }
+        }
+    }
+
+    const SolutionRegistry& SolutionRegistry::get()
+    {
+        static const SolutionRegistry r;
+        return r;
+    }
+
+    std::vector<const Solution*> SolutionRegistry::forClass(int cls) const
+    {
+        std::vector<const Solution*> out;
+        for(const Solution& s : mAll)
+            if(s.cls == cls)
+                out.push_back(&s);
+        return out;
+    }
+
+    const Solution* SolutionRegistry::byUid(uint64_t uid) const
+    {
+        for(const Solution& s : mAll)
+            if(s.uid == uid)
+                return &s;
+        return nullptr;
+    }
+
+    bool solution_fits(const Solution& s, const GemmView& v)
+    {
+        if(s.cls != v.cls)
+            return false;
+        hiptk_problem_t p{};
+        p.cls     = v.cls;
+        p.tile_id = s.tile_id;
+        p.x_kfast = v.x_kfast;
+        p.y_kfast = v.y_kfast;
+        p.x_vec   = v.x_vec;
+        p.y_vec   = v.y_vec;
+        return hiptk_kernel_available(&p) != 0;
+    }
+
+    double class_flops_per_clk_cu(int cls)
+    {
+        switch(cls)
+        {
+        case HIPTK_F16:
+        case HIPTK_BF16:
+        case HIPTK_F32_AS_F16:
+        case HIPTK_F32_AS_BF16: return 4096.0;
+        case HIPTK_F64:
+        case HIPTK_C64: return 128.0;
+        default: return 256.0;
+        }
+    }
+
+    double class_flops_per_mac(int cls)
+    {
+        return (cls == HIPTK_C32 || cls == HIPTK_C64) ? 8.0 : 2.0;
+    }
+
+    int class_acc_bytes(int cls)
+    {
+        switch(cls)
+        {
+        case HIPTK_F64:
+        case HIPTK_C32: return 8;
+        case HIPTK_C64: return 16;
+        default: return 4;
+        }
+    }
+
+    double estimate_us(const Solution& s, const GemmView& v, int split, const DeviceModel& dev)
+    {
+        const double tiles  = std::ceil((double)v.P / s.bp) * std::ceil((double)v.Q / s.bq);
+        const double ktiles = std::ceil((double)v.K / s.bk);
+        const double kper   = std::ceil(ktiles / split) * s.bk;
+        // Workgroups that fit on one CU at a time (LDS bound; big tiles also fill the
+        // register file on their own).
+        int resident = std::max(1, std::min(4, dev.lds_per_cu / std::max(1, s.lds_bytes)));
+        if(s.bp * s.bq >= 256 * 256)
+            resident = 1;
+        const double slots = (double)dev.cus * resident;
+        const double waves = std::ceil(tiles * split / slots);
+        // Fraction of the CU's MFMA peak a full set of resident workgroups of this tile
+        // sustains: larger tiles re-use each LDS fragment in more MFMAs.
+        const double area = (double)s.bp * s.bq;
+        double       eff  = area >= 65536 ? 0.75 : area >= 16384 ? 0.55 : area >= 4096 ? 0.30 : 0.15;
+        if(v.x_vec == 1 || v.y_vec == 1)
+            eff *= 0.35; // scalar gathers are issue bound
+        const double flops_wg = class_flops_per_mac(v.cls) * area * kper;
+        const double rate_wg  = class_flops_per_clk_cu(v.cls) * eff / resident; // flop / clk
+        double       us       = waves * flops_wg / rate_wg / (dev.clock_ghz * 1e3);
+        // memory floor: every operand once (+ C and D)
+        const double bytes = ((double)v.P * v.K + (double)v.Q * v.K + (double)v.P * v.Q * (v.bilinear ? 2 : 1))
+                             * v.elem_bytes;
+        us = std::max(us, bytes / (dev.hbm_gbs * 1e3));
+        // fixed cost per workgroup (prologue, epilogue) and launch
+        us += 1.0 + waves * 1.5;
+        if(split > 1)
+        {
+            const double ws = (double)split * v.P * v.Q * class_acc_bytes(v.cls);
+            us += 2.0 * ws / (dev.hbm_gbs * 1e3 * 0.5) + 3.0; // write + read partials, second launch
+        }
+        return us;
+    }
+
+    std::vector<Choice> rank_choices(const std::vector<const Solution*>& candidates,
+                                     const GemmView&                     v,
+                                     uint64_t                            max_ws,
+                                     const DeviceModel&                  dev)
+    {
+        std::vector<Choice> out;
+        for(const Solution* s : candidates)
+        {
+            if(!s || !solution_fits(*s, v))
+                continue;
+            const int ktiles = (int)((v.K + s->bk - 1) / s->bk);
+            for(int split = 1; split <= 64 && split <= ktiles; split *= 2)
+            {
+                const uint64_t ws = split > 1 ? (uint64_t)split * (uint64_t)v.P * (uint64_t)v.Q
+                                                    * (uint64_t)class_acc_bytes(v.cls)
+                                              : 0;
+                if(ws > max_ws)
+                    break;
+                Choice c;
+                c.sol      = s;
+                c.split_k  = split;
+                c.ws_bytes = ws;
+                c.est_us   = estimate_us(*s, v, split, dev);
+                out.push_back(c);
+            }
+        }
+        std::stable_sort(out.begin(), out.end(), [](const Choice& a, const Choice& b) { return a.est_us < b.est_us; });
+        return out;
+    }
+}

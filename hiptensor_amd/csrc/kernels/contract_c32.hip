@@ -1,0 +1,16 @@
+// complex f32 kernels (two v_mfma_f32_32x32x2_f32 per complex k).
+#include "contract_w.hpp"
+
+namespace hiptk
+{
+    static const KernelEntry k_entries[] = {
+        HIPTK_W_TILE(WTraitsC32, 0, 128, 128, 8, 2, 2),
+        HIPTK_W_TILE(WTraitsC32, 1, 64, 64, 8, 2, 2),
+    };
+
+    const KernelEntry* entries_c32(int* count)
+    {
+        *count = (int)(sizeof(k_entries) / sizeof(k_entries[0]));
+        return k_entries;
+    }
+}

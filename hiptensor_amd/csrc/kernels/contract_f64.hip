@@ -1,0 +1,16 @@
+// f64 kernels (v_mfma_f64_16x16x4_f64).
+#include "contract_w.hpp"
+
+namespace hiptk
+{
+    static const KernelEntry k_entries[] = {
+        HIPTK_W_TILE(WTraitsF64, 0, 128, 128, 16, 2, 2),
+        HIPTK_W_TILE(WTraitsF64, 1, 64, 64, 16, 2, 2),
+    };
+
+    const KernelEntry* entries_f64(int* count)
+    {
+        *count = (int)(sizeof(k_entries) / sizeof(k_entries[0]));
+        return k_entries;
+    }
+}

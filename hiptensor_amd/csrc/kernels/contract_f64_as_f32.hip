@@ -1,0 +1,16 @@
+// f64 storage computed in f32 (inputs narrowed when staged).
+#include "contract_w.hpp"
+
+namespace hiptk
+{
+    static const KernelEntry k_entries[] = {
+        HIPTK_W_TILE(WTraitsF64AsF32, 0, 128, 128, 16, 2, 2),
+        HIPTK_W_TILE(WTraitsF64AsF32, 1, 64, 64, 16, 2, 2),
+    };
+
+    const KernelEntry* entries_f64_as_f32(int* count)
+    {
+        *count = (int)(sizeof(k_entries) / sizeof(k_entries[0]));
+        return k_entries;
+    }
+}

@@ -1,0 +1,451 @@
+// 16-bit (f16 / bf16) contraction kernel for gfx950.
+//
+//   acc[p][q] = sum_k X[xp[p] + xk[k]] * Y[yq[q] + yk[k]]        (f32 accumulate)
+//   D[dp[p] + dq[q]] = alpha * acc (+ beta * C[cp[p] + cq[q]])    (f32 epilogue, one rounding)
+//
+// One workgroup of WP x WQ wavefronts (64 lanes each) owns a BP x BQ output tile and
+// walks K in steps of BK.  Per step the X and Y tiles are gathered from global memory
+// through the offset tables into registers (one step ahead of their use), written
+// into one of two LDS buffers, and consumed by v_mfma_f32_32x32x16_{f16,bf16}.
+//
+// LDS layout depends on which way an operand's contiguous vectors run:
+//   vectors along k  ("k-fast"):  tile[row][BK + 8]; a lane's MFMA operand (8
+//       consecutive k of one row) is one ds_read_b128, the +8 pad (16 B) staggers
+//       rows over the banks.
+//   vectors along the row index:  tile[k][BR + 16]; the operand is assembled by two
+//       ds_read_b64_tr_b16 (the transposing LDS read of CDNA4), so no software
+//       transpose is needed.  The +16 pad (32 B) puts the four k-rows a 16-lane group
+//       touches into disjoint bank ranges.
+//
+// MFMA operand / result register layouts used here (verified on hardware):
+//   operand: lane l holds row (l % 32), k = 8 * (l / 32) .. + 7
+//   result : lane l, register r holds p = 8 * (r / 4) + 4 * (l / 32) + r % 4, q = l % 32
+// X feeds the first MFMA operand (p is register-varying), Y the second (q is
+// lane-varying), so at a fixed register the 32 lanes of a half-wave write 32
+// consecutive q: the planner orients the problem so that q is D's contiguous index.
+#pragma once
+#include "kargs.h"
+
+namespace hiptk
+{
+    typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+    typedef __bf16   bf16x8_t __attribute__((ext_vector_type(8)));
+    typedef float    f32x16_t __attribute__((ext_vector_type(16)));
+    typedef short    short4_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+    __device__ inline uint16_t f32_to_bf16_rne(float f)
+    {
+        uint32_t x = __float_as_uint(f);
+        if((~x & 0x7F800000u) == 0)
+        {
+            if(x & 0xFFFFu)
+                x |= 0x10000u;
+        }
+        else
+            x += 0x7FFFu + ((x >> 16) & 1u);
+        return (uint16_t)(x >> 16);
+    }
+
+    struct TraitsF16
+    {
+        static constexpr int CLS = HIPTK_F16;
+        typedef uint16_t     src_t;
+        static __device__ inline f32x16_t mfma(u32x4_t x, u32x4_t y, f32x16_t acc)
+        {
+            return __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                __builtin_bit_cast(half8_t, x), __builtin_bit_cast(half8_t, y), acc, 0, 0, 0);
+        }
+        static __device__ inline uint16_t from_f32(float f)
+        {
+            return __builtin_bit_cast(uint16_t, (_Float16)f);
+        }
+        static __device__ inline float to_f32(uint16_t h)
+        {
+            return (float)__builtin_bit_cast(_Float16, h);
+        }
+        static __device__ inline uint16_t stage(uint16_t v) { return v; }
+    };
+
+    struct TraitsBF16
+    {
+        static constexpr int CLS = HIPTK_BF16;
+        typedef uint16_t     src_t;
+        static __device__ inline f32x16_t mfma(u32x4_t x, u32x4_t y, f32x16_t acc)
+        {
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(bf16x8_t, x), __builtin_bit_cast(bf16x8_t, y), acc, 0, 0, 0);
+        }
+        static __device__ inline uint16_t from_f32(float f) { return f32_to_bf16_rne(f); }
+        static __device__ inline float    to_f32(uint16_t h)
+        {
+            return __uint_as_float((uint32_t)h << 16);
+        }
+        static __device__ inline uint16_t stage(uint16_t v) { return v; }
+    };
+
+    // LDS tile geometry of one operand (16-bit elements).
+    template <bool KF, int BR, int BK>
+    struct TileLds
+    {
+        static constexpr int PITCH = KF ? BK + 8 : BR + 16;
+        static constexpr int ELEMS = (KF ? BR : BK) * PITCH;
+    };
+
+    // Global -> register -> LDS staging of one operand tile.
+    template <typename Tr, bool KF, int V, int BR, int BK, int NT>
+    struct Stager
+    {
+        typedef typename Tr::src_t src_t;
+        static constexpr int PER   = KF ? BK / V : BR / V; // vectors along the vector direction
+        static constexpr int STEP  = NT / PER; // rows (k-fast) or k's covered per pass
+        static constexpr int N     = (BR * BK / V) / NT; // vectors per thread
+        static constexpr int W     = V >= 2 ? V / 2 : 1; // 32-bit words per staged vector
+        static constexpr int PITCH = TileLds<KF, BR, BK>::PITCH;
+        static_assert(NT % PER == 0, "thread count must cover whole vector rows");
+        static_assert((BR * BK / V) % NT == 0 && N >= 1, "tile must split evenly over threads");
+        static_assert(sizeof(src_t) == 2, "16-bit storage");
+
+        uint32_t data[N][W];
+        int32_t  roff[KF ? N : 1]; // row-table offsets (loop invariant)
+        int32_t  koff[KF ? 1 : N]; // k-table offsets of the tile being fetched
+        int      a, b; // k-fast: a = vector slot along k, b = first row; else a = row vector, b = first k
+
+        __device__ inline void init(const int32_t* rtab, int r0, int tid)
+        {
+            a = tid % PER;
+            b = tid / PER;
+            if constexpr(KF)
+            {
+#pragma unroll
+                for(int i = 0; i < N; i++)
+                    roff[i] = rtab[r0 + b + i * STEP];
+            }
+            else
+                roff[0] = rtab[r0 + a * V];
+        }
+
+        __device__ inline void load_koffs(const int32_t* ktab, int k0)
+        {
+            if constexpr(KF)
+                koff[0] = ktab[k0 + a * V];
+            else
+            {
+#pragma unroll
+                for(int i = 0; i < N; i++)
+                    koff[i] = ktab[k0 + b + i * STEP];
+            }
+        }
+
+        __device__ inline void fetch_one(const src_t* base, uint32_t off, bool ok, uint32_t (&d)[W])
+        {
+            const src_t* p = base + off;
+            if constexpr(V == 8)
+            {
+                u32x4_t v = {0u, 0u, 0u, 0u};
+                if(ok)
+                    v = *(const u32x4_t*)p;
+                d[0] = v[0];
+                d[1] = v[1];
+                d[2] = v[2];
+                d[3] = v[3];
+            }
+            else if constexpr(V == 4)
+            {
+                u32x2_t v = {0u, 0u};
+                if(ok)
+                    v = *(const u32x2_t*)p;
+                d[0] = v[0];
+                d[1] = v[1];
+            }
+            else if constexpr(V == 2)
+                d[0] = ok ? *(const uint32_t*)p : 0u;
+            else
+                d[0] = ok ? (uint32_t)*p : 0u;
+        }
+
+        // Fetch the tile whose first k is k0 (koffs for it must be loaded already).
+        __device__ inline void fetch(const void* base, int k0, int K)
+        {
+            const src_t* bp = (const src_t*)base;
+            if constexpr(KF)
+            {
+                const bool ok = (k0 + a * V) < K;
+#pragma unroll
+                for(int i = 0; i < N; i++)
+                    fetch_one(bp, (uint32_t)roff[i] + (uint32_t)koff[0], ok, data[i]);
+            }
+            else
+            {
+#pragma unroll
+                for(int i = 0; i < N; i++)
+                    fetch_one(bp,
+                              (uint32_t)roff[0] + (uint32_t)koff[i],
+                              (k0 + b + i * STEP) < K,
+                              data[i]);
+            }
+        }
+
+        __device__ inline void commit(uint16_t* lds)
+        {
+#pragma unroll
+            for(int i = 0; i < N; i++)
+            {
+                uint16_t* dst = KF ? lds + (b + i * STEP) * PITCH + a * V
+                                   : lds + (b + i * STEP) * PITCH + a * V;
+                if constexpr(V == 8)
+                {
+                    u32x4_t v = {data[i][0], data[i][1], data[i][2], data[i][3]};
+                    *(u32x4_t*)dst = v;
+                }
+                else if constexpr(V == 4)
+                {
+                    u32x2_t v      = {data[i][0], data[i][1]};
+                    *(u32x2_t*)dst = v;
+                }
+                else if constexpr(V == 2)
+                    *(uint32_t*)dst = data[i][0];
+                else
+                    *dst = (uint16_t)data[i][0];
+            }
+        }
+    };
+
+    // MFMA operand fetch from LDS for the 32-row block starting at row r0, k-substep ks.
+    template <bool KF, int PITCH>
+    __device__ inline int frag_base(int lane)
+    {
+        if constexpr(KF)
+            return (lane & 31) * PITCH + 8 * (lane >> 5);
+        else
+            return (8 * (lane >> 5) + ((lane & 15) >> 2)) * PITCH + 16 * ((lane >> 4) & 1)
+                   + 4 * (lane & 3);
+    }
+
+    template <bool KF, int PITCH>
+    __device__ inline u32x4_t frag_load(const uint16_t* lds, int base, int r0, int ks)
+    {
+        if constexpr(KF)
+            return *(const u32x4_t*)(lds + base + r0 * PITCH + ks * 16);
+        else
+        {
+            typedef short4_t __attribute__((address_space(3))) * lds_s4_ptr;
+            const uint16_t* p  = lds + base + ks * 16 * PITCH + r0;
+            short4_t        lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(p));
+            short4_t        hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(p + 4 * PITCH));
+            u32x2_t         l2 = __builtin_bit_cast(u32x2_t, lo);
+            u32x2_t         h2 = __builtin_bit_cast(u32x2_t, hi);
+            u32x4_t         v  = {l2[0], l2[1], h2[0], h2[1]};
+            return v;
+        }
+    }
+
+    template <typename Tr,
+              int  BP,
+              int  BQ,
+              int  BK,
+              int  WP,
+              int  WQ,
+              bool XKF,
+              bool YKF,
+              int  XV,
+              int  YV>
+    __global__ void __launch_bounds__(WP* WQ * 64) contract_h_kernel(const KArgs a)
+    {
+        constexpr int NT  = WP * WQ * 64;
+        constexpr int WTP = BP / WP, WTQ = BQ / WQ;
+        constexpr int TP = WTP / 32, TQ = WTQ / 32;
+        static_assert(WTP % 32 == 0 && WTQ % 32 == 0 && BK % 16 == 0, "tile shape");
+        typedef TileLds<XKF, BP, BK> LX;
+        typedef TileLds<YKF, BQ, BK> LY;
+        constexpr int STAGE = LX::ELEMS + LY::ELEMS;
+
+        extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+
+        const int tid  = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = tid >> 6;
+        const int wp   = wave / WQ;
+        const int wq   = wave % WQ;
+
+        int tp, tq;
+        tile_coords(blockIdx.x, a.tiles_p, a.tiles_q, tp, tq);
+        const int p0 = tp * BP;
+        const int q0 = tq * BQ;
+
+        const int kt_begin = blockIdx.z * a.ktiles_per_split;
+        int       kt_end   = kt_begin + a.ktiles_per_split;
+        const int kt_all   = (a.K + BK - 1) / BK;
+        if(kt_end > kt_all)
+            kt_end = kt_all;
+
+        Stager<Tr, XKF, XV, BP, BK, NT> sx;
+        Stager<Tr, YKF, YV, BQ, BK, NT> sy;
+        sx.init(a.xp, p0, tid);
+        sy.init(a.yq, q0, tid);
+
+        f32x16_t acc[TP][TQ];
+#pragma unroll
+        for(int i = 0; i < TP; i++)
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+#pragma unroll
+                for(int r = 0; r < 16; r++)
+                    acc[i][j][r] = 0.f;
+
+        const int xbase = frag_base<XKF, LX::PITCH>(lane) + (XKF ? wp * WTP * LX::PITCH : wp * WTP);
+        const int ybase = frag_base<YKF, LY::PITCH>(lane) + (YKF ? wq * WTQ * LY::PITCH : wq * WTQ);
+
+        if(kt_begin < kt_end)
+        {
+            sx.load_koffs(a.xk, kt_begin * BK);
+            sy.load_koffs(a.yk, kt_begin * BK);
+            sx.fetch(a.X, kt_begin * BK, a.K);
+            sy.fetch(a.Y, kt_begin * BK, a.K);
+            sx.load_koffs(a.xk, (kt_begin + 1) * BK);
+            sy.load_koffs(a.yk, (kt_begin + 1) * BK);
+        }
+
+        int buf = 0;
+        for(int kt = kt_begin; kt < kt_end; kt++)
+        {
+            uint16_t* lx = lds + buf * STAGE;
+            uint16_t* ly = lx + LX::ELEMS;
+            sx.commit(lx);
+            sy.commit(ly);
+            __syncthreads();
+            if(kt + 1 < kt_end)
+            {
+                sx.fetch(a.X, (kt + 1) * BK, a.K);
+                sy.fetch(a.Y, (kt + 1) * BK, a.K);
+                sx.load_koffs(a.xk, (kt + 2) * BK);
+                sy.load_koffs(a.yk, (kt + 2) * BK);
+            }
+#pragma unroll
+            for(int ks = 0; ks < BK / 16; ks++)
+            {
+                u32x4_t xf[TP], yf[TQ];
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+                    xf[i] = frag_load<XKF, LX::PITCH>(lx, xbase, XKF ? i * 32 : i * 32, ks);
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+                    yf[j] = frag_load<YKF, LY::PITCH>(ly, ybase, YKF ? j * 32 : j * 32, ks);
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+#pragma unroll
+                    for(int j = 0; j < TQ; j++)
+                        acc[i][j] = Tr::mfma(xf[i], yf[j], acc[i][j]);
+            }
+            buf ^= 1;
+        }
+
+        // ---- epilogue ----
+        const int   pw = p0 + wp * WTP + 4 * (lane >> 5);
+        const int   qw = q0 + wq * WTQ + (lane & 31);
+        const float alpha = (float)a.alpha[0];
+        const float beta  = (float)a.beta[0];
+        if(a.split_k > 1)
+        {
+            float* ws = (float*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+            {
+                const int q = qw + j * 32;
+                if(q >= a.Q)
+                    continue;
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                    {
+                        const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
+                        if(p < a.P)
+                            ws[(size_t)p * a.Q + q] = acc[i][j][r];
+                    }
+            }
+            return;
+        }
+        uint16_t*       Dp = (uint16_t*)a.D;
+        const uint16_t* Cp = (const uint16_t*)a.C;
+#pragma unroll
+        for(int j = 0; j < TQ; j++)
+        {
+            const int q = qw + j * 32;
+            if(q >= a.Q)
+                continue;
+            const uint32_t dqo = (uint32_t)a.dq[q];
+            const uint32_t cqo = a.bilinear ? (uint32_t)a.cq[q] : 0u;
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+#pragma unroll
+                for(int r = 0; r < 16; r++)
+                {
+                    const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
+                    if(p < a.P)
+                    {
+                        float v = alpha * acc[i][j][r];
+                        if(a.bilinear)
+                            v += beta * Tr::to_f32(Cp[(uint32_t)a.cp[p] + cqo]);
+                        Dp[(uint32_t)a.dp[p] + dqo] = Tr::from_f32(v);
+                    }
+                }
+        }
+    }
+
+    template <typename Tr,
+              int  BP,
+              int  BQ,
+              int  BK,
+              int  WP,
+              int  WQ,
+              bool XKF,
+              bool YKF,
+              int  XV,
+              int  YV>
+    int launch_h(const KArgs& a, hipStream_t stream)
+    {
+        typedef TileLds<XKF, BP, BK> LX;
+        typedef TileLds<YKF, BQ, BK> LY;
+        constexpr int                LDS = 2 * (LX::ELEMS + LY::ELEMS) * 2;
+        auto kern = contract_h_kernel<Tr, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV>;
+        static const hipError_t attr = hipFuncSetAttribute(
+            (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        if(attr != hipSuccess)
+            return (int)attr;
+        dim3 grid(a.tiles_p * a.tiles_q, 1, a.split_k);
+        hipLaunchKernelGGL(kern, grid, dim3(WP * WQ * 64), LDS, stream, a);
+        return (int)hipGetLastError();
+    }
+
+    template <int BP, int BQ, int BK, bool XKF, bool YKF>
+    constexpr int lds_bytes_h()
+    {
+        return 2 * (TileLds<XKF, BP, BK>::ELEMS + TileLds<YKF, BQ, BK>::ELEMS) * 2;
+    }
+}
+
+// One registry line: class traits, tile id, tile shape, wave grid, layouts, vectors.
+#define HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV)                         \
+    {                                                                                       \
+        TR::CLS, ID, XKF, YKF, XV, YV, BP, BQ, BK, WP *WQ * 64,                             \
+            hiptk::lds_bytes_h<BP, BQ, BK, XKF, YKF>(),                                     \
+            #TR "_" #BP "x" #BQ "x" #BK "_x" #XKF #XV "_y" #YKF #YV,                        \
+            &hiptk::launch_h<hiptk::TR, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV>               \
+    }
+
+// The four layout combinations of a tile whose operands are both gathered 8 wide.
+#define HIPTK_H_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ)               \
+    HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 8),  \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 8, 8), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 8), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, 8, 8)
+
+// Combinations in which at least one operand is a scalar gather (always staged k-fast).
+#define HIPTK_H_TILE_V1(TR, ID, BP, BQ, BK, WP, WQ)               \
+    HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 1, 1),  \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 1), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 1), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 1, 8), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 1, 8)

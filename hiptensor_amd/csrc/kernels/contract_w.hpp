@@ -1,0 +1,576 @@
+// 32/64-bit contraction kernels for gfx950: f32, f64, complex f32, complex f64 and
+// f64 storage computed in f32.
+//
+//   acc[p][q] = sum_k X[xp[p] + xk[k]] * Y[yq[q] + yk[k]]
+//   D[dp[p] + dq[q]] = alpha * acc (+ beta * C[cp[p] + cq[q]])
+//
+// These MFMA shapes take one element per lane per operand (v_mfma_f32_32x32x2_f32:
+// lane l supplies row l % 32 at k = l / 32; v_mfma_f64_16x16x4_f64: row l % 16 at
+// k = l / 16), so both operand tiles live in LDS as tile[k][row + pad] and a lane's
+// operand is one ds_read of consecutive rows across lanes: conflict free.
+//
+// Complex products use the same real MFMA by treating (re, im) as two adjacent k:
+//   Re += [xr, -xi] . [yr, yi]      Im += [xi, xr] . [yr, yi]
+// The lanes of the second k-slot read the same complex element and pick / negate the
+// part they need, so a 32x32 complex tile costs two MFMAs per complex k: all four
+// real products of every complex multiply run on the matrix core, none is wasted,
+// and there is no split into separate re/im arrays.
+//
+// Result layouts (verified on hardware):
+//   32x32: lane l, register r -> p = 8 * (r / 4) + 4 * (l / 32) + r % 4, q = l % 32
+//   f64 16x16: lane l, register r -> p = 4 * r + l / 16, q = l % 16
+#pragma once
+#include "kargs.h"
+
+namespace hiptk
+{
+    typedef float  wf32x16_t __attribute__((ext_vector_type(16)));
+    typedef double wf64x4_t __attribute__((ext_vector_type(4)));
+
+    enum
+    {
+        GATHER_MN_VEC = 0, // vectors of VMAX along the row index
+        GATHER_K_VEC  = 1, // vectors of VMAX along k
+        GATHER_SCALAR = 2
+    };
+
+    // ---- per-class traits -------------------------------------------------------
+
+    struct WTraitsF32
+    {
+        static constexpr int CLS = HIPTK_F32;
+        typedef float        E; // storage element
+        typedef float        S; // element as staged in LDS
+        typedef float        XF;
+        typedef float        YF;
+        typedef float        O; // accumulator element written to split-K workspace
+        static constexpr int TILE = 32, KM = 2, NREG = 16, VMAX = 4;
+        struct Acc
+        {
+            wf32x16_t v;
+        };
+        static __device__ inline S    stage(E e) { return e; }
+        static __device__ inline int  kslot(int lane) { return lane >> 5; }
+        static __device__ inline XF   prep_x(S s, int) { return s; }
+        static __device__ inline YF   prep_y(S s, int) { return s; }
+        static __device__ inline void zero(Acc& a)
+        {
+#pragma unroll
+            for(int r = 0; r < 16; r++)
+                a.v[r] = 0.f;
+        }
+        static __device__ inline void mma(XF x, YF y, Acc& a)
+        {
+            a.v = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, a.v, 0, 0, 0);
+        }
+        static __device__ inline int p_of(int r, int lane)
+        {
+            return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        }
+        static __device__ inline int q_of(int lane) { return lane & 31; }
+        static __device__ inline O   get(const Acc& a, int r) { return a.v[r]; }
+        // alpha * x + beta * c with separately rounded products, as the CPU path does.
+        static __device__ inline E finish(O x, const double* al, const double* be, bool bil, const E* c)
+        {
+            float y = __fmul_rn((float)al[0], x);
+            if(bil)
+                y = __fadd_rn(y, __fmul_rn((float)be[0], *c));
+            return y;
+        }
+    };
+
+    struct WTraitsF64
+    {
+        static constexpr int CLS = HIPTK_F64;
+        typedef double       E;
+        typedef double       S;
+        typedef double       XF;
+        typedef double       YF;
+        typedef double       O;
+        static constexpr int TILE = 16, KM = 4, NREG = 4, VMAX = 2;
+        struct Acc
+        {
+            wf64x4_t v;
+        };
+        static __device__ inline S    stage(E e) { return e; }
+        static __device__ inline int  kslot(int lane) { return lane >> 4; }
+        static __device__ inline XF   prep_x(S s, int) { return s; }
+        static __device__ inline YF   prep_y(S s, int) { return s; }
+        static __device__ inline void zero(Acc& a)
+        {
+#pragma unroll
+            for(int r = 0; r < 4; r++)
+                a.v[r] = 0.0;
+        }
+        static __device__ inline void mma(XF x, YF y, Acc& a)
+        {
+            a.v = __builtin_amdgcn_mfma_f64_16x16x4f64(x, y, a.v, 0, 0, 0);
+        }
+        static __device__ inline int p_of(int r, int lane) { return 4 * r + (lane >> 4); }
+        static __device__ inline int q_of(int lane) { return lane & 15; }
+        static __device__ inline O   get(const Acc& a, int r) { return a.v[r]; }
+        // alpha and beta are narrowed to float first: the reference's Bilinear / Scale
+        // functors hold them as float even for f64 data.
+        static __device__ inline E finish(O x, const double* al, const double* be, bool bil, const E* c)
+        {
+            double y = __dmul_rn((double)(float)al[0], x);
+            if(bil)
+                y = __dadd_rn(y, __dmul_rn((double)(float)be[0], *c));
+            return y;
+        }
+    };
+
+    // f64 storage, inputs narrowed to f32 when staged, f32 MFMA, f32 accumulate.
+    struct WTraitsF64AsF32 : WTraitsF32
+    {
+        static constexpr int CLS = HIPTK_F64_AS_F32;
+        typedef double       E;
+        static constexpr int VMAX = 2;
+        static __device__ inline S stage(E e) { return (float)e; }
+        static __device__ inline E finish(O x, const double* al, const double* be, bool bil, const E* c)
+        {
+            double y = __dmul_rn((double)(float)al[0], (double)x);
+            if(bil)
+                y = __dadd_rn(y, __dmul_rn((double)(float)be[0], *c));
+            return y;
+        }
+    };
+
+    struct WTraitsC32
+    {
+        static constexpr int CLS = HIPTK_C32;
+        typedef float2       E;
+        typedef float2       S;
+        typedef float2       XF; // (operand of the Re chain, operand of the Im chain)
+        typedef float        YF;
+        typedef float2       O;
+        static constexpr int TILE = 32, KM = 1, NREG = 16, VMAX = 2;
+        struct Acc
+        {
+            wf32x16_t re, im;
+        };
+        static __device__ inline S   stage(E e) { return e; }
+        static __device__ inline int kslot(int) { return 0; }
+        static __device__ inline XF  prep_x(S s, int lane)
+        {
+            return (lane >> 5) ? make_float2(-s.y, s.x) : make_float2(s.x, s.y);
+        }
+        static __device__ inline YF   prep_y(S s, int lane) { return (lane >> 5) ? s.y : s.x; }
+        static __device__ inline void zero(Acc& a)
+        {
+#pragma unroll
+            for(int r = 0; r < 16; r++)
+            {
+                a.re[r] = 0.f;
+                a.im[r] = 0.f;
+            }
+        }
+        static __device__ inline void mma(XF x, YF y, Acc& a)
+        {
+            a.re = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, y, a.re, 0, 0, 0);
+            a.im = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, y, a.im, 0, 0, 0);
+        }
+        static __device__ inline int p_of(int r, int lane)
+        {
+            return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        }
+        static __device__ inline int q_of(int lane) { return lane & 31; }
+        static __device__ inline O   get(const Acc& a, int r) { return make_float2(a.re[r], a.im[r]); }
+        static __device__ inline E finish(O x, const double* al, const double* be, bool bil, const E* c)
+        {
+            const float ar = (float)al[0], ai = (float)al[1];
+            float       yr = __fsub_rn(__fmul_rn(ar, x.x), __fmul_rn(ai, x.y));
+            float       yi = __fadd_rn(__fmul_rn(ai, x.x), __fmul_rn(ar, x.y));
+            if(bil)
+            {
+                const float  br = (float)be[0], bi = (float)be[1];
+                const float2 cv = *c;
+                yr = __fadd_rn(yr, __fsub_rn(__fmul_rn(br, cv.x), __fmul_rn(bi, cv.y)));
+                yi = __fadd_rn(yi, __fadd_rn(__fmul_rn(bi, cv.x), __fmul_rn(br, cv.y)));
+            }
+            return make_float2(yr, yi);
+        }
+    };
+
+    struct WTraitsC64
+    {
+        static constexpr int CLS = HIPTK_C64;
+        typedef double2      E;
+        typedef double2      S;
+        typedef double2      XF;
+        typedef double       YF;
+        typedef double2      O;
+        static constexpr int TILE = 16, KM = 2, NREG = 4, VMAX = 1;
+        struct Acc
+        {
+            wf64x4_t re, im;
+        };
+        static __device__ inline S   stage(E e) { return e; }
+        static __device__ inline int kslot(int lane) { return lane >> 5; }
+        static __device__ inline XF  prep_x(S s, int lane)
+        {
+            return ((lane >> 4) & 1) ? make_double2(-s.y, s.x) : make_double2(s.x, s.y);
+        }
+        static __device__ inline YF   prep_y(S s, int lane) { return ((lane >> 4) & 1) ? s.y : s.x; }
+        static __device__ inline void zero(Acc& a)
+        {
+#pragma unroll
+            for(int r = 0; r < 4; r++)
+            {
+                a.re[r] = 0.0;
+                a.im[r] = 0.0;
+            }
+        }
+        static __device__ inline void mma(XF x, YF y, Acc& a)
+        {
+            a.re = __builtin_amdgcn_mfma_f64_16x16x4f64(x.x, y, a.re, 0, 0, 0);
+            a.im = __builtin_amdgcn_mfma_f64_16x16x4f64(x.y, y, a.im, 0, 0, 0);
+        }
+        static __device__ inline int p_of(int r, int lane) { return 4 * r + (lane >> 4); }
+        static __device__ inline int q_of(int lane) { return lane & 15; }
+        static __device__ inline O   get(const Acc& a, int r) { return make_double2(a.re[r], a.im[r]); }
+        static __device__ inline E finish(O x, const double* al, const double* be, bool bil, const E* c)
+        {
+            const double ar = al[0], ai = al[1];
+            double       yr = __dsub_rn(__dmul_rn(ar, x.x), __dmul_rn(ai, x.y));
+            double       yi = __dadd_rn(__dmul_rn(ai, x.x), __dmul_rn(ar, x.y));
+            if(bil)
+            {
+                const double  br = be[0], bi = be[1];
+                const double2 cv = *c;
+                yr = __dadd_rn(yr, __dsub_rn(__dmul_rn(br, cv.x), __dmul_rn(bi, cv.y)));
+                yi = __dadd_rn(yi, __dadd_rn(__dmul_rn(bi, cv.x), __dmul_rn(br, cv.y)));
+            }
+            return make_double2(yr, yi);
+        }
+    };
+
+    // ---- staging: global -> registers -> LDS tile[k][BR + PAD] ---------------------
+
+    template <typename Tr, int BR, int BK, int NT>
+    struct WStager
+    {
+        typedef typename Tr::E E;
+        typedef typename Tr::S S;
+        static constexpr int   V     = Tr::VMAX;
+        static constexpr int   N     = BR * BK / NT; // elements per thread
+        static constexpr int   PAD   = (sizeof(S) >= 8 ? 2 : 4);
+        static constexpr int   PITCH = BR + PAD;
+        static constexpr int   ELEMS = BK * PITCH;
+        static_assert(BR * BK % NT == 0 && N % V == 0, "tile must split evenly over threads");
+        static_assert(NT % (BR / V) == 0 && NT % BK == 0 && NT % (BK / V) == 0, "thread mapping");
+
+        E       data[N];
+        int32_t off[N]; // varying-table offsets (k for MN vectors, rows otherwise)
+        int32_t fixed; // the other table's offset
+        int     mode, a, b;
+
+        __device__ inline void init(int mode_, const int32_t* rtab, int r0, int tid)
+        {
+            mode = mode_;
+            if(mode == GATHER_MN_VEC)
+            {
+                constexpr int PER = BR / V;
+                a                 = tid % PER;
+                b                 = tid / PER;
+                fixed             = rtab[r0 + a * V];
+            }
+            else if(mode == GATHER_K_VEC)
+            {
+                constexpr int PER = BK / V, STEP = NT / PER;
+                a = tid % PER;
+                b = tid / PER;
+#pragma unroll
+                for(int i = 0; i < N / V; i++)
+                    off[i] = rtab[r0 + b + i * STEP];
+            }
+            else
+            {
+                constexpr int STEP = NT / BK;
+                a                  = tid % BK;
+                b                  = tid / BK;
+#pragma unroll
+                for(int i = 0; i < N; i++)
+                    off[i] = rtab[r0 + b + i * STEP];
+            }
+        }
+
+        __device__ inline void load_koffs(const int32_t* ktab, int k0)
+        {
+            if(mode == GATHER_MN_VEC)
+            {
+                constexpr int STEP = NT / (BR / V);
+#pragma unroll
+                for(int i = 0; i < N / V; i++)
+                    off[i] = ktab[k0 + b + i * STEP];
+            }
+            else if(mode == GATHER_K_VEC)
+                fixed = ktab[k0 + a * V];
+            else
+                fixed = ktab[k0 + a];
+        }
+
+        template <int W>
+        static __device__ inline void vload(const E* p, bool ok, E* dst)
+        {
+            struct alignas(sizeof(E) * W) Pack
+            {
+                E e[W];
+            };
+            Pack v;
+#pragma unroll
+            for(int j = 0; j < W; j++)
+                v.e[j] = E{};
+            if(ok)
+                v = *(const Pack*)p;
+#pragma unroll
+            for(int j = 0; j < W; j++)
+                dst[j] = v.e[j];
+        }
+
+        __device__ inline void fetch(const void* base, int k0, int K)
+        {
+            const E* bp = (const E*)base;
+            if(mode == GATHER_MN_VEC)
+            {
+                constexpr int STEP = NT / (BR / V);
+#pragma unroll
+                for(int i = 0; i < N / V; i++)
+                    vload<V>(bp + ((uint32_t)fixed + (uint32_t)off[i]),
+                             (k0 + b + i * STEP) < K,
+                             &data[i * V]);
+            }
+            else if(mode == GATHER_K_VEC)
+            {
+                const bool ok = (k0 + a * V) < K;
+#pragma unroll
+                for(int i = 0; i < N / V; i++)
+                    vload<V>(bp + ((uint32_t)off[i] + (uint32_t)fixed), ok, &data[i * V]);
+            }
+            else
+            {
+                const bool ok = (k0 + a) < K;
+#pragma unroll
+                for(int i = 0; i < N; i++)
+                    vload<1>(bp + ((uint32_t)off[i] + (uint32_t)fixed), ok, &data[i]);
+            }
+        }
+
+        __device__ inline void commit(S* lds)
+        {
+            if(mode == GATHER_MN_VEC)
+            {
+                constexpr int STEP = NT / (BR / V);
+#pragma unroll
+                for(int i = 0; i < N / V; i++)
+#pragma unroll
+                    for(int j = 0; j < V; j++)
+                        lds[(b + i * STEP) * PITCH + a * V + j] = Tr::stage(data[i * V + j]);
+            }
+            else if(mode == GATHER_K_VEC)
+            {
+                constexpr int STEP = NT / (BK / V);
+#pragma unroll
+                for(int i = 0; i < N / V; i++)
+#pragma unroll
+                    for(int j = 0; j < V; j++)
+                        lds[(a * V + j) * PITCH + b + i * STEP] = Tr::stage(data[i * V + j]);
+            }
+            else
+            {
+                constexpr int STEP = NT / BK;
+#pragma unroll
+                for(int i = 0; i < N; i++)
+                    lds[a * PITCH + b + i * STEP] = Tr::stage(data[i]);
+            }
+        }
+    };
+
+    template <typename Tr, int BP, int BQ, int BK, int WP, int WQ>
+    __global__ void __launch_bounds__(WP* WQ * 64) contract_w_kernel(const KArgs a, int xmode, int ymode)
+    {
+        constexpr int NT   = WP * WQ * 64;
+        constexpr int TILE = Tr::TILE;
+        constexpr int WTP = BP / WP, WTQ = BQ / WQ;
+        constexpr int TP = WTP / TILE, TQ = WTQ / TILE;
+        static_assert(WTP % TILE == 0 && WTQ % TILE == 0 && BK % Tr::KM == 0, "tile shape");
+        typedef typename Tr::S        S;
+        typedef typename Tr::E        E;
+        typedef typename Tr::O        O;
+        typedef WStager<Tr, BP, BK, NT> SX;
+        typedef WStager<Tr, BQ, BK, NT> SY;
+        constexpr int                 STAGE = SX::ELEMS + SY::ELEMS;
+
+        extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+        S* lds = (S*)lds_raw;
+
+        const int tid  = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = tid >> 6;
+        const int wp   = wave / WQ;
+        const int wq   = wave % WQ;
+
+        int tp, tq;
+        tile_coords(blockIdx.x, a.tiles_p, a.tiles_q, tp, tq);
+        const int p0 = tp * BP;
+        const int q0 = tq * BQ;
+
+        const int kt_begin = blockIdx.z * a.ktiles_per_split;
+        int       kt_end   = kt_begin + a.ktiles_per_split;
+        const int kt_all   = (a.K + BK - 1) / BK;
+        if(kt_end > kt_all)
+            kt_end = kt_all;
+
+        SX sx;
+        SY sy;
+        sx.init(xmode, a.xp, p0, tid);
+        sy.init(ymode, a.yq, q0, tid);
+
+        typename Tr::Acc acc[TP][TQ];
+#pragma unroll
+        for(int i = 0; i < TP; i++)
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+                Tr::zero(acc[i][j]);
+
+        const int row   = lane & (TILE - 1);
+        const int kslot = Tr::kslot(lane);
+        const int xfo   = kslot * SX::PITCH + wp * WTP + row;
+        const int yfo   = kslot * SY::PITCH + wq * WTQ + row;
+
+        if(kt_begin < kt_end)
+        {
+            sx.load_koffs(a.xk, kt_begin * BK);
+            sy.load_koffs(a.yk, kt_begin * BK);
+            sx.fetch(a.X, kt_begin * BK, a.K);
+            sy.fetch(a.Y, kt_begin * BK, a.K);
+        }
+
+        int buf = 0;
+        for(int kt = kt_begin; kt < kt_end; kt++)
+        {
+            S* lx = lds + buf * STAGE;
+            S* ly = lx + SX::ELEMS;
+            sx.commit(lx);
+            sy.commit(ly);
+            __syncthreads();
+            if(kt + 1 < kt_end)
+            {
+                sx.load_koffs(a.xk, (kt + 1) * BK);
+                sy.load_koffs(a.yk, (kt + 1) * BK);
+                sx.fetch(a.X, (kt + 1) * BK, a.K);
+                sy.fetch(a.Y, (kt + 1) * BK, a.K);
+            }
+#pragma unroll
+            for(int ks = 0; ks < BK / Tr::KM; ks++)
+            {
+                typename Tr::XF xf[TP];
+                typename Tr::YF yf[TQ];
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+                    xf[i] = Tr::prep_x(lx[xfo + ks * Tr::KM * SX::PITCH + i * TILE], lane);
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+                    yf[j] = Tr::prep_y(ly[yfo + ks * Tr::KM * SY::PITCH + j * TILE], lane);
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+#pragma unroll
+                    for(int j = 0; j < TQ; j++)
+                        Tr::mma(xf[i], yf[j], acc[i][j]);
+            }
+            buf ^= 1;
+        }
+
+        // ---- epilogue ----
+        const int pw = p0 + wp * WTP;
+        const int qw = q0 + wq * WTQ + Tr::q_of(lane);
+        if(a.split_k > 1)
+        {
+            O* ws = (O*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+            {
+                const int q = qw + j * TILE;
+                if(q >= a.Q)
+                    continue;
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+#pragma unroll
+                    for(int r = 0; r < Tr::NREG; r++)
+                    {
+                        const int p = pw + i * TILE + Tr::p_of(r, lane);
+                        if(p < a.P)
+                            ws[(size_t)p * a.Q + q] = Tr::get(acc[i][j], r);
+                    }
+            }
+            return;
+        }
+        E*         Dp  = (E*)a.D;
+        const E*   Cp  = (const E*)a.C;
+        const bool bil = a.bilinear != 0;
+#pragma unroll
+        for(int j = 0; j < TQ; j++)
+        {
+            const int q = qw + j * TILE;
+            if(q >= a.Q)
+                continue;
+            const uint32_t dqo = (uint32_t)a.dq[q];
+            const uint32_t cqo = bil ? (uint32_t)a.cq[q] : 0u;
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+#pragma unroll
+                for(int r = 0; r < Tr::NREG; r++)
+                {
+                    const int p = pw + i * TILE + Tr::p_of(r, lane);
+                    if(p < a.P)
+                    {
+                        const E* cptr = bil ? Cp + ((uint32_t)a.cp[p] + cqo) : nullptr;
+                        Dp[(uint32_t)a.dp[p] + dqo]
+                            = Tr::finish(Tr::get(acc[i][j], r), a.alpha, a.beta, bil, cptr);
+                    }
+                }
+        }
+    }
+
+    template <typename Tr, int BP, int BQ, int BK>
+    constexpr int lds_bytes_w()
+    {
+        return 2 * (WStager<Tr, BP, BK, 256>::ELEMS + WStager<Tr, BQ, BK, 256>::ELEMS)
+               * (int)sizeof(typename Tr::S);
+    }
+
+    template <typename Tr, int BP, int BQ, int BK, int WP, int WQ, int XM, int YM>
+    int launch_w(const KArgs& a, hipStream_t stream)
+    {
+        static_assert(WP * WQ * 64 == 256, "wide kernels use 256 threads");
+        constexpr int LDS  = lds_bytes_w<Tr, BP, BQ, BK>();
+        auto          kern = contract_w_kernel<Tr, BP, BQ, BK, WP, WQ>;
+        static const hipError_t attr = hipFuncSetAttribute(
+            (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+        if(attr != hipSuccess)
+            return (int)attr;
+        dim3 grid(a.tiles_p * a.tiles_q, 1, a.split_k);
+        hipLaunchKernelGGL(kern, grid, dim3(256), LDS, stream, a, XM, YM);
+        return (int)hipGetLastError();
+    }
+}
+
+// gather mode <-> (kfast, vec) as the registry describes it
+#define HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, XM, YM)                                      \
+    {                                                                                          \
+        hiptk::TR::CLS, ID, (XM != hiptk::GATHER_MN_VEC), (YM != hiptk::GATHER_MN_VEC),        \
+            (XM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX),                                \
+            (YM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX), BP, BQ, BK, 256,               \
+            hiptk::lds_bytes_w<hiptk::TR, BP, BQ, BK>(), #TR "_" #BP "x" #BQ "x" #BK "_" #XM #YM, \
+            &hiptk::launch_w<hiptk::TR, BP, BQ, BK, WP, WQ, XM, YM>                            \
+    }
+
+#define HIPTK_W_TILE(TR, ID, BP, BQ, BK, WP, WQ)                                               \
+    HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 0, 0), HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 0, 1), \
+        HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 0, 2),                                       \
+        HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 1, 0),                                       \
+        HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 1, 1),                                       \
+        HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 1, 2),                                       \
+        HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 2, 0),                                       \
+        HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 2, 1),                                       \
+        HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 2, 2)

@@ -1,0 +1,73 @@
+// Device-side argument block shared by every contraction kernel, and the launcher
+// signature each kernel family exports to the dispatcher.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "hiptk_kernels.h"
+
+namespace hiptk
+{
+    struct KArgs
+    {
+        const void* X; // rows operand   (MFMA "A": register-varying output index p)
+        const void* Y; // columns operand (MFMA "B": lane-varying output index q)
+        const void* C;
+        void*       D;
+        void*       ws; // split-K partials, [split][P][Q] accumulator-typed
+        const int32_t *xp, *xk, *yq, *yk, *cp, *cq, *dp, *dq;
+        int32_t P, Q, K;
+        int32_t ktiles_per_split; // K tiles (of BK) each z-slice reduces
+        int32_t split_k;
+        int32_t bilinear;
+        int32_t tiles_p, tiles_q;
+        double  alpha[2], beta[2];
+    };
+
+    // Tile-level launcher: returns hipError_t as int.
+    typedef int (*launch_fn)(const KArgs&, hipStream_t);
+
+    struct KernelEntry
+    {
+        int32_t     cls, tile_id;
+        int32_t     x_kfast, y_kfast, x_vec, y_vec;
+        int32_t     bp, bq, bk, threads, lds_bytes;
+        const char* name;
+        launch_fn   launch;
+    };
+
+    // Each kernel translation unit contributes its table.
+    const KernelEntry* entries_f16_vec(int* count);
+    const KernelEntry* entries_f16_gen(int* count);
+    const KernelEntry* entries_bf16_vec(int* count);
+    const KernelEntry* entries_bf16_gen(int* count);
+    const KernelEntry* entries_f32(int* count);
+    const KernelEntry* entries_f64(int* count);
+    const KernelEntry* entries_c32(int* count);
+    const KernelEntry* entries_c64(int* count);
+    const KernelEntry* entries_f64_as_f32(int* count);
+
+    // XCD-aware mapping of the linear workgroup id to an output tile.  Workgroups are
+    // handed to the 8 XCDs round-robin, so ids that are congruent mod 8 share an L2.
+    // Give each XCD a contiguous band of the tile space and walk that band in
+    // column-groups of GROUP rows so that the X rows / Y columns a band touches
+    // stay resident in that XCD's L2.
+    __device__ inline void tile_coords(int wg, int tiles_p, int tiles_q, int& tp, int& tq)
+    {
+        const int total = tiles_p * tiles_q;
+        int       lin   = wg;
+        if(total % 8 == 0)
+        {
+            const int per = total / 8;
+            lin           = (wg & 7) * per + (wg >> 3);
+        }
+        constexpr int GROUP = 4;
+        const int     band  = GROUP * tiles_q;
+        const int     g     = lin / band;
+        const int     first = g * GROUP;
+        const int     rows  = (tiles_p - first) < GROUP ? (tiles_p - first) : GROUP;
+        const int     r     = lin - g * band;
+        tp                  = first + r % rows;
+        tq                  = r / rows;
+    }
+}

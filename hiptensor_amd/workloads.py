@@ -1,0 +1,300 @@
+"""Benchmark / test workloads of the contraction path and their seeded inputs.
+
+A workload is a plain dict:
+  dtype    "f16" | "bf16" | "f32" | "f64" | "c32" | "c64"
+  compute  hiptensorComputeType_t value
+  modes    {"A": [...], "B": [...], "D": [...]}   mode labels (ints)
+  extent   {label: extent}
+  strides  {"A": [...], "B": [...], "C": [...] or None, "D": [...]}  in elements, per listed mode
+  alpha, beta   python float or complex; beta None => scale (no C)
+
+Input values follow the closed form of the reference's test harness
+(test/device/common.hpp:68-108): value(i) = (float(pcg_hash(i + seed)) / 2^32 - 0.5) * 2
+cast to the element type, with seeds 255 / 256 / 257 for A / B / C
+(test/01_contraction/contraction_test.cpp:381-476).  The element whose packed index over
+the tensor's listed modes (first listed fastest) is i receives value(i) and is stored at
+its strided offset; padding between elements is NaN so that a stray read poisons the
+result.  Complex tensors draw re from `seed` and im from `seed + 0x9E3779B9`
+(the reference's own fill sets im = re; independent parts exercise the kernels harder).
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import api
+
+HIP_TYPE = {"f32": api.HIP_R_32F, "f64": api.HIP_R_64F, "f16": api.HIP_R_16F,
+            "bf16": api.HIP_R_16BF, "c32": api.HIP_C_32F, "c64": api.HIP_C_64F}
+ELEM_BYTES = {"f16": 2, "bf16": 2, "f32": 4, "f64": 8, "c32": 8, "c64": 16}
+# numpy storage type (bf16 is kept as its 16-bit pattern)
+NP_STORE = {"f16": np.float16, "bf16": np.uint16, "f32": np.float32, "f64": np.float64,
+            "c32": np.complex64, "c64": np.complex128}
+SEED_A, SEED_B, SEED_C = 255, 256, 257
+IM_SEED_OFFSET = 0x9E3779B9
+
+
+def pcg_hash(x):
+    x = np.asarray(x, dtype=np.uint32)
+    with np.errstate(over="ignore"):
+        state = x * np.uint32(747796405) + np.uint32(2891336453)
+        shift = (state >> np.uint32(28)) + np.uint32(4)
+        word = ((state >> shift) ^ state) * np.uint32(277803737)
+        return (word >> np.uint32(22)) ^ word
+
+
+def gen_values(n, seed):
+    """float32 values in [-1, 1) for packed indices 0..n-1."""
+    idx = (np.arange(n, dtype=np.uint64) + np.uint64(seed)) % np.uint64(0xFFFFFFFF)
+    h = pcg_hash(idx.astype(np.uint32))
+    return (h.astype(np.float32) / np.float32(4294967296.0) - np.float32(0.5)) * np.float32(2.0)
+
+
+def f32_to_bf16_bits(x):
+    """Round-to-nearest-even float32 -> bf16 bit pattern (uint16)."""
+    b = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    nan = (b & np.uint32(0x7F800000)) == np.uint32(0x7F800000)
+    with np.errstate(over="ignore"):
+        r = b + np.uint32(0x7FFF) + ((b >> np.uint32(16)) & np.uint32(1))
+    r = np.where(nan, np.where((b & np.uint32(0xFFFF)) != 0, b | np.uint32(0x10000), b), r)
+    return (r >> np.uint32(16)).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b):
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def span_elems(lens, strides):
+    return 1 + sum((l - 1) * s for l, s in zip(lens, strides)) if all(l > 0 for l in lens) else 0
+
+
+def packed_strides(lens):
+    """Generalised column-major: first listed mode fastest."""
+    out, s = [], 1
+    for l in lens:
+        out.append(s)
+        s *= l
+    return out
+
+
+def storage_order_strides(listed, lens_by_mode, order, pad_after_first=0):
+    """Strides (per listed mode) of a tensor stored with `order[0]` fastest; the leading
+    dimension (stride of order[1]) is padded by `pad_after_first` elements."""
+    stride, s = {}, 1
+    for i, m in enumerate(order):
+        stride[m] = s
+        s *= lens_by_mode[m]
+        if i == 0:
+            s += pad_after_first
+    return [stride[m] for m in listed]
+
+
+def fill_tensor(dtype, lens, strides, seed, nan_gaps=True):
+    """Host buffer (1-D numpy array of the storage type, span elements) with seeded values."""
+    n = int(np.prod(lens)) if lens else 1
+    span = span_elems(lens, strides) if lens else 1
+    if dtype in ("c32", "c64"):
+        vals = gen_values(n, seed).astype(np.float64) + 1j * gen_values(n, seed + IM_SEED_OFFSET).astype(np.float64)
+        vals = vals.astype(NP_STORE[dtype])
+        gap = np.nan + 1j * np.nan
+    elif dtype == "bf16":
+        vals = f32_to_bf16_bits(gen_values(n, seed))
+        gap = np.uint16(0x7FC0)
+    else:
+        vals = gen_values(n, seed).astype(NP_STORE[dtype])
+        gap = np.nan
+    buf = np.empty(span, dtype=NP_STORE[dtype])
+    if span != n and nan_gaps:
+        buf[...] = gap
+    elif span != n:
+        buf[...] = 0
+    if not lens:
+        buf[0] = vals[0]
+        return buf
+    item = buf.dtype.itemsize
+    view = np.lib.stride_tricks.as_strided(buf, shape=tuple(lens), strides=tuple(s * item for s in strides))
+    view[...] = vals.reshape(tuple(lens), order="F")
+    return buf
+
+
+def nan_buffer(dtype, span):
+    buf = np.empty(span, dtype=NP_STORE[dtype])
+    if dtype == "bf16":
+        buf[...] = np.uint16(0x7FC0)
+    elif dtype in ("c32", "c64"):
+        buf[...] = np.nan + 1j * np.nan
+    else:
+        buf[...] = np.nan
+    return buf
+
+
+def to_float(dtype, arr):
+    """Storage array -> float64 / complex128 numpy array for comparisons."""
+    if dtype == "bf16":
+        return bf16_bits_to_f32(arr).astype(np.float64)
+    if dtype in ("c32", "c64"):
+        return arr.astype(np.complex128)
+    return arr.astype(np.float64)
+
+
+def scalar_ctype(compute, value):
+    """ctypes object holding alpha / beta in the layout of the compute type."""
+    if value is None:
+        return None
+    if compute == api.HIPTENSOR_COMPUTE_32F:
+        return C.c_float(float(value))
+    if compute == api.HIPTENSOR_COMPUTE_64F:
+        return C.c_double(float(value))
+    if compute == api.HIPTENSOR_COMPUTE_C32F:
+        v = complex(value)
+        return (C.c_float * 2)(v.real, v.imag)
+    if compute == api.HIPTENSOR_COMPUTE_C64F:
+        v = complex(value)
+        return (C.c_double * 2)(v.real, v.imag)
+    if compute == api.HIPTENSOR_COMPUTE_16F:
+        return C.c_uint16(int(np.float16(value).view(np.uint16)))
+    if compute == api.HIPTENSOR_COMPUTE_16BF:
+        return C.c_uint16(int(f32_to_bf16_bits(np.float32(value))))
+    raise ValueError(f"compute type {compute}")
+
+
+def make_workload(dtype, compute, modeA, modeB, modeD, extent, alpha, beta,
+                  strideA=None, strideB=None, strideC=None, strideD=None, name=""):
+    lens = {t: [extent[m] for m in modes] for t, modes in (("A", modeA), ("B", modeB), ("D", modeD))}
+    w = {
+        "name": name, "dtype": dtype, "compute": compute,
+        "modes": {"A": list(modeA), "B": list(modeB), "D": list(modeD)},
+        "extent": dict(extent), "lens": lens, "alpha": alpha, "beta": beta,
+        "strides": {
+            "A": list(strideA) if strideA is not None else packed_strides(lens["A"]),
+            "B": list(strideB) if strideB is not None else packed_strides(lens["B"]),
+            "D": list(strideD) if strideD is not None else packed_strides(lens["D"]),
+        },
+    }
+    w["strides"]["C"] = None if beta is None else (list(strideC) if strideC is not None else list(w["strides"]["D"]))
+    return w
+
+
+def dims(w):
+    """(M, N, K) of the flattened problem."""
+    a, b, d = set(w["modes"]["A"]), set(w["modes"]["B"]), set(w["modes"]["D"])
+    M = int(np.prod([w["extent"][m] for m in w["modes"]["D"] if m in a] or [1]))
+    N = int(np.prod([w["extent"][m] for m in w["modes"]["D"] if m in b] or [1]))
+    K = int(np.prod([w["extent"][m] for m in w["modes"]["A"] if m in b and m not in d] or [1]))
+    return M, N, K
+
+
+def flops(w):
+    M, N, K = dims(w)
+    return (8.0 if w["dtype"] in ("c32", "c64") else 2.0) * M * N * K
+
+
+def algorithmic_bytes(w):
+    """Every logical element of A, B, (C,) D touched once."""
+    M, N, K = dims(w)
+    e = ELEM_BYTES[w["dtype"]]
+    return e * (M * K + N * K + M * N * (2 if w["beta"] is not None else 1))
+
+
+# ---------------------------------------------------------------------------
+# The configurations the benchmark is quoted on.
+# Mode labels: m* = 0.., n* = 10.., k* = 20..
+# ---------------------------------------------------------------------------
+
+def _rank4(dtype, compute, m, n, k, alpha, beta, name):
+    ext = {0: m[0], 1: m[1], 10: n[0], 11: n[1], 20: k[0], 21: k[1]}
+    return make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, alpha, beta, name=name)
+
+
+def config1():
+    return _rank4("f32", api.HIPTENSOR_COMPUTE_32F, (16, 16), (16, 16), (16, 16), 1.1, 0.9, "cfg1_f32_bilinear_256")
+
+
+def config2(dtype="f16", bilinear=False):
+    return _rank4(dtype, api.HIPTENSOR_COMPUTE_32F, (64, 64), (64, 64), (64, 64), 1.0,
+                  1.0 if bilinear else None, f"cfg2_{dtype}_{'bilinear' if bilinear else 'scale'}_4096")
+
+
+def config3():
+    return _rank4("f64", api.HIPTENSOR_COMPUTE_64F, (48, 40), (48, 40), (32, 24), 2.0, -0.5, "cfg3_f64_bilinear_1920x1920x768")
+
+
+def config4():
+    return _rank4("c32", api.HIPTENSOR_COMPUTE_C32F, (32, 32), (32, 32), (32, 16), 1.0 + 0.5j, 0.25 - 0.75j,
+                  "cfg4_c32_bilinear_1024x1024x512")
+
+
+def config5(scale=1):
+    """Rank-6 f16 bilinear with permuted A / B storage and a padded leading dimension on C / D.
+    `scale` > 1 divides the three largest extents (for parity runs the oracle can finish)."""
+    m0, m1, m2, n0, n1, n2, k0, k1, k2 = 0, 1, 2, 10, 11, 12, 20, 21, 22
+    ext = {m0: 32, m1: 7, m2: 24 // scale, n0: 24, n1: 9, n2: 32 // scale, k0: 17, k1: 8, k2: 30 // scale}
+    mA, mB, mD = [m0, m1, m2, k0, k1, k2], [n0, n1, n2, k0, k1, k2], [m0, m1, m2, n0, n1, n2]
+    sA = storage_order_strides(mA, ext, [k1, m0, k0, m2, m1, k2])
+    sB = storage_order_strides(mB, ext, [n2, k0, n0, k2, k1, n1])
+    sD = storage_order_strides(mD, ext, mD, pad_after_first=8)
+    return make_workload("f16", api.HIPTENSOR_COMPUTE_32F, mA, mB, mD, ext, 1.0, 1.0,
+                         strideA=sA, strideB=sB, strideC=sD, strideD=sD,
+                         name="cfg5_f16_bilinear_rank6_permuted" + (f"_div{scale}" if scale > 1 else ""))
+
+
+def baseline_configs():
+    return {
+        "cfg1": config1(),
+        "cfg2_f16_scale": config2("f16", False),
+        "cfg2_bf16_scale": config2("bf16", False),
+        "cfg2_f16_bilinear": config2("f16", True),
+        "cfg2_bf16_bilinear": config2("bf16", True),
+        "cfg3": config3(),
+        "cfg4": config4(),
+        "cfg5": config5(),
+    }
+
+
+def host_inputs(w, nan_gaps=True):
+    """Seeded host buffers {"A", "B", "C" (or None)} plus spans."""
+    A = fill_tensor(w["dtype"], w["lens"]["A"], w["strides"]["A"], SEED_A, nan_gaps)
+    B = fill_tensor(w["dtype"], w["lens"]["B"], w["strides"]["B"], SEED_B, nan_gaps)
+    Cb = None
+    if w["beta"] is not None:
+        Cb = fill_tensor(w["dtype"], w["lens"]["D"], w["strides"]["C"], SEED_C, nan_gaps)
+    return {"A": A, "B": B, "C": Cb, "spanD": span_elems(w["lens"]["D"], w["strides"]["D"])}
+
+
+class Contraction:
+    """Descriptor -> find -> workspace -> plan for one workload, through the public API."""
+
+    def __init__(self, handle, w, algo=api.HIPTENSOR_ALGO_DEFAULT, pref=api.HIPTENSOR_WORKSPACE_RECOMMENDED,
+                 align=16, workspace_limit=None):
+        self.handle, self.w = handle, w
+        t = HIP_TYPE[w["dtype"]]
+        chk = api.check
+        self.dA = chk(api.hiptensorInitTensorDescriptor(handle, w["lens"]["A"], w["strides"]["A"], t), "descA")
+        self.dB = chk(api.hiptensorInitTensorDescriptor(handle, w["lens"]["B"], w["strides"]["B"], t), "descB")
+        self.dD = chk(api.hiptensorInitTensorDescriptor(handle, w["lens"]["D"], w["strides"]["D"], t), "descD")
+        bil = w["beta"] is not None
+        self.dC = chk(api.hiptensorInitTensorDescriptor(handle, w["lens"]["D"], w["strides"]["C"], t), "descC") if bil else None
+        m = w["modes"]
+        self.desc = chk(api.hiptensorInitContractionDescriptor(
+            handle, self.dA, m["A"], align, self.dB, m["B"], align,
+            self.dC, m["D"] if bil else None, align if bil else 0, self.dD, m["D"], align, w["compute"]), "contraction desc")
+        self.find = chk(api.hiptensorInitContractionFind(handle, algo), "find")
+        self.workspace_bytes = chk(api.hiptensorContractionGetWorkspaceSize(handle, self.desc, self.find, pref), "workspace")
+        if workspace_limit is not None:
+            self.workspace_bytes = min(self.workspace_bytes, workspace_limit)
+        self.plan = chk(api.hiptensorInitContractionPlan(handle, self.desc, self.find, self.workspace_bytes), "plan")
+        self.info = api.planInfo(self.plan)
+        self.alpha = scalar_ctype(w["compute"], w["alpha"])
+        self.beta = scalar_ctype(w["compute"], w["beta"])
+
+    def run(self, A, B, Cb, D, workspace=None, stream=0, workspace_bytes=None):
+        """A, B, Cb, D, workspace: device addresses (ints)."""
+        return api.hiptensorContraction(
+            self.handle, self.plan, self.alpha, A, B, self.beta, Cb, D, workspace,
+            self.workspace_bytes if workspace_bytes is None else workspace_bytes, stream or None)
+
+    def close(self):
+        api.destroy("plan", self.plan)
+        api.destroy("find", self.find)
+        api.destroy("contraction", self.desc)
+        for d in (self.dA, self.dB, self.dC, self.dD):
+            api.destroy("tensor", d)

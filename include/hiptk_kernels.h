@@ -1,0 +1,116 @@
+/*
+ * Kernel-layer C ABI: the only interface between the host-side planner (plain
+ * C++) and the HIP translation units.  Everything crossing it is a plain pointer,
+ * an integer or the POD below; no kernel template is visible to host code.
+ *
+ * It takes the place of the Composable Kernel device-operation objects that the
+ * reference drives through BaseOperator / BaseArgument / BaseInvoker pointers
+ * (library/src/contraction/contraction_solution.hpp:147-150) and whose Run() is
+ * the device boundary (library/src/contraction/contraction_solution.cpp:258).
+ *
+ * A contraction arrives here already folded into one GEMM view
+ *     acc[p][q] = sum_k X[xp[p] + xk[k]] * Y[yq[q] + yk[k]]
+ *     D[dp[p] + dq[q]] = alpha * acc[p][q] (+ beta * C[cp[p] + cq[q]])
+ * where the eight offset tables (element units, device memory) carry every mode
+ * extent and stride of the original tensors.
+ */
+#ifndef HIPTK_KERNELS_H
+#define HIPTK_KERNELS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element classes the kernels are instantiated for */
+enum
+{
+    HIPTK_F16  = 0, /* f16 storage, f16 MFMA inputs, f32 accumulate        */
+    HIPTK_BF16 = 1, /* bf16 storage, bf16 MFMA inputs, f32 accumulate      */
+    HIPTK_F32  = 2, /* f32 storage, f32 MFMA                              */
+    HIPTK_F64  = 3, /* f64 storage, f64 MFMA                              */
+    HIPTK_C32  = 4, /* complex f32 storage, f32 MFMA on (re,im) K pairs    */
+    HIPTK_C64  = 5, /* complex f64 storage, f64 MFMA on (re,im) K pairs    */
+    HIPTK_F32_AS_F16  = 6, /* f32 storage, inputs rounded to f16 when staged  */
+    HIPTK_F32_AS_BF16 = 7, /* f32 storage, inputs rounded to bf16 when staged */
+    HIPTK_F64_AS_F32  = 8, /* f64 storage, inputs narrowed to f32 when staged */
+    HIPTK_NUM_CLASSES = 9
+};
+
+enum
+{
+    HIPTK_OP_SCALE    = 0,
+    HIPTK_OP_BILINEAR = 1
+};
+
+enum
+{
+    HIPTK_OK             = 0,
+    HIPTK_ERR_ARG        = 1, /* malformed problem (caught on the host, nothing launched) */
+    HIPTK_ERR_NO_KERNEL  = 2, /* no instantiation for (class, tile, layout, vector)       */
+    HIPTK_ERR_WORKSPACE  = 3, /* split-K asked for and workspace too small                */
+    HIPTK_ERR_LAUNCH     = 4  /* hipLaunchKernel reported an error                        */
+};
+
+/* One tile configuration of one element class. */
+typedef struct hiptk_tile_info
+{
+    int32_t tile_id;
+    int32_t bp, bq, bk; /* workgroup tile                                    */
+    int32_t threads;    /* workgroup size                                    */
+    int32_t lds_bytes;  /* static LDS                                        */
+    char    name[64];
+} hiptk_tile_info_t;
+
+typedef struct hiptk_problem
+{
+    int32_t cls;     /* HIPTK_F16 ...                                         */
+    int32_t op;      /* HIPTK_OP_SCALE / HIPTK_OP_BILINEAR                    */
+    int32_t tile_id; /* index into the class's tile list                      */
+    int32_t split_k; /* >= 1; > 1 needs workspace                             */
+    int64_t P, Q, K; /* GEMM view extents (rows, columns, reduction)          */
+    /* offset tables, element units.  xp / cp / dp hold P entries padded up to a
+     * multiple of 256 with valid offsets; yq / cq / dq likewise for Q; xk / yk
+     * hold K entries padded with zeros up to a multiple of 256.               */
+    const int32_t *xp, *xk, *yq, *yk, *cp, *cq, *dp, *dq;
+    int32_t x_kfast; /* 1: X vectors run along k, 0: along p                   */
+    int32_t y_kfast; /* 1: Y vectors run along k, 0: along q                   */
+    int32_t x_vec;   /* contiguous elements per X vector (1 = scalar gather)   */
+    int32_t y_vec;
+    int32_t cd_vec;  /* contiguous elements along q shared by C and D          */
+    int32_t reserved;
+} hiptk_problem_t;
+
+/* Number of tile configurations of a class, and their description. */
+int hiptk_tile_count(int cls);
+int hiptk_tile_info(int cls, int tile_id, hiptk_tile_info_t* out);
+
+/* 1 when a kernel is instantiated for the problem's (class, tile, layout, vector)
+ * combination; its name ("" if none). */
+int         hiptk_kernel_available(const hiptk_problem_t* prob);
+const char* hiptk_kernel_name(const hiptk_problem_t* prob);
+
+/* Bytes of workspace the problem needs (0 when split_k == 1). */
+uint64_t hiptk_workspace_bytes(const hiptk_problem_t* prob);
+
+/* Enqueue the contraction on `stream` (a hipStream_t passed as void*).  alpha and
+ * beta point to host scalars: float for the 16/32-bit real classes, double for
+ * HIPTK_F64 and HIPTK_F64_AS_F32, float[2] for HIPTK_C32, double[2] for HIPTK_C64.
+ * Returns a HIPTK_* code; *hip_error (optional) receives the hipError_t. */
+int hiptk_contract(const hiptk_problem_t* prob,
+                   const void*            alpha,
+                   const void*            beta,
+                   const void*            X,
+                   const void*            Y,
+                   const void*            C,
+                   void*                  D,
+                   void*                  workspace,
+                   uint64_t               workspace_bytes,
+                   void*                  stream,
+                   int*                   hip_error);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPTK_KERNELS_H */
