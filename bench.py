@@ -1,0 +1,174 @@
+#!/usr/bin/env python3
+"""Benchmark of the contraction path on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all] [--no-cpu]
+
+A step is one hiptensorContraction call (through the flat C ABI) on inputs that are already
+resident in HBM; plan creation is outside the timed region.  The headline workload is the
+f16 scale contraction at M = N = K = 4096 (extents 64^6, packed column-major).  The run
+prints ONE JSON line: metric / value (TFLOP/s of the headline workload), a `roofline` object
+for its kernel (average launch duration measured with HIP events on the launch stream), a
+`cpu_baseline` object (the reference's own CPU contraction, or the oracle port, timed on a
+bounded slab of the same workload on this host) and, with --all, the other configurations.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# dense MFMA peaks of MI355X in TFLOP/s: 256 CUs x 2.4 GHz x {4096, 256, 128} flop/clk/CU
+PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "f32": 157.3, "c32": 157.3, "f64": 78.6, "c64": 78.6}
+FLOP_PER_CLK_CU = {"f16": 4096, "bf16": 4096, "f32": 256, "c32": 256, "f64": 128, "c64": 128}
+HBM_PEAK_GBS = 8000.0
+
+
+def measure(handle, w, steps, warmup):
+    """Returns dict(ms_per_step wall, kernel_ms from HIP events, info)."""
+    import torch
+
+    from hiptensor_amd import workloads as wl
+
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import gpu_util
+
+    inp = wl.host_inputs(w, nan_gaps=False)
+    A, B = gpu_util.to_device(inp["A"]), gpu_util.to_device(inp["B"])
+    Cd = gpu_util.to_device(inp["C"]) if inp["C"] is not None else None
+    D = torch.empty(inp["spanD"] * wl.ELEM_BYTES[w["dtype"]], dtype=torch.uint8, device="cuda")
+    c = wl.Contraction(handle, w)
+    ws = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream()
+    args = (A.data_ptr(), B.data_ptr(), Cd.data_ptr() if Cd is not None else None, D.data_ptr(),
+            ws.data_ptr() if c.workspace_bytes else None, stream.cuda_stream)
+    for _ in range(warmup):
+        assert c.run(*args) == 0
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(steps):
+        st = c.run(*args)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    assert st == 0
+    out = {"ms_per_step": (t1 - t0) * 1e3 / steps, "kernel_ms": e0.elapsed_time(e1) / steps, "info": dict(c.info)}
+    c.close()
+    return out
+
+
+def cpu_baseline(w, budget_macs=1.2e9):
+    """Times the CPU contraction on a slab of the workload: the outputs whose slowest M mode
+    lies in a leading sub-range, full N and K.  Uses the compiled reference when oracle/_ref
+    is present, else the oracle port."""
+    import numpy as np
+
+    import oracle
+    from hiptensor_amd import workloads as wl
+
+    M, N, K = wl.dims(w)
+    # slowest M mode of D in listed order = the last M mode listed (packed column-major)
+    a_modes = set(w["modes"]["A"])
+    m_modes = [m for m in w["modes"]["D"] if m in a_modes]
+    slow = max(m_modes, key=lambda m: w["strides"]["D"][w["modes"]["D"].index(m)])
+    full = w["extent"][slow]
+    per = M // full * N * K
+    take = max(1, min(full, int(budget_macs // per)))
+    sub = dict(w, extent=dict(w["extent"]), lens={k: list(v) for k, v in w["lens"].items()})
+    sub["extent"][slow] = take
+    for t in ("A", "D"):
+        sub["lens"][t][w["modes"][t].index(slow)] = take
+    inp = wl.host_inputs(w, nan_gaps=False)  # full tensors: the slab reads a leading sub-range in place
+    threads = os.cpu_count() or 1
+    use_ref = oracle.ref_lib() is not None
+    t0 = time.perf_counter()
+    if use_ref:
+        oracle.ref_contract(sub, inp["A"], inp["B"], inp["C"])
+    else:
+        oracle.contract(sub, inp["A"], inp["B"], inp["C"], threads=threads)
+    dt = time.perf_counter() - t0
+    frac = take / full
+    fl = wl.flops(w) * frac
+    return {
+        "value": fl / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "reference" if use_ref else "port",
+        "sample": f"outputs with mode {slow} in [0,{take}) of {full} ({frac:.4f} of D), full N and K",
+        "ms_sample": dt * 1e3,
+        "ms_full_extrapolated": dt * 1e3 / frac,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg2_f16_scale")
+    ap.add_argument("--all", action="store_true", help="also time every other configuration")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus must be 1 (the path would shard by output "
+              "tiles across devices, which is not part of this run)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    from hiptensor_amd import api
+    from hiptensor_amd import workloads as wl
+
+    torch.zeros(1, device="cuda")
+    prop = torch.cuda.get_device_properties(0)
+    clock_ghz = getattr(prop, "clock_rate", 2400000) / 1e6
+    cus = prop.multi_processor_count
+    handle = api.check(api.hiptensorCreate(), "hiptensorCreate")
+    cfgs = wl.baseline_configs()
+    w = cfgs[a.workload]
+    r = measure(handle, w, a.steps, a.warmup)
+    fl = wl.flops(w)
+    tflops = fl / (r["kernel_ms"] * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[w["dtype"]]
+    M, N, K = wl.dims(w)
+    out = {
+        "metric": "contraction TFLOP/s (and fraction of dense MFMA peak) on 1 MI355X",
+        "value": fl / (r["ms_per_step"] * 1e-3) / 1e12,
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": r["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": w["name"], "M": M, "N": N, "K": K, "op": "bilinear" if w["beta"] is not None else "scale",
+                   "kernel": r["info"]["kernel_name"], "split_k": r["info"]["split_k"]},
+        "roofline": {"bound": "mfma", "achieved": tflops, "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak,
+                     "traffic": None, "kernel_ms": r["kernel_ms"],
+                     "peak_from_device_clock": cus * clock_ghz * FLOP_PER_CLK_CU[w["dtype"]] / 1e3,
+                     "hbm_GBs_algorithmic": wl.algorithmic_bytes(w) / (r["kernel_ms"] * 1e-3) / 1e9},
+        "device": {"name": prop.name, "cus": cus, "clock_ghz": clock_ghz},
+    }
+    if a.all:
+        others = {}
+        for name, cw in cfgs.items():
+            if name == a.workload:
+                continue
+            steps = max(5, a.steps // 2)
+            rr = measure(handle, cw, steps, a.warmup)
+            tf = wl.flops(cw) / (rr["kernel_ms"] * 1e-3) / 1e12
+            others[name] = {"kernel_ms": rr["kernel_ms"], "tflops": tf, "frac_peak": tf / PEAK_TFLOPS[cw["dtype"]],
+                            "hbm_GBs_algorithmic": wl.algorithmic_bytes(cw) / (rr["kernel_ms"] * 1e-3) / 1e9,
+                            "kernel": rr["info"]["kernel_name"], "split_k": rr["info"]["split_k"], "dtype": cw["dtype"]}
+        out["others"] = others
+    if not a.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(w)
+    api.hiptensorDestroy(handle)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -10,12 +10,15 @@ A workload is a plain dict:
 
 Input values follow the closed form of the reference's test harness
 (test/device/common.hpp:68-108): value(i) = (float(pcg_hash(i + seed)) / 2^32 - 0.5) * 2
-cast to the element type, with seeds 255 / 256 / 257 for A / B / C
-(test/01_contraction/contraction_test.cpp:381-476).  The element whose packed index over
-the tensor's listed modes (first listed fastest) is i receives value(i) and is stored at
-its strided offset; padding between elements is NaN so that a stray read poisons the
-result.  Complex tensors draw re from `seed` and im from `seed + 0x9E3779B9`
-(the reference's own fill sets im = re; independent parts exercise the kernels harder).
+cast to the element type.  The element whose packed index over the tensor's listed modes
+(first listed fastest) is i receives value(i) and is stored at its strided offset; padding
+between elements is NaN so that a stray read poisons the result.
+
+The harness seeds A, B, C with 255, 256, 257, which makes B the same stream as A shifted by
+one element: D then holds sums of squares that grow like K, and the CPU algorithm's own f32
+rounding error reaches the 1e-5 the results are compared at.  The workloads are specified
+as i.i.d. inputs, so the seeds here are 2^28 apart (tensors are smaller than that, so the
+index ranges the hash sees are disjoint); imaginary parts use the range 2^31 above.
 """
 import ctypes as C
 
@@ -29,8 +32,8 @@ ELEM_BYTES = {"f16": 2, "bf16": 2, "f32": 4, "f64": 8, "c32": 8, "c64": 16}
 # numpy storage type (bf16 is kept as its 16-bit pattern)
 NP_STORE = {"f16": np.float16, "bf16": np.uint16, "f32": np.float32, "f64": np.float64,
             "c32": np.complex64, "c64": np.complex128}
-SEED_A, SEED_B, SEED_C = 255, 256, 257
-IM_SEED_OFFSET = 0x9E3779B9
+SEED_A, SEED_B, SEED_C = 255, 256 + (1 << 28), 257 + (2 << 28)
+IM_SEED_OFFSET = 1 << 31
 
 
 def pcg_hash(x):

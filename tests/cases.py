@@ -103,8 +103,56 @@ def error_metric(dtype, got, ref):
     return float(np.max(np.abs(g - r) / (np.abs(g) + np.abs(r) + 1.0))) if g.size else 0.0
 
 
-# relative tolerance per element type, as the benchmark contract states them
+# Relative tolerance per element type, as the benchmark contract states them.
 TOLERANCE = {"f32": 1e-5, "c32": 1e-5, "f16": 1e-2, "bf16": 1e-2, "f64": 1e-12, "c64": 1e-12}
+
+
+def harness_tolerance(w):
+    """Tolerance of the reference's own GPU-vs-CPU comparison on its element-wise metric
+    (test/01_contraction/contraction_test.cpp:882-905): 2 K eps of the compute type, plus
+    2 * 2^-7 for bf16 and 2 * 2^-10 for f16 results."""
+    K = wl.dims(w)[2]
+    eps = np.finfo(np.float64).eps if w["dtype"] in ("f64", "c64") else np.finfo(np.float32).eps
+    t = 2.0 * K * eps
+    if w["dtype"] == "bf16":
+        t += 2.0 * 2.0 ** -7
+    if w["dtype"] == "f16":
+        t += 2.0 * 2.0 ** -10
+    return float(t)
+
+
+def relative_error(dtype, got, ref):
+    """max |d - r| / max |r|: the error relative to the magnitude of the reference result."""
+    g = wl.to_float(dtype, got)
+    r = wl.to_float(dtype, ref)
+    if np.iscomplexobj(g):
+        g = np.stack([g.real, g.imag])
+        r = np.stack([r.real, r.imag])
+    if not (np.all(np.isfinite(g)) and np.all(np.isfinite(r))):
+        return float("inf")
+    if g.size == 0:
+        return 0.0
+    return float(np.max(np.abs(g - r)) / max(float(np.max(np.abs(r))), np.finfo(np.float64).tiny))
+
+
+def assert_parity(w, got, ref, what=""):
+    """The two checks every GPU result must pass against the CPU oracle:
+
+    1. relative error (max |d - r| / max |r|) within the contract's tolerance for the
+       element type: 1e-5 f32 / c32, 1e-2 f16 / bf16, 1e-12 f64 / c64;
+    2. the reference harness's own element-wise metric |d - r| / (|d| + |r| + 1) within
+       the reference harness's own tolerance 2 K eps (+ 16-bit terms).
+
+    The element-wise metric turns into an absolute error for outputs near zero, where a
+    sequential f32 sum over K terms is itself a few K eps |partial| away from the exact
+    value (the CPU oracle is 2e-5 from the f64 result on the 1024 x 1024 x 512 complex
+    configuration), so it is held to the bound the reference uses, not to 1e-5.
+    NaN or Inf anywhere fails both."""
+    rel = relative_error(w["dtype"], got, ref)
+    elt = error_metric(w["dtype"], got, ref)
+    assert rel <= TOLERANCE[w["dtype"]], f"{w['name']} {what}: relative error {rel:.3e} > {TOLERANCE[w['dtype']]:.0e}"
+    assert elt <= harness_tolerance(w), f"{w['name']} {what}: element-wise metric {elt:.3e} > {harness_tolerance(w):.3e}"
+    return rel, elt
 
 
 def logical_view(w, buf):

@@ -1,0 +1,38 @@
+"""Runs a workload on the GPU through the public API (flat C ABI) with torch-owned buffers."""
+import numpy as np
+
+from hiptensor_amd import api
+from hiptensor_amd import workloads as wl
+
+
+def to_device(buf):
+    import torch
+
+    return torch.from_numpy(buf.view(np.uint8).copy()).cuda()
+
+
+def run_gpu(handle, w, inp=None, algo=api.HIPTENSOR_ALGO_DEFAULT, pref=api.HIPTENSOR_WORKSPACE_RECOMMENDED,
+            d_alias_c=False, workspace_limit=None, return_info=False):
+    """Returns D as a host array of the storage type (span elements)."""
+    import torch
+
+    if inp is None:
+        inp = wl.host_inputs(w)
+    A, B = to_device(inp["A"]), to_device(inp["B"])
+    Cd = to_device(inp["C"]) if inp["C"] is not None else None
+    if d_alias_c:
+        D = Cd
+    else:
+        D = to_device(wl.nan_buffer(w["dtype"], inp["spanD"]))
+    # alignment from the pointers, the way the reference's samples and tests obtain it
+    c = wl.Contraction(handle, w, algo=algo, pref=pref, workspace_limit=workspace_limit)
+    ws = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    st = c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr() if Cd is not None else None, D.data_ptr(),
+               ws.data_ptr() if c.workspace_bytes else None, stream)
+    torch.cuda.synchronize()
+    info = dict(c.info)
+    c.close()
+    api.check(st, "hiptensorContraction " + w["name"])
+    out = D.cpu().numpy().view(wl.NP_STORE[w["dtype"]])
+    return (out, info) if return_info else out

@@ -1,0 +1,108 @@
+"""GPU parity: the HIP path (through the flat C ABI) against the CPU oracle on the same
+seeded inputs, at sizes the oracle finishes in seconds.  Every comparison goes through
+cases.assert_parity: relative error within 1e-5 (f32, c32), 1e-2 (f16, bf16), 1e-12 (f64,
+c64), and the reference harness's element-wise metric within its own 2 K eps bound."""
+import numpy as np
+import pytest
+
+import cases
+import gpu_util
+from hiptensor_amd import api
+from hiptensor_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+ALL = ["f16", "bf16", "f32", "f64", "c32", "c64"]
+AB_REAL = [(0.0, 2.0), (1.0, None), (1.0, 2.0)]  # the reference's alpha / beta rows
+AB_CPLX = [(0.0 + 0.0j, 2.0 + 2.0j), (1.0 + 1.0j, None), (1.1 + 1.2j, 2.2 + 2.3j)]
+
+
+def _ab(dtype):
+    return AB_CPLX if dtype.startswith("c") else AB_REAL
+
+
+def check(handle, oracle_mod, w, **kw):
+    print(f"[case] {w['name']} dtype={w['dtype']} beta={w['beta']}", flush=True)
+    inp = wl.host_inputs(w)
+    exp = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
+    got, info = gpu_util.run_gpu(handle, w, inp, return_info=True, **kw)
+    # padding gaps of D must be left untouched (NaN), logical elements must match
+    gv, ev = cases.logical_view(w, got), cases.logical_view(w, exp)
+    cases.assert_parity(w, gv, ev, info["kernel_name"])
+    if got.size != gv.size:
+        mask = np.ones(got.size, dtype=bool)
+        mask[np.unique(np.lib.stride_tricks.as_strided(
+            np.arange(got.size), shape=tuple(w["lens"]["D"]),
+            strides=tuple(s * 8 for s in w["strides"]["D"])).ravel())] = False
+        gaps = wl.to_float(w["dtype"], got[mask])
+        assert np.all(np.isnan(gaps)), f"{w['name']}: wrote into D's padding"
+    return info
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("rank", [2, 3, 4, 5, 6])
+def test_rank_cases_default_strides(gpu_handle, oracle_mod, dtype, rank):
+    for alpha, beta in _ab(dtype):
+        check(gpu_handle, oracle_mod, cases.rank_case(rank, dtype, alpha, beta))
+
+
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("i", [0, 1, 2])
+def test_rank1_shapes(gpu_handle, oracle_mod, dtype, i):
+    for alpha, beta in _ab(dtype)[1:]:
+        check(gpu_handle, oracle_mod, cases.rank1_case(i, dtype, alpha, beta))
+
+
+@pytest.mark.parametrize("i", range(len(cases.MODE_CASES)))
+def test_mode_cases(gpu_handle, oracle_mod, i):
+    check(gpu_handle, oracle_mod, cases.mode_case(i, "c32", 1.1 + 1.2j, None))
+    check(gpu_handle, oracle_mod, cases.mode_case(i, "f16", 1.0, None))
+    check(gpu_handle, oracle_mod, cases.mode_case(i, "f64", 1.0, None))
+
+
+@pytest.mark.parametrize("dtype", ALL)
+def test_column_major_vector_paths(gpu_handle, oracle_mod, dtype):
+    """Packed column-major rank-4 problems whose runs are multiples of the vector width:
+    exercises the vectorised gathers (row-index-fast A and B, like the benchmark shapes)."""
+    a, b = _ab(dtype)[-1]
+    w = wl._rank4(dtype, cases.COMPUTE[dtype], (16, 6), (8, 10), (8, 9), a, b, f"colmajor_{dtype}")
+    info = check(gpu_handle, oracle_mod, w)
+    assert info["x_vec"] > 1 and info["y_vec"] > 1 or dtype == "c64"
+    # k-fast operands: A[k.., m..] style storage
+    ext = {0: 16, 1: 6, 10: 8, 11: 10, 20: 16, 21: 5}
+    mA, mB, mD = [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1]
+    w2 = wl.make_workload(dtype, cases.COMPUTE[dtype], mA, mB, mD, ext, a, b, name=f"kfast_{dtype}")
+    info = check(gpu_handle, oracle_mod, w2)
+    assert info["x_kfast"] == 1 and info["y_kfast"] == 1
+    # mixed: A k-fast, B n-fast
+    w3 = wl.make_workload(dtype, cases.COMPUTE[dtype], mA, [10, 11, 20, 21], [0, 1, 10, 11], ext, a, b, name=f"mixed_{dtype}")
+    check(gpu_handle, oracle_mod, w3)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32", "f64", "c32"])
+def test_tile_edges_and_k_tails(gpu_handle, oracle_mod, dtype):
+    """Extents that are not multiples of any tile: partial tiles in M, N and K."""
+    a, b = _ab(dtype)[-1]
+    for (m, n, k) in [((8, 37), (16, 19), (24, 5)), ((24, 11), (8, 3), (8, 41))]:
+        check(gpu_handle, oracle_mod, wl._rank4(dtype, cases.COMPUTE[dtype], m, n, k, a, b, f"edges_{dtype}_{m}_{n}_{k}"))
+
+
+def test_config5_layout_reduced(gpu_handle, oracle_mod):
+    """The benchmark's rank-6 permuted / padded layout at reduced extents."""
+    info = check(gpu_handle, oracle_mod, wl.config5(scale=2))
+    assert info["x_vec"] == 8 and info["y_vec"] == 8, info
+
+
+def test_invariants(gpu_handle, oracle_mod):
+    """alpha = 0 gives beta * C exactly; D may alias C."""
+    for dtype in ("f32", "f16", "f64", "c32"):
+        w = wl._rank4(dtype, cases.COMPUTE[dtype], (8, 5), (8, 7), (8, 6), 0.0, 2.0, f"alpha0_{dtype}")
+        inp = wl.host_inputs(w)
+        got = gpu_util.run_gpu(gpu_handle, w, inp)
+        exp = 2.0 * wl.to_float(dtype, inp["C"])
+        assert np.array_equal(wl.to_float(dtype, got), exp), dtype
+        w = wl._rank4(dtype, cases.COMPUTE[dtype], (8, 5), (8, 7), (8, 6), 1.0, 2.0, f"alias_{dtype}")
+        inp = wl.host_inputs(w)
+        ref = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
+        got = gpu_util.run_gpu(gpu_handle, w, inp, d_alias_c=True)
+        cases.assert_parity(w, got, ref, "D aliasing C")
