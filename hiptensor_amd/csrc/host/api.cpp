@@ -729,6 +729,9 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         p.x_vec                = v.x_vec;
         p.y_vec                = v.y_vec;
         p.cd_vec               = v.cd_vec;
+        p.k_affine             = v.k_affine;
+        p.xk_stride            = (int32_t)v.xk_stride;
+        p.yk_stride            = (int32_t)v.yk_stride;
         fresh->kernel_name     = hiptk_kernel_name(&p);
         if(!h->hostOnly())
             if(auto e = uploadTables(*fresh); e != HIPTENSOR_STATUS_SUCCESS)

@@ -79,6 +79,9 @@ namespace hipta
         p.x_vec   = v.x_vec;
         p.y_vec   = v.y_vec;
         p.cd_vec  = v.cd_vec;
+        p.k_affine  = v.k_affine;
+        p.xk_stride = (int32_t)v.xk_stride;
+        p.yk_stride = (int32_t)v.yk_stride;
         p.xp      = base + offs[0];
         p.xk      = base + offs[1];
         p.yq      = base + offs[2];

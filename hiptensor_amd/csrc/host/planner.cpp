@@ -339,6 +339,15 @@ namespace hipta
             return PlanStatus::UNSUPPORTED_SHAPE;
         }
 
+        if(v.kdims.size() <= 1)
+        {
+            v.k_affine  = 1;
+            v.xk_stride = v.kdims.empty() ? 0 : v.kdims[0].sx;
+            v.yk_stride = v.kdims.empty() ? 0 : v.kdims[0].sy;
+            if(v.xk_stride > 0x7FFFFFFFll || v.yk_stride > 0x7FFFFFFFll)
+                v.k_affine = 0;
+        }
+
         // ---- gather direction and vector width per operand ----
         const int maxv = class_max_vec(v.cls);
         const TensorIn& Xt = v.swapped ? B : A;

@@ -55,6 +55,9 @@ namespace hipta
         // offset tables (element units), padded as the kernel ABI requires
         std::vector<int32_t> xp, xk, yq, yk, cp, cq, dp, dq;
         int x_kfast = 1, y_kfast = 1, x_vec = 1, y_vec = 1, cd_vec = 1;
+        // the K modes fused into (at most) one: k offsets are k * stride
+        int     k_affine = 0;
+        int64_t xk_stride = 0, yk_stride = 0;
         int elem_bytes = 0;
         // bytes each tensor spans in memory (1 + sum (len-1)*stride elements)
         int64_t spanA = 0, spanB = 0, spanC = 0, spanD = 0;

@@ -74,6 +74,7 @@ namespace hipta
         p.y_kfast = v.y_kfast;
         p.x_vec   = v.x_vec;
         p.y_vec   = v.y_vec;
+        p.k_affine = v.k_affine;
         return hiptk_kernel_available(&p) != 0;
     }
 

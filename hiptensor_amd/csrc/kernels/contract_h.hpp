@@ -94,7 +94,14 @@ namespace hiptk
     };
 
     // Global -> register -> LDS staging of one operand tile.
-    template <typename Tr, bool KF, int V, int BR, int BK, int NT>
+    //
+    // KAFF: the reduction index maps to memory with one stride (all K modes fused into
+    // one), so k offsets are a multiply instead of a table lookup.
+    // Loads are never predicated: beyond K the k offset is 0 (the tables are zero padded;
+    // the affine form clamps), which is a valid element of the same row, and the loaded
+    // bits are masked to zero afterwards.  Keeping the loads unconditional lets all of a
+    // tile's loads be in flight together.
+    template <typename Tr, bool KF, int V, int BR, int BK, int NT, bool KAFF>
     struct Stager
     {
         typedef typename Tr::src_t src_t;
@@ -126,64 +133,76 @@ namespace hiptk
                 roff[0] = rtab[r0 + a * V];
         }
 
+        // k offsets of the tile that starts at k0 (table form; one tile ahead of its fetch)
         __device__ inline void load_koffs(const int32_t* ktab, int k0)
         {
-            if constexpr(KF)
-                koff[0] = ktab[k0 + a * V];
-            else
+            if constexpr(!KAFF)
             {
+                if constexpr(KF)
+                    koff[0] = ktab[k0 + a * V];
+                else
+                {
 #pragma unroll
-                for(int i = 0; i < N; i++)
-                    koff[i] = ktab[k0 + b + i * STEP];
+                    for(int i = 0; i < N; i++)
+                        koff[i] = ktab[k0 + b + i * STEP];
+                }
             }
         }
 
-        __device__ inline void fetch_one(const src_t* base, uint32_t off, bool ok, uint32_t (&d)[W])
+        __device__ inline void fetch_one(const src_t* p, uint32_t mask, uint32_t (&d)[W])
         {
-            const src_t* p = base + off;
             if constexpr(V == 8)
             {
-                u32x4_t v = {0u, 0u, 0u, 0u};
-                if(ok)
-                    v = *(const u32x4_t*)p;
-                d[0] = v[0];
-                d[1] = v[1];
-                d[2] = v[2];
-                d[3] = v[3];
+                const u32x4_t v = *(const u32x4_t*)p;
+                d[0]            = v[0] & mask;
+                d[1]            = v[1] & mask;
+                d[2]            = v[2] & mask;
+                d[3]            = v[3] & mask;
             }
             else if constexpr(V == 4)
             {
-                u32x2_t v = {0u, 0u};
-                if(ok)
-                    v = *(const u32x2_t*)p;
-                d[0] = v[0];
-                d[1] = v[1];
+                const u32x2_t v = *(const u32x2_t*)p;
+                d[0]            = v[0] & mask;
+                d[1]            = v[1] & mask;
             }
             else if constexpr(V == 2)
-                d[0] = ok ? *(const uint32_t*)p : 0u;
+                d[0] = *(const uint32_t*)p & mask;
             else
-                d[0] = ok ? (uint32_t)*p : 0u;
+                d[0] = (uint32_t)*p & mask;
         }
 
-        // Fetch the tile whose first k is k0 (koffs for it must be loaded already).
-        __device__ inline void fetch(const void* base, int k0, int K)
+        // Fetch the tile whose first k is k0.  TAIL: the tile may reach beyond K.
+        template <bool TAIL>
+        __device__ inline void fetch(const void* base, int k0, int K, int kstride)
         {
             const src_t* bp = (const src_t*)base;
             if constexpr(KF)
             {
-                const bool ok = (k0 + a * V) < K;
+                const int      k    = k0 + a * V;
+                const uint32_t mask = (!TAIL || k < K) ? 0xFFFFFFFFu : 0u;
+                uint32_t       ko;
+                if constexpr(KAFF)
+                    ko = (uint32_t)((TAIL && k >= K) ? 0 : k) * (uint32_t)kstride;
+                else
+                    ko = (uint32_t)koff[0];
 #pragma unroll
                 for(int i = 0; i < N; i++)
-                    fetch_one(bp, (uint32_t)roff[i] + (uint32_t)koff[0], ok, data[i]);
+                    fetch_one(bp + ((uint32_t)roff[i] + ko), mask, data[i]);
             }
             else
             {
 #pragma unroll
                 for(int i = 0; i < N; i++)
-                    fetch_one(bp,
-                              (uint32_t)roff[0] + (uint32_t)koff[i],
-                              (k0 + b + i * STEP) < K,
-                              data[i]);
+                {
+                    const int      k    = k0 + b + i * STEP;
+                    const uint32_t mask = (!TAIL || k < K) ? 0xFFFFFFFFu : 0u;
+                    uint32_t       ko;
+                    if constexpr(KAFF)
+                        ko = (uint32_t)((TAIL && k >= K) ? 0 : k) * (uint32_t)kstride;
+                    else
+                        ko = (uint32_t)koff[i];
+                    fetch_one(bp + ((uint32_t)roff[0] + ko), mask, data[i]);
+                }
             }
         }
 
@@ -192,8 +211,7 @@ namespace hiptk
 #pragma unroll
             for(int i = 0; i < N; i++)
             {
-                uint16_t* dst = KF ? lds + (b + i * STEP) * PITCH + a * V
-                                   : lds + (b + i * STEP) * PITCH + a * V;
+                uint16_t* dst = lds + (b + i * STEP) * PITCH + a * V;
                 if constexpr(V == 8)
                 {
                     u32x4_t v = {data[i][0], data[i][1], data[i][2], data[i][3]};
@@ -250,7 +268,8 @@ namespace hiptk
               bool XKF,
               bool YKF,
               int  XV,
-              int  YV>
+              int  YV,
+              bool KAFF>
     __global__ void __launch_bounds__(WP* WQ * 64) contract_h_kernel(const KArgs a)
     {
         constexpr int NT  = WP * WQ * 64;
@@ -280,8 +299,8 @@ namespace hiptk
         if(kt_end > kt_all)
             kt_end = kt_all;
 
-        Stager<Tr, XKF, XV, BP, BK, NT> sx;
-        Stager<Tr, YKF, YV, BQ, BK, NT> sy;
+        Stager<Tr, XKF, XV, BP, BK, NT, KAFF> sx;
+        Stager<Tr, YKF, YV, BQ, BK, NT, KAFF> sy;
         sx.init(a.xp, p0, tid);
         sy.init(a.yq, q0, tid);
 
@@ -297,12 +316,23 @@ namespace hiptk
         const int xbase = frag_base<XKF, LX::PITCH>(lane) + (XKF ? wp * WTP * LX::PITCH : wp * WTP);
         const int ybase = frag_base<YKF, LY::PITCH>(lane) + (YKF ? wq * WTQ * LY::PITCH : wq * WTQ);
 
+        // tiles below kt_full lie entirely inside K
+        const int kt_full = a.K / BK;
+
         if(kt_begin < kt_end)
         {
             sx.load_koffs(a.xk, kt_begin * BK);
             sy.load_koffs(a.yk, kt_begin * BK);
-            sx.fetch(a.X, kt_begin * BK, a.K);
-            sy.fetch(a.Y, kt_begin * BK, a.K);
+            if(kt_begin < kt_full)
+            {
+                sx.template fetch<false>(a.X, kt_begin * BK, a.K, a.xk_stride);
+                sy.template fetch<false>(a.Y, kt_begin * BK, a.K, a.yk_stride);
+            }
+            else
+            {
+                sx.template fetch<true>(a.X, kt_begin * BK, a.K, a.xk_stride);
+                sy.template fetch<true>(a.Y, kt_begin * BK, a.K, a.yk_stride);
+            }
             sx.load_koffs(a.xk, (kt_begin + 1) * BK);
             sy.load_koffs(a.yk, (kt_begin + 1) * BK);
         }
@@ -315,10 +345,17 @@ namespace hiptk
             sx.commit(lx);
             sy.commit(ly);
             __syncthreads();
-            if(kt + 1 < kt_end)
+            if(kt + 1 < kt_full)
             {
-                sx.fetch(a.X, (kt + 1) * BK, a.K);
-                sy.fetch(a.Y, (kt + 1) * BK, a.K);
+                sx.template fetch<false>(a.X, (kt + 1) * BK, a.K, a.xk_stride);
+                sy.template fetch<false>(a.Y, (kt + 1) * BK, a.K, a.yk_stride);
+                sx.load_koffs(a.xk, (kt + 2) * BK);
+                sy.load_koffs(a.yk, (kt + 2) * BK);
+            }
+            else if(kt + 1 < kt_end)
+            {
+                sx.template fetch<true>(a.X, (kt + 1) * BK, a.K, a.xk_stride);
+                sy.template fetch<true>(a.Y, (kt + 1) * BK, a.K, a.yk_stride);
                 sx.load_koffs(a.xk, (kt + 2) * BK);
                 sy.load_koffs(a.yk, (kt + 2) * BK);
             }
@@ -328,10 +365,10 @@ namespace hiptk
                 u32x4_t xf[TP], yf[TQ];
 #pragma unroll
                 for(int i = 0; i < TP; i++)
-                    xf[i] = frag_load<XKF, LX::PITCH>(lx, xbase, XKF ? i * 32 : i * 32, ks);
+                    xf[i] = frag_load<XKF, LX::PITCH>(lx, xbase, i * 32, ks);
 #pragma unroll
                 for(int j = 0; j < TQ; j++)
-                    yf[j] = frag_load<YKF, LY::PITCH>(ly, ybase, YKF ? j * 32 : j * 32, ks);
+                    yf[j] = frag_load<YKF, LY::PITCH>(ly, ybase, j * 32, ks);
 #pragma unroll
                 for(int i = 0; i < TP; i++)
 #pragma unroll
@@ -403,13 +440,14 @@ namespace hiptk
               bool XKF,
               bool YKF,
               int  XV,
-              int  YV>
+              int  YV,
+              bool KAFF>
     int launch_h(const KArgs& a, hipStream_t stream)
     {
         typedef TileLds<XKF, BP, BK> LX;
         typedef TileLds<YKF, BQ, BK> LY;
         constexpr int                LDS = 2 * (LX::ELEMS + LY::ELEMS) * 2;
-        auto kern = contract_h_kernel<Tr, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV>;
+        auto kern = contract_h_kernel<Tr, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF>;
         static const hipError_t attr = hipFuncSetAttribute(
             (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         if(attr != hipSuccess)
@@ -426,26 +464,27 @@ namespace hiptk
     }
 }
 
-// One registry line: class traits, tile id, tile shape, wave grid, layouts, vectors.
-#define HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV)                         \
+// One registry line: class traits, tile id, tile shape, wave grid, layouts, vectors,
+// affine-K flag.
+#define HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF)                   \
     {                                                                                       \
-        TR::CLS, ID, XKF, YKF, XV, YV, BP, BQ, BK, WP *WQ * 64,                             \
+        TR::CLS, ID, XKF, YKF, XV, YV, KAFF, BP, BQ, BK, WP *WQ * 64,                       \
             hiptk::lds_bytes_h<BP, BQ, BK, XKF, YKF>(),                                     \
-            #TR "_" #BP "x" #BQ "x" #BK "_x" #XKF #XV "_y" #YKF #YV,                        \
-            &hiptk::launch_h<hiptk::TR, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV>               \
+            #TR "_" #BP "x" #BQ "x" #BK "_x" #XKF #XV "_y" #YKF #YV "_kaff" #KAFF,          \
+            &hiptk::launch_h<hiptk::TR, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF>         \
     }
 
 // The four layout combinations of a tile whose operands are both gathered 8 wide.
-#define HIPTK_H_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ)               \
-    HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 8),  \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 8, 8), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 8), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, 8, 8)
+#define HIPTK_H_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ, KAFF)                   \
+    HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 8, KAFF),      \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 8, 8, KAFF), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 8, KAFF), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, 8, 8, KAFF)
 
 // Combinations in which at least one operand is a scalar gather (always staged k-fast).
-#define HIPTK_H_TILE_V1(TR, ID, BP, BQ, BK, WP, WQ)               \
-    HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 1, 1),  \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 1), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 1), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 1, 8), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 1, 8)
+#define HIPTK_H_TILE_V1(TR, ID, BP, BQ, BK, WP, WQ)                         \
+    HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 1, 1, false),     \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 1, false), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 1, false), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 1, 8, false), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 1, 8, false)

@@ -560,7 +560,7 @@ namespace hiptk
     {                                                                                          \
         hiptk::TR::CLS, ID, (XM != hiptk::GATHER_MN_VEC), (YM != hiptk::GATHER_MN_VEC),        \
             (XM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX),                                \
-            (YM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX), BP, BQ, BK, 256,               \
+            (YM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX), 0, BP, BQ, BK, 256,               \
             hiptk::lds_bytes_w<hiptk::TR, BP, BQ, BK>(), #TR "_" #BP "x" #BQ "x" #BK "_" #XM #YM, \
             &hiptk::launch_w<hiptk::TR, BP, BQ, BK, WP, WQ, XM, YM>                            \
     }

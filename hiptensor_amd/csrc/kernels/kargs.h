@@ -21,6 +21,7 @@ namespace hiptk
         int32_t split_k;
         int32_t bilinear;
         int32_t tiles_p, tiles_q;
+        int32_t xk_stride, yk_stride; // element stride of k when the K modes fused into one
         double  alpha[2], beta[2];
     };
 
@@ -31,6 +32,7 @@ namespace hiptk
     {
         int32_t     cls, tile_id;
         int32_t     x_kfast, y_kfast, x_vec, y_vec;
+        int32_t     k_affine; // 1: k offsets are k * stride, no table lookups
         int32_t     bp, bq, bk, threads, lds_bytes;
         const char* name;
         launch_fn   launch;
@@ -38,6 +40,8 @@ namespace hiptk
 
     // Each kernel translation unit contributes its table.
     const KernelEntry* entries_f16_vec(int* count);
+    const KernelEntry* entries_f16_aff(int* count);
+    const KernelEntry* entries_bf16_aff(int* count);
     const KernelEntry* entries_f16_gen(int* count);
     const KernelEntry* entries_bf16_vec(int* count);
     const KernelEntry* entries_bf16_gen(int* count);

@@ -17,7 +17,9 @@ namespace hiptk
             Registry()
             {
                 typedef const KernelEntry* (*src_fn)(int*);
-                const src_fn sources[] = {entries_f16_vec,
+                const src_fn sources[] = {entries_f16_aff,
+                                          entries_bf16_aff,
+                                          entries_f16_vec,
                                           entries_f16_gen,
                                           entries_bf16_vec,
                                           entries_bf16_gen,
@@ -144,15 +146,23 @@ namespace hiptk
             }
         }
 
+        // The affine-K variant is preferred when the problem allows it; the table variant
+        // serves every problem.
         const KernelEntry* find_entry(const hiptk_problem_t* p)
         {
+            const KernelEntry* table = nullptr;
             for(const KernelEntry& e : registry().all)
             {
                 if(e.cls == p->cls && e.tile_id == p->tile_id && e.x_kfast == (p->x_kfast != 0)
                    && e.y_kfast == (p->y_kfast != 0) && e.x_vec == p->x_vec && e.y_vec == p->y_vec)
-                    return &e;
+                {
+                    if(e.k_affine && p->k_affine)
+                        return &e;
+                    if(!e.k_affine && !table)
+                        table = &e;
+                }
             }
-            return nullptr;
+            return table;
         }
     }
 }
@@ -253,7 +263,9 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
     a.P  = (int32_t)prob->P;
     a.Q  = (int32_t)prob->Q;
     a.K  = (int32_t)prob->K;
-    a.bilinear = bil ? 1 : 0;
+    a.bilinear  = bil ? 1 : 0;
+    a.xk_stride = prob->xk_stride;
+    a.yk_stride = prob->yk_stride;
     a.tiles_p  = (int32_t)((prob->P + e->bp - 1) / e->bp);
     a.tiles_q  = (int32_t)((prob->Q + e->bq - 1) / e->bq);
     const int ktiles = (int)((prob->K + e->bk - 1) / e->bk);

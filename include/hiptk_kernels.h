@@ -79,6 +79,10 @@ typedef struct hiptk_problem
     int32_t x_vec;   /* contiguous elements per X vector (1 = scalar gather)   */
     int32_t y_vec;
     int32_t cd_vec;  /* contiguous elements along q shared by C and D          */
+    int32_t k_affine; /* 1: xk[k] == k * xk_stride and yk[k] == k * yk_stride for all k < K;
+                         a kernel that multiplies instead of reading xk / yk is used when
+                         one is instantiated (the tables must still be valid)          */
+    int32_t xk_stride, yk_stride;
     int32_t reserved;
 } hiptk_problem_t;
 
