@@ -34,6 +34,16 @@ namespace hiptk
     typedef short    short4_t __attribute__((ext_vector_type(4)));
     typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
     typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+    typedef float    f32x4_t __attribute__((ext_vector_type(4)));
+
+    // Workgroup barrier that orders LDS traffic only: global loads that are still in
+    // flight (the next tile's gather) are not waited for.
+    __device__ inline void lds_barrier()
+    {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    }
 
     __device__ inline uint16_t f32_to_bf16_rne(float f)
     {
@@ -319,73 +329,117 @@ namespace hiptk
         // tiles below kt_full lie entirely inside K
         const int kt_full = a.K / BK;
 
+        auto fetch_tile = [&](int t) {
+            if(t < kt_full)
+            {
+                sx.template fetch<false>(a.X, t * BK, a.K, a.xk_stride);
+                sy.template fetch<false>(a.Y, t * BK, a.K, a.yk_stride);
+            }
+            else
+            {
+                sx.template fetch<true>(a.X, t * BK, a.K, a.xk_stride);
+                sy.template fetch<true>(a.Y, t * BK, a.K, a.yk_stride);
+            }
+        };
+        auto compute = [&](const uint16_t* lx, const uint16_t* ly, int ks) {
+            u32x4_t xf[TP], yf[TQ];
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+                xf[i] = frag_load<XKF, LX::PITCH>(lx, xbase, i * 32, ks);
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+                yf[j] = frag_load<YKF, LY::PITCH>(ly, ybase, j * 32, ks);
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+                    acc[i][j] = Tr::mfma(xf[i], yf[j], acc[i][j]);
+        };
+        constexpr int KS = BK / 16;
+
+        // Software pipeline over K tiles.  While tile t is being multiplied out of one LDS
+        // buffer, tile t+1 moves from registers into the other buffer and tile t+2 is
+        // gathered from global memory into those registers; one barrier per tile.
         if(kt_begin < kt_end)
         {
             sx.load_koffs(a.xk, kt_begin * BK);
             sy.load_koffs(a.yk, kt_begin * BK);
-            if(kt_begin < kt_full)
-            {
-                sx.template fetch<false>(a.X, kt_begin * BK, a.K, a.xk_stride);
-                sy.template fetch<false>(a.Y, kt_begin * BK, a.K, a.yk_stride);
-            }
-            else
-            {
-                sx.template fetch<true>(a.X, kt_begin * BK, a.K, a.xk_stride);
-                sy.template fetch<true>(a.Y, kt_begin * BK, a.K, a.yk_stride);
-            }
+            fetch_tile(kt_begin);
             sx.load_koffs(a.xk, (kt_begin + 1) * BK);
             sy.load_koffs(a.yk, (kt_begin + 1) * BK);
+            sx.commit(lds);
+            sy.commit(lds + LX::ELEMS);
+            if(kt_begin + 1 < kt_end)
+            {
+                fetch_tile(kt_begin + 1);
+                sx.load_koffs(a.xk, (kt_begin + 2) * BK);
+                sy.load_koffs(a.yk, (kt_begin + 2) * BK);
+            }
+            lds_barrier();
         }
 
         int buf = 0;
-        for(int kt = kt_begin; kt < kt_end; kt++)
+        int kt  = kt_begin;
+        // steady state: tile kt+2 exists and is a full tile
+        const int steady_end = (kt_end < kt_full ? kt_end : kt_full) - 2;
+        for(; kt < steady_end; kt++)
         {
-            uint16_t* lx = lds + buf * STAGE;
-            uint16_t* ly = lx + LX::ELEMS;
-            sx.commit(lx);
-            sy.commit(ly);
-            __syncthreads();
-            if(kt + 1 < kt_full)
+            const uint16_t* lx = lds + buf * STAGE;
+            const uint16_t* ly = lx + LX::ELEMS;
+            uint16_t*       nx = lds + (buf ^ 1) * STAGE;
+            uint16_t*       ny = nx + LX::ELEMS;
+#pragma unroll
+            for(int ks = 0; ks < KS; ks++)
             {
-                sx.template fetch<false>(a.X, (kt + 1) * BK, a.K, a.xk_stride);
-                sy.template fetch<false>(a.Y, (kt + 1) * BK, a.K, a.yk_stride);
-                sx.load_koffs(a.xk, (kt + 2) * BK);
-                sy.load_koffs(a.yk, (kt + 2) * BK);
+                compute(lx, ly, ks);
+                if(ks == 0)
+                    sx.commit(nx);
+                if(ks == (KS > 1 ? 1 : 0))
+                    sy.commit(ny);
+                if(ks == (KS > 2 ? 2 : KS - 1))
+                {
+                    sx.template fetch<false>(a.X, (kt + 2) * BK, a.K, a.xk_stride);
+                    sy.template fetch<false>(a.Y, (kt + 2) * BK, a.K, a.yk_stride);
+                    sx.load_koffs(a.xk, (kt + 3) * BK);
+                    sy.load_koffs(a.yk, (kt + 3) * BK);
+                }
             }
-            else if(kt + 1 < kt_end)
+            lds_barrier();
+            buf ^= 1;
+        }
+        // drain: at most the last three tiles (and every tile of a short K)
+        for(; kt < kt_end; kt++)
+        {
+            const uint16_t* lx = lds + buf * STAGE;
+            const uint16_t* ly = lx + LX::ELEMS;
+            uint16_t*       nx = lds + (buf ^ 1) * STAGE;
+            uint16_t*       ny = nx + LX::ELEMS;
+#pragma unroll
+            for(int ks = 0; ks < KS; ks++)
+                compute(lx, ly, ks);
+            if(kt + 1 < kt_end)
             {
-                sx.template fetch<true>(a.X, (kt + 1) * BK, a.K, a.xk_stride);
-                sy.template fetch<true>(a.Y, (kt + 1) * BK, a.K, a.yk_stride);
-                sx.load_koffs(a.xk, (kt + 2) * BK);
-                sy.load_koffs(a.yk, (kt + 2) * BK);
+                sx.commit(nx);
+                sy.commit(ny);
+                if(kt + 2 < kt_end)
+                {
+                    fetch_tile(kt + 2);
+                    sx.load_koffs(a.xk, (kt + 3) * BK);
+                    sy.load_koffs(a.yk, (kt + 3) * BK);
+                }
             }
-#pragma unroll
-            for(int ks = 0; ks < BK / 16; ks++)
-            {
-                u32x4_t xf[TP], yf[TQ];
-#pragma unroll
-                for(int i = 0; i < TP; i++)
-                    xf[i] = frag_load<XKF, LX::PITCH>(lx, xbase, i * 32, ks);
-#pragma unroll
-                for(int j = 0; j < TQ; j++)
-                    yf[j] = frag_load<YKF, LY::PITCH>(ly, ybase, j * 32, ks);
-#pragma unroll
-                for(int i = 0; i < TP; i++)
-#pragma unroll
-                    for(int j = 0; j < TQ; j++)
-                        acc[i][j] = Tr::mfma(xf[i], yf[j], acc[i][j]);
-            }
+            lds_barrier();
             buf ^= 1;
         }
 
         // ---- epilogue ----
-        const int   pw = p0 + wp * WTP + 4 * (lane >> 5);
-        const int   qw = q0 + wq * WTQ + (lane & 31);
         const float alpha = (float)a.alpha[0];
         const float beta  = (float)a.beta[0];
         if(a.split_k > 1)
         {
-            float* ws = (float*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
+            const int pw = p0 + wp * WTP + 4 * (lane >> 5);
+            const int qw = q0 + wq * WTQ + (lane & 31);
+            float*    ws = (float*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
 #pragma unroll
             for(int j = 0; j < TQ; j++)
             {
@@ -406,28 +460,95 @@ namespace hiptk
         }
         uint16_t*       Dp = (uint16_t*)a.D;
         const uint16_t* Cp = (const uint16_t*)a.C;
-#pragma unroll
-        for(int j = 0; j < TQ; j++)
+        if(a.cd_vec == 8)
         {
-            const int q = qw + j * 32;
-            if(q >= a.Q)
-                continue;
-            const uint32_t dqo = (uint32_t)a.dq[q];
-            const uint32_t cqo = a.bilinear ? (uint32_t)a.cq[q] : 0u;
+            // C and D are contiguous along q in runs of 8: route each 32-row slab of the
+            // wave's accumulators through LDS (the operand buffers are free now) so that a
+            // lane ends up with 8 consecutive q of one row and moves them as one 16-byte
+            // access; 16 lanes cover 256 contiguous bytes of a row.
+            constexpr int EP = WTQ + 4; // floats per staged row
+            static_assert(32 * EP * 4 * WP * WQ <= 2 * STAGE * 2, "epilogue staging must fit the operand buffers");
+            float*    st = (float*)lds + wave * (32 * EP);
+            const int pw = p0 + wp * WTP;
+            const int qw = q0 + wq * WTQ;
 #pragma unroll
             for(int i = 0; i < TP; i++)
+            {
 #pragma unroll
-                for(int r = 0; r < 16; r++)
+                for(int j = 0; j < TQ; j++)
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                        st[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
+                lds_barrier();
+#pragma unroll
+                for(int v = 0; v < (32 * WTQ / 8) / 64; v++)
                 {
-                    const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
-                    if(p < a.P)
+                    constexpr int VPR  = WTQ / 8; // 8-element vectors per staged row
+                    const int     slot = v * 64 + lane;
+                    const int     row  = slot / VPR;
+                    const int     qv   = (slot % VPR) * 8;
+                    const int p = pw + i * 32 + row;
+                    const int q = qw + qv;
+                    if(p < a.P && q < a.Q)
                     {
-                        float v = alpha * acc[i][j][r];
+                        const float*   src = st + row * EP + qv;
+                        const f32x4_t  lo  = *(const f32x4_t*)src;
+                        const f32x4_t  hi  = *(const f32x4_t*)(src + 4);
+                        float          v8[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        const uint32_t doff  = (uint32_t)a.dp[p] + (uint32_t)a.dq[q];
                         if(a.bilinear)
-                            v += beta * Tr::to_f32(Cp[(uint32_t)a.cp[p] + cqo]);
-                        Dp[(uint32_t)a.dp[p] + dqo] = Tr::from_f32(v);
+                        {
+                            const u32x4_t c4 = *(const u32x4_t*)(Cp + ((uint32_t)a.cp[p] + (uint32_t)a.cq[q]));
+#pragma unroll
+                            for(int e = 0; e < 8; e++)
+                            {
+                                const uint16_t cb = (uint16_t)(c4[e >> 1] >> ((e & 1) * 16));
+                                v8[e]             = alpha * v8[e] + beta * Tr::to_f32(cb);
+                            }
+                        }
+                        else
+                        {
+#pragma unroll
+                            for(int e = 0; e < 8; e++)
+                                v8[e] = alpha * v8[e];
+                        }
+                        u32x4_t o;
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                            o[e] = (uint32_t)Tr::from_f32(v8[2 * e]) | ((uint32_t)Tr::from_f32(v8[2 * e + 1]) << 16);
+                        *(u32x4_t*)(Dp + doff) = o;
                     }
                 }
+                lds_barrier();
+            }
+            return;
+        }
+        {
+            const int pw = p0 + wp * WTP + 4 * (lane >> 5);
+            const int qw = q0 + wq * WTQ + (lane & 31);
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+            {
+                const int q = qw + j * 32;
+                if(q >= a.Q)
+                    continue;
+                const uint32_t dqo = (uint32_t)a.dq[q];
+                const uint32_t cqo = a.bilinear ? (uint32_t)a.cq[q] : 0u;
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                    {
+                        const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
+                        if(p < a.P)
+                        {
+                            float v = alpha * acc[i][j][r];
+                            if(a.bilinear)
+                                v += beta * Tr::to_f32(Cp[(uint32_t)a.cp[p] + cqo]);
+                            Dp[(uint32_t)a.dp[p] + dqo] = Tr::from_f32(v);
+                        }
+                    }
+            }
         }
     }
 

@@ -22,6 +22,7 @@ namespace hiptk
         int32_t bilinear;
         int32_t tiles_p, tiles_q;
         int32_t xk_stride, yk_stride; // element stride of k when the K modes fused into one
+        int32_t cd_vec; // contiguous elements along q shared by C and D
         double  alpha[2], beta[2];
     };
 

@@ -266,6 +266,7 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
     a.bilinear  = bil ? 1 : 0;
     a.xk_stride = prob->xk_stride;
     a.yk_stride = prob->yk_stride;
+    a.cd_vec    = prob->cd_vec;
     a.tiles_p  = (int32_t)((prob->P + e->bp - 1) / e->bp);
     a.tiles_q  = (int32_t)((prob->Q + e->bq - 1) / e->bq);
     const int ktiles = (int)((prob->K + e->bk - 1) / e->bk);
