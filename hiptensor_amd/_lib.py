@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libhiptensor_amd.so")
+# HIPTENSOR_AMD_LIBRARY points at another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("HIPTENSOR_AMD_LIBRARY") or os.path.join(_HERE, "lib", "libhiptensor_amd.so")
 
 
 class LibraryMissing(ImportError):
