@@ -226,11 +226,14 @@ def config4():
                   "cfg4_c32_bilinear_1024x1024x512")
 
 
-def config5(scale=1):
+def config5(scale=1, extents=None):
     """Rank-6 f16 bilinear with permuted A / B storage and a padded leading dimension on C / D.
-    `scale` > 1 divides the three largest extents (for parity runs the oracle can finish)."""
+    `scale` > 1 divides the three largest extents (for parity runs the oracle can finish);
+    `extents` replaces all nine (m0, m1, m2, n0, n1, n2, k0, k1, k2) for small fixtures."""
     m0, m1, m2, n0, n1, n2, k0, k1, k2 = 0, 1, 2, 10, 11, 12, 20, 21, 22
     ext = {m0: 32, m1: 7, m2: 24 // scale, n0: 24, n1: 9, n2: 32 // scale, k0: 17, k1: 8, k2: 30 // scale}
+    if extents is not None:
+        ext = dict(zip((m0, m1, m2, n0, n1, n2, k0, k1, k2), extents))
     mA, mB, mD = [m0, m1, m2, k0, k1, k2], [n0, n1, n2, k0, k1, k2], [m0, m1, m2, n0, n1, n2]
     sA = storage_order_strides(mA, ext, [k1, m0, k0, m2, m1, k2])
     sB = storage_order_strides(mB, ext, [n2, k0, n0, k2, k1, n1])
