@@ -61,7 +61,7 @@ def measure(handle, w, steps, warmup):
     return out
 
 
-def cpu_baseline(w, budget_macs=1.2e9):
+def cpu_baseline(w, budget_macs=8.6e9):
     """Times the CPU contraction on a slab of the workload: the outputs whose slowest M mode
     lies in a leading sub-range, full N and K.  Uses the compiled reference when oracle/_ref
     is present, else the oracle port."""

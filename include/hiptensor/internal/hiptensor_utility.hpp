@@ -12,7 +12,9 @@
 #include <string>
 #include <vector>
 
+#include <hip/hip_bfloat16.h>
 #include <hip/hip_complex.h>
+#include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
 #include "../hiptensor_types.hpp"
@@ -54,6 +56,12 @@ namespace hiptensor_detail
                                   __LINE__);                                              \
     } while(0)
 #endif
+
+// Half-precision values print as float (the stream has no inserter of its own for them).
+inline std::ostream& operator<<(std::ostream& os, const _Float16& v)
+{
+    return os << static_cast<float>(v);
+}
 
 // "re + imi" / "re-imi" formatting of complex scalars.
 inline std::ostream& operator<<(std::ostream& os, const hipFloatComplex& z)
@@ -110,6 +118,18 @@ inline bool operator==(const hiptensorTensorDescriptor_t& a, const hiptensorTens
 inline bool operator!=(const hiptensorTensorDescriptor_t& a, const hiptensorTensorDescriptor_t& b)
 {
     return !(a == b);
+}
+
+// "dim N, lengths {..}, strides {..}" (reference: hiptensor_utility.hpp:140-157).
+inline std::ostream& operator<<(std::ostream& os, const hiptensorTensorDescriptor_t& desc)
+{
+    os << "dim " << desc.mLengths.size() << ", lengths {";
+    for(size_t i = 0; i < desc.mLengths.size(); ++i)
+        os << desc.mLengths[i] << (i + 1 < desc.mLengths.size() ? ", " : "");
+    os << "}, strides {";
+    for(size_t i = 0; i < desc.mStrides.size(); ++i)
+        os << desc.mStrides[i] << (i + 1 < desc.mStrides.size() ? ", " : "");
+    return os << "}";
 }
 
 #endif // HIPTENSOR_UTILITY_INTERNAL_HPP

@@ -1,0 +1,52 @@
+"""The C++ API as a drop-in: programs written against <hiptensor/hiptensor.hpp> build against
+this repository's headers and link against libhiptensor_amd.so."""
+import os
+import subprocess
+
+import pytest
+
+from hiptensor_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "cpp", "bin", "dropin_contraction")
+REF_SAMPLES = "/root/reference/samples"
+HIPCC = "/opt/rocm/bin/hipcc"
+
+
+def build_dropin():
+    os.makedirs(os.path.dirname(BIN), exist_ok=True)
+    subprocess.run([HIPCC, "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"),
+                    os.path.join(ROOT, "tests", "cpp", "dropin_contraction.cpp"), "-o", BIN,
+                    "-L" + os.path.dirname(_lib.LIB_PATH), "-lhiptensor_amd",
+                    "-Wl,-rpath,$ORIGIN/../../../hiptensor_amd/lib"], check=True, capture_output=True)
+
+
+def test_dropin_program_builds_and_links():
+    build_dropin()
+    assert os.path.exists(BIN)
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_SAMPLES), reason="reference tree not mounted")
+@pytest.mark.parametrize("sample", [
+    "simple_bilinear_contraction_f32_f32_f32_f32_compute_f32",
+    "simple_bilinear_contraction_f16_f16_f16_f16_compute_f16",
+    "simple_scale_contraction_cf32_cf32_cf32_compute_cf32",
+    "simple_scale_contraction_bf16_bf16_bf16_compute_bf16",
+])
+def test_reference_samples_compile_unchanged(sample, tmp_path):
+    """The reference's own sample programs, compiled where they lie, against these headers and
+    this library (they are not run: they refuse every architecture but gfx908 .. gfx942)."""
+    src = os.path.join(REF_SAMPLES, "01_contraction", sample + ".cpp")
+    out = tmp_path / sample
+    subprocess.run([HIPCC, "-std=c++17", "-O0", "-I" + os.path.join(ROOT, "include"), "-I" + REF_SAMPLES, src,
+                    "-o", str(out), "-L" + os.path.dirname(_lib.LIB_PATH), "-lhiptensor_amd"],
+                   check=True, capture_output=True)
+    assert out.exists()
+
+
+@pytest.mark.gpu
+def test_dropin_program_runs():
+    assert os.path.exists(BIN), "tests/cpp/bin/dropin_contraction is not built (build() makes it)"
+    r = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0 and "dropin_contraction: ok" in r.stdout
