@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <sstream>
@@ -704,8 +705,12 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         size_t pick = 0;
         if(find->mSelectionAlgorithm == HIPTENSOR_ALGO_DEFAULT_PATIENT && !h->hostOnly())
         {
+            // HIPTENSOR_AMD_PATIENT_TOP widens (or narrows) the measured set
+            size_t      top = 4;
+            if(const char* e = std::getenv("HIPTENSOR_AMD_PATIENT_TOP"))
+                top = (size_t)std::max(1, std::atoi(e));
             std::string trace;
-            pick = hipta::time_choices(*h, v, ranked, 4, trace);
+            pick = hipta::time_choices(*h, v, ranked, top, trace);
             if(!trace.empty())
                 log.heuristics(fn, trace.c_str());
         }

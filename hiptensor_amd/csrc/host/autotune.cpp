@@ -105,7 +105,7 @@ namespace hipta
         }
         size_t best   = 0;
         float  bestMs = 1e30f;
-        char   line[160];
+        char   line[200];
         for(size_t i = 0; i < n; i++)
         {
             p.tile_id = ranked[i].sol->tile_id;

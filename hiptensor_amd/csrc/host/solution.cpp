@@ -108,37 +108,68 @@ namespace hipta
         }
     }
 
+    namespace
+    {
+        // Measured on MI355X with this library's kernels, as fractions of the class's
+        // nominal MFMA peak per CU: `alone` is what one workgroup of the tile sustains when
+        // it has a CU to itself (latency bound), `full` what a CU sustains with as many of
+        // them resident as fit.  (The f64 figures are against the published 128 flop/clk/CU;
+        // a loop of nothing but v_mfma_f64_16x16x4_f64 sustains 0.46 of that on this part,
+        // so 0.45 is the ceiling there.)
+        struct TileRate
+        {
+            double alone, full;
+        };
+
+        TileRate tile_rate(int cls, int area)
+        {
+            switch(cls)
+            {
+            case HIPTK_F16:
+            case HIPTK_BF16:
+            case HIPTK_F32_AS_F16:
+            case HIPTK_F32_AS_BF16:
+                return area >= 65536 ? TileRate{0.33, 0.33} : area >= 16384 ? TileRate{0.18, 0.29} : TileRate{0.07, 0.20};
+            case HIPTK_F64:
+            case HIPTK_C64: return area >= 16384 ? TileRate{0.385, 0.42} : TileRate{0.20, 0.45};
+            default: return area >= 16384 ? TileRate{0.45, 0.50} : TileRate{0.27, 0.52};
+            }
+        }
+    }
+
     double estimate_us(const Solution& s, const GemmView& v, int split, const DeviceModel& dev)
     {
         const double tiles  = std::ceil((double)v.P / s.bp) * std::ceil((double)v.Q / s.bq);
         const double ktiles = std::ceil((double)v.K / s.bk);
         const double kper   = std::ceil(ktiles / split) * s.bk;
-        // Workgroups that fit on one CU at a time (LDS bound; big tiles also fill the
-        // register file on their own).
+        // workgroups that fit on one CU at a time (LDS bound; the 256 x 256 tile also fills
+        // the register file on its own)
         int resident = std::max(1, std::min(4, dev.lds_per_cu / std::max(1, s.lds_bytes)));
         if(s.bp * s.bq >= 256 * 256)
             resident = 1;
-        const double slots = (double)dev.cus * resident;
-        const double waves = std::ceil(tiles * split / slots);
-        // Fraction of the CU's MFMA peak a full set of resident workgroups of this tile
-        // sustains: larger tiles re-use each LDS fragment in more MFMAs.
-        const double area = (double)s.bp * s.bq;
-        double       eff  = area >= 65536 ? 0.75 : area >= 16384 ? 0.55 : area >= 4096 ? 0.30 : 0.15;
+        const double wgs     = tiles * split;
+        const double per_cu  = std::ceil(wgs / dev.cus); // workgroups the busiest CU runs
+        const double sharing = std::min<double>(resident, per_cu);
+        TileRate     r       = tile_rate(v.cls, s.bp * s.bq);
         if(v.x_vec == 1 || v.y_vec == 1)
-            eff *= 0.35; // scalar gathers are issue bound
-        const double flops_wg = class_flops_per_mac(v.cls) * area * kper;
-        const double rate_wg  = class_flops_per_clk_cu(v.cls) * eff / resident; // flop / clk
-        double       us       = waves * flops_wg / rate_wg / (dev.clock_ghz * 1e3);
+        {
+            r.alone *= 0.35; // scalar gathers are issue bound
+            r.full *= 0.35;
+        }
+        const double frac     = std::min(sharing * r.alone, r.full);
+        const double flops_wg = class_flops_per_mac(v.cls) * (double)s.bp * s.bq * kper;
+        const double cu_rate  = class_flops_per_clk_cu(v.cls) * dev.clock_ghz * 1e3; // flop / us
+        double       us       = per_cu * flops_wg / (frac * cu_rate);
         // memory floor: every operand once (+ C and D)
         const double bytes = ((double)v.P * v.K + (double)v.Q * v.K + (double)v.P * v.Q * (v.bilinear ? 2 : 1))
                              * v.elem_bytes;
-        us = std::max(us, bytes / (dev.hbm_gbs * 1e3));
-        // fixed cost per workgroup (prologue, epilogue) and launch
-        us += 1.0 + waves * 1.5;
+        us = std::max(us, bytes / (dev.hbm_gbs * 1e3 * 0.6));
+        // launch, and prologue + epilogue of every round of workgroups on a CU
+        us += 3.0 + 1.5 * std::ceil(per_cu / sharing);
         if(split > 1)
         {
             const double ws = (double)split * v.P * v.Q * class_acc_bytes(v.cls);
-            us += 2.0 * ws / (dev.hbm_gbs * 1e3 * 0.5) + 3.0; // write + read partials, second launch
+            us += 2.0 * ws / (dev.hbm_gbs * 1e3 * 0.4) + 3.0; // partials out and back, second launch
         }
         return us;
     }

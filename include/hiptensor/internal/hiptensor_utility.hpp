@@ -58,10 +58,12 @@ namespace hiptensor_detail
 #endif
 
 // Half-precision values print as float (the stream has no inserter of its own for them).
+#ifdef __FLT16_MANT_DIG__
 inline std::ostream& operator<<(std::ostream& os, const _Float16& v)
 {
     return os << static_cast<float>(v);
 }
+#endif
 
 // "re + imi" / "re-imi" formatting of complex scalars.
 inline std::ostream& operator<<(std::ostream& os, const hipFloatComplex& z)
