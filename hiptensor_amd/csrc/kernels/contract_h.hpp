@@ -240,6 +240,14 @@ namespace hiptk
         }
     };
 
+    // Orders one wave's own LDS writes before its later LDS reads (and the reverse): enough
+    // when the data never leaves the wave, since a wave's LDS operations execute in order.
+    __device__ inline void wave_lds_fence()
+    {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront", "local");
+        __builtin_amdgcn_wave_barrier();
+    }
+
     // MFMA operand fetch from LDS for the 32-row block starting at row r0, k-substep ks.
     template <bool KF, int PITCH>
     __device__ inline int frag_base(int lane)
@@ -479,7 +487,7 @@ namespace hiptk
 #pragma unroll
                     for(int r = 0; r < 16; r++)
                         st[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
-                lds_barrier();
+                wave_lds_fence();
 #pragma unroll
                 for(int v = 0; v < (32 * WTQ / 8) / 64; v++)
                 {
@@ -519,7 +527,7 @@ namespace hiptk
                         *(u32x4_t*)(Dp + doff) = o;
                     }
                 }
-                lds_barrier();
+                wave_lds_fence();
             }
             return;
         }
