@@ -132,7 +132,7 @@ namespace hipta
                 return area >= 65536 ? TileRate{0.33, 0.33} : area >= 16384 ? TileRate{0.18, 0.29} : TileRate{0.07, 0.20};
             case HIPTK_F64:
             case HIPTK_C64: return area >= 16384 ? TileRate{0.385, 0.42} : TileRate{0.20, 0.45};
-            default: return area >= 16384 ? TileRate{0.45, 0.50} : TileRate{0.24, 0.52};
+            default: return area >= 16384 ? TileRate{0.45, 0.50} : TileRate{0.24, 0.60};
             }
         }
     }
@@ -169,7 +169,7 @@ namespace hipta
         if(split > 1)
         {
             const double ws = (double)split * v.P * v.Q * class_acc_bytes(v.cls);
-            us += 2.0 * ws / (dev.hbm_gbs * 1e3 * 0.4) + 3.0; // partials out and back, second launch
+            us += 2.0 * ws / (dev.hbm_gbs * 1e3 * 0.6) + 3.0; // partials out and back, second launch
         }
         return us;
     }
