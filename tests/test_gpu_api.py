@@ -1,0 +1,137 @@
+"""API behaviour that needs a device: measured selection, workspace errors, streams,
+the performance-trace log line, plan reuse and concurrent execution."""
+import ctypes as C
+import re
+import threading
+
+import numpy as np
+import pytest
+
+import cases
+import gpu_util
+from hiptensor_amd import api
+from hiptensor_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+
+def test_patient_selection_matches_oracle(gpu_handle, oracle_mod):
+    """HIPTENSOR_ALGO_DEFAULT_PATIENT times candidates on scratch tensors (sized by span, so
+    the padded layout is safe) and the plan it returns computes the right thing."""
+    for w in (wl.config5(extents=(32, 3, 4, 8, 3, 32, 5, 8, 6)), wl.config1()):
+        inp = wl.host_inputs(w)
+        exp = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
+        got, info = gpu_util.run_gpu(gpu_handle, w, inp, algo=api.HIPTENSOR_ALGO_DEFAULT_PATIENT,
+                                     pref=api.HIPTENSOR_WORKSPACE_MAX, return_info=True)
+        cases.assert_parity(w, cases.logical_view(w, got), cases.logical_view(w, exp), "patient " + info["kernel_name"])
+    w = wl.config1()
+    got = gpu_util.run_gpu(gpu_handle, w, algo=api.HIPTENSOR_ALGO_ACTOR_CRITIC)
+    exp = oracle_mod.contract(w, *[wl.host_inputs(w)[k] for k in ("A", "B", "C")])
+    cases.assert_parity(w, got, exp, "actor-critic")
+
+
+def test_split_k_and_workspace_contract(gpu_handle, oracle_mod):
+    import torch
+
+    w = wl.config1()  # small output: the recommended plan splits K and needs workspace
+    inp = wl.host_inputs(w)
+    exp = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
+    c = wl.Contraction(gpu_handle, w, pref=api.HIPTENSOR_WORKSPACE_RECOMMENDED)
+    assert c.info["split_k"] > 1 and c.workspace_bytes >= c.info["workspace_bytes"] > 0
+    A, B, Cd = (gpu_util.to_device(inp[k]) for k in ("A", "B", "C"))
+    D = gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"]))
+    ws = torch.empty(c.workspace_bytes, dtype=torch.uint8, device="cuda")
+    # too little workspace, or none: refused before anything is launched
+    st = c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(), ws.data_ptr(), workspace_bytes=c.info["workspace_bytes"] - 1)
+    assert st == api.HIPTENSOR_STATUS_INSUFFICIENT_WORKSPACE
+    st = c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(), None, workspace_bytes=0)
+    assert st == api.HIPTENSOR_STATUS_INSUFFICIENT_WORKSPACE
+    torch.cuda.synchronize()
+    assert np.all(np.isnan(D.cpu().numpy().view(np.float32)))
+    assert c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(), ws.data_ptr()) == 0
+    torch.cuda.synchronize()
+    cases.assert_parity(w, D.cpu().numpy().view(np.float32), exp, "split-K")
+    c.close()
+    # a plan made with no workspace runs single-pass and gives the same answer
+    got, info = gpu_util.run_gpu(gpu_handle, w, inp, pref=api.HIPTENSOR_WORKSPACE_MIN, return_info=True)
+    assert info["split_k"] == 1 and info["workspace_bytes"] == 0
+    cases.assert_parity(w, got, exp, "no workspace")
+    # bilinear needs C and beta
+    c = wl.Contraction(gpu_handle, w, pref=api.HIPTENSOR_WORKSPACE_MIN)
+    st = api.hiptensorContraction(gpu_handle, c.plan, c.alpha, A.data_ptr(), B.data_ptr(), c.beta, None, D.data_ptr(), None, 0, None)
+    assert st == api.HIPTENSOR_STATUS_INVALID_VALUE
+    c.close()
+
+
+def test_runs_on_the_callers_stream(gpu_handle, oracle_mod):
+    """Work is enqueued on the given stream and not synchronised: a long fill queued first on
+    that stream must be ordered before it (also for the complex path, which in the reference
+    runs its pack / unpack kernels on the null stream)."""
+    import torch
+
+    w = wl._rank4("c32", cases.COMPUTE["c32"], (16, 8), (16, 8), (16, 8), 1.0 + 0.5j, 0.25 - 0.75j, "stream_c32")
+    inp = wl.host_inputs(w)
+    exp = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
+    s = torch.cuda.Stream()
+    c = wl.Contraction(gpu_handle, w)
+    ws = torch.empty(max(c.workspace_bytes, 16), dtype=torch.uint8, device="cuda")
+    B, Cd = gpu_util.to_device(inp["B"]), gpu_util.to_device(inp["C"])
+    D = gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"]))
+    Ahost = torch.from_numpy(inp["A"].view(np.uint8).copy()).pin_memory()
+    A = torch.zeros_like(Ahost, device="cuda")
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        big = torch.empty(1 << 28, dtype=torch.uint8, device="cuda")
+        for _ in range(8):
+            big.fill_(1)  # keeps the stream busy
+        A.copy_(Ahost, non_blocking=True)  # A only becomes valid behind the fills, on stream s
+        st = c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(),
+                   ws.data_ptr() if c.workspace_bytes else None, s.cuda_stream)
+    assert st == 0
+    s.synchronize()
+    cases.assert_parity(w, D.cpu().numpy().view(np.complex64), exp, "stream")
+    c.close()
+
+
+def test_perf_trace_line(gpu_handle, tmp_path):
+    """With PERF_TRACE on, every contraction logs its time, TFlops and GB/s in the
+    reference's format (hiptensor_contraction.cpp:799-807)."""
+    log = tmp_path / "perf.log"
+    assert api.hiptensorLoggerOpenFile(str(log)) == 0
+    assert api.hiptensorLoggerSetMask(api.HIPTENSOR_LOG_LEVEL_PERF_TRACE) == 0
+    try:
+        gpu_util.run_gpu(gpu_handle, cases.rank1_case(0, "f32", 1.0, None))
+    finally:
+        api.hiptensorLoggerSetMask(0)
+        api.hiptensorLoggerOpenFile("")
+    text = log.read_text()
+    assert re.search(r"\[hipTensor\]\[Performance\]\[hiptensorContraction\] KernelId: \d+ KernelName: \S+, \d+\.\d+ ms, \d+\.\d+ TFlops, \d+\.\d+ GB/s", text)
+    assert "[hiptensorInitContractionPlan] Algo: -1, KernelId:" in text
+
+
+def test_concurrent_execution_of_one_plan(gpu_handle, oracle_mod):
+    """The plan is immutable: threads may execute it at once on their own streams."""
+    import torch
+
+    w = wl._rank4("f16", cases.COMPUTE["f16"], (16, 8), (16, 8), (16, 8), 1.0, 1.0, "threads_f16")
+    inp = wl.host_inputs(w)
+    exp = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
+    c = wl.Contraction(gpu_handle, w, pref=api.HIPTENSOR_WORKSPACE_MIN)
+    A, B, Cd = (gpu_util.to_device(inp[k]) for k in ("A", "B", "C"))
+    outs = [gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"])) for _ in range(4)]
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    torch.cuda.synchronize()
+    status = [None] * 4
+
+    def work(i):
+        for _ in range(20):
+            status[i] = c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), outs[i].data_ptr(), None, streams[i].cuda_stream)
+
+    ts = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    [t.start() for t in ts]
+    [t.join() for t in ts]
+    torch.cuda.synchronize()
+    assert status == [0, 0, 0, 0]
+    for o in outs:
+        cases.assert_parity(w, o.cpu().numpy().view(np.float16), exp, "threads")
+    c.close()
