@@ -25,6 +25,13 @@ PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "f32": 157.3, "c32": 157.3, "f64":
 FLOP_PER_CLK_CU = {"f16": 4096, "bf16": 4096, "f32": 256, "c32": 256, "f64": 128, "c64": 128}
 HBM_PEAK_GBS = 8000.0
 
+# Bytes per launch crossing the L2 <-> memory boundary, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of this script (profiles/contract_h_kernel_f16_4096cubed_scale.md gives the commands, the
+# raw readings and the copy-kernel scale factors).  Keyed by (workload, kernel); null otherwise.
+MEASURED_TRAFFIC_BYTES = {
+    ("cfg2_f16_scale_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue"): (2.0 * 98533.9 + 1.0 * 32768.0) * 1024,
+}
+
 
 def measure(handle, w, steps, warmup):
     """Returns dict(ms_per_step wall, kernel_ms from HIP events, info)."""
@@ -112,6 +119,9 @@ def main():
     ap.add_argument("--workload", default="cfg2_f16_scale")
     ap.add_argument("--all", action="store_true", help="also time every other configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run 3 plain device copies of 256 MiB (a kernel of known traffic, to scale "
+                         "the profiler's FETCH_SIZE / WRITE_SIZE counters by)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus must be 1 (the path would shard by output "
@@ -147,7 +157,8 @@ def main():
         "config": {"workload": w["name"], "M": M, "N": N, "K": K, "op": "bilinear" if w["beta"] is not None else "scale",
                    "kernel": r["info"]["kernel_name"], "split_k": r["info"]["split_k"]},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak,
-                     "traffic": None, "kernel_ms": r["kernel_ms"],
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((w["name"], r["info"]["kernel_name"])),
+                     "kernel_ms": r["kernel_ms"],
                      "peak_from_device_clock": cus * clock_ghz * FLOP_PER_CLK_CU[w["dtype"]] / 1e3,
                      "hbm_GBs_algorithmic": wl.algorithmic_bytes(w) / (r["kernel_ms"] * 1e-3) / 1e9},
         "device": {"name": prop.name, "cus": cus, "clock_ghz": clock_ghz},
@@ -164,6 +175,13 @@ def main():
                             "hbm_GBs_algorithmic": wl.algorithmic_bytes(cw) / (rr["kernel_ms"] * 1e-3) / 1e9,
                             "kernel": rr["info"]["kernel_name"], "split_k": rr["info"]["split_k"], "dtype": cw["dtype"]}
         out["others"] = others
+    if a.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["copy_calibration"] = {"bytes_read": 1 << 28, "bytes_written": 1 << 28, "launches": 3}
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w)
     api.hiptensorDestroy(handle)
