@@ -129,7 +129,11 @@ namespace hipta
             case HIPTK_BF16:
             case HIPTK_F32_AS_F16:
             case HIPTK_F32_AS_BF16:
-                return area >= 65536 ? TileRate{0.33, 0.33} : area >= 16384 ? TileRate{0.18, 0.29} : TileRate{0.07, 0.20};
+                return area >= 65536   ? TileRate{0.35, 0.35}
+                       : area >= 49152 ? TileRate{0.34, 0.34}
+                       : area >= 32768 ? TileRate{0.30, 0.30}
+                       : area >= 16384 ? TileRate{0.18, 0.29}
+                                       : TileRate{0.07, 0.20};
             case HIPTK_F64:
             case HIPTK_C64: return area >= 16384 ? TileRate{0.385, 0.42} : TileRate{0.20, 0.45};
             default: return area >= 16384 ? TileRate{0.45, 0.50} : TileRate{0.24, 0.60};
@@ -145,7 +149,7 @@ namespace hipta
         // workgroups that fit on one CU at a time (LDS bound; the 256 x 256 tile also fills
         // the register file on its own)
         int resident = std::max(1, std::min(4, dev.lds_per_cu / std::max(1, s.lds_bytes)));
-        if(s.bp * s.bq >= 256 * 256)
+        if(s.threads >= 512)
             resident = 1;
         const double wgs     = tiles * split;
         const double per_cu  = std::ceil(wgs / dev.cus); // workgroups the busiest CU runs
