@@ -61,7 +61,8 @@ namespace hiptk
     struct TraitsF16
     {
         static constexpr int CLS = HIPTK_F16;
-        typedef uint16_t     src_t;
+        typedef uint16_t     src_t; // storage of A and B
+        typedef uint16_t     out_t; // storage of C and D
         static __device__ inline f32x16_t mfma(u32x4_t x, u32x4_t y, f32x16_t acc)
         {
             return __builtin_amdgcn_mfma_f32_32x32x16_f16(
@@ -76,12 +77,19 @@ namespace hiptk
             return (float)__builtin_bit_cast(_Float16, h);
         }
         static __device__ inline uint16_t stage(uint16_t v) { return v; }
+        static __device__ inline out_t    out_from_f32(float f) { return from_f32(f); }
+        static __device__ inline float    out_to_f32(out_t v) { return to_f32(v); }
+        static __device__ inline float    axpby(float al, float x, float be, float c, bool bil)
+        {
+            return bil ? al * x + be * c : al * x;
+        }
     };
 
     struct TraitsBF16
     {
         static constexpr int CLS = HIPTK_BF16;
         typedef uint16_t     src_t;
+        typedef uint16_t     out_t;
         static __device__ inline f32x16_t mfma(u32x4_t x, u32x4_t y, f32x16_t acc)
         {
             return __builtin_amdgcn_mfma_f32_32x32x16_bf16(
@@ -93,6 +101,45 @@ namespace hiptk
             return __uint_as_float((uint32_t)h << 16);
         }
         static __device__ inline uint16_t stage(uint16_t v) { return v; }
+        static __device__ inline out_t    out_from_f32(float f) { return from_f32(f); }
+        static __device__ inline float    out_to_f32(out_t v) { return to_f32(v); }
+        static __device__ inline float    axpby(float al, float x, float be, float c, bool bil)
+        {
+            return bil ? al * x + be * c : al * x;
+        }
+    };
+
+    // f32 storage, operands rounded to f16 / bf16 when they are staged into LDS (the
+    // reference's "compute type" for these rows), f32 accumulate, f32 results.
+    struct TraitsF32AsF16 : TraitsF16
+    {
+        static constexpr int CLS = HIPTK_F32_AS_F16;
+        typedef float        src_t;
+        typedef float        out_t;
+        static __device__ inline uint16_t stage(float v) { return TraitsF16::from_f32(v); }
+        static __device__ inline out_t    out_from_f32(float f) { return f; }
+        static __device__ inline float    out_to_f32(out_t v) { return v; }
+        // separately rounded products, as the CPU path computes alpha * x + beta * c
+        static __device__ inline float axpby(float al, float x, float be, float c, bool bil)
+        {
+            const float y = __fmul_rn(al, x);
+            return bil ? __fadd_rn(y, __fmul_rn(be, c)) : y;
+        }
+    };
+
+    struct TraitsF32AsBF16 : TraitsBF16
+    {
+        static constexpr int CLS = HIPTK_F32_AS_BF16;
+        typedef float        src_t;
+        typedef float        out_t;
+        static __device__ inline uint16_t stage(float v) { return f32_to_bf16_rne(v); }
+        static __device__ inline out_t    out_from_f32(float f) { return f; }
+        static __device__ inline float    out_to_f32(out_t v) { return v; }
+        static __device__ inline float    axpby(float al, float x, float be, float c, bool bil)
+        {
+            const float y = __fmul_rn(al, x);
+            return bil ? __fadd_rn(y, __fmul_rn(be, c)) : y;
+        }
     };
 
     // LDS tile geometry of one operand (16-bit elements).
@@ -122,7 +169,8 @@ namespace hiptk
         static constexpr int PITCH = TileLds<KF, BR, BK>::PITCH;
         static_assert(NT % PER == 0, "thread count must cover whole vector rows");
         static_assert((BR * BK / V) % NT == 0 && N >= 1, "tile must split evenly over threads");
-        static_assert(sizeof(src_t) == 2, "16-bit storage");
+        static constexpr bool SRC32 = sizeof(src_t) == 4; // f32 storage, rounded when staged
+        static_assert(!SRC32 || V == 4 || V == 1, "f32 sources are gathered 16 bytes or one element at a time");
 
         uint32_t data[N][W];
         int32_t  roff[KF ? N : 1]; // row-table offsets (loop invariant)
@@ -161,7 +209,15 @@ namespace hiptk
 
         __device__ inline void fetch_one(const src_t* p, uint32_t mask, uint32_t (&d)[W])
         {
-            if constexpr(V == 8)
+            if constexpr(SRC32 && V == 4)
+            {
+                const f32x4_t v = *(const f32x4_t*)p;
+                d[0] = ((uint32_t)Tr::stage(v[0]) | ((uint32_t)Tr::stage(v[1]) << 16)) & mask;
+                d[1] = ((uint32_t)Tr::stage(v[2]) | ((uint32_t)Tr::stage(v[3]) << 16)) & mask;
+            }
+            else if constexpr(SRC32)
+                d[0] = (uint32_t)Tr::stage(*p) & mask;
+            else if constexpr(V == 8)
             {
                 const u32x4_t v = *(const u32x4_t*)p;
                 d[0]            = v[0] & mask;
@@ -466,8 +522,10 @@ namespace hiptk
             }
             return;
         }
-        uint16_t*       Dp = (uint16_t*)a.D;
-        const uint16_t* Cp = (const uint16_t*)a.C;
+        typedef typename Tr::out_t out_t;
+        out_t*       Dp = (out_t*)a.D;
+        const out_t* Cp = (const out_t*)a.C;
+        if constexpr(sizeof(out_t) == 2)
         if(a.cd_vec == 8)
         {
             // C and D are contiguous along q in runs of 8: route each 32-row slab of the
@@ -550,10 +608,9 @@ namespace hiptk
                         const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
                         if(p < a.P)
                         {
-                            float v = alpha * acc[i][j][r];
-                            if(a.bilinear)
-                                v += beta * Tr::to_f32(Cp[(uint32_t)a.cp[p] + cqo]);
-                            Dp[(uint32_t)a.dp[p] + dqo] = Tr::from_f32(v);
+                            const float c = a.bilinear ? Tr::out_to_f32(Cp[(uint32_t)a.cp[p] + cqo]) : 0.f;
+                            Dp[(uint32_t)a.dp[p] + dqo]
+                                = Tr::out_from_f32(Tr::axpby(alpha, acc[i][j][r], beta, c, a.bilinear != 0));
                         }
                     }
             }
@@ -603,17 +660,19 @@ namespace hiptk
             &hiptk::launch_h<hiptk::TR, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF>         \
     }
 
-// The four layout combinations of a tile whose operands are both gathered 8 wide.
-#define HIPTK_H_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ, KAFF)                   \
-    HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 8, KAFF),      \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 8, 8, KAFF), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 8, KAFF), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, 8, 8, KAFF)
+// The four layout combinations of a tile whose operands are both gathered V wide.
+#define HIPTK_H_TILE_VV(TR, ID, BP, BQ, BK, WP, WQ, V, KAFF)                   \
+    HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, V, V, KAFF),         \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, V, V, KAFF),    \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, V, V, KAFF),    \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, V, V, KAFF)
+#define HIPTK_H_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ, KAFF) HIPTK_H_TILE_VV(TR, ID, BP, BQ, BK, WP, WQ, 8, KAFF)
 
 // Combinations in which at least one operand is a scalar gather (always staged k-fast).
-#define HIPTK_H_TILE_V1(TR, ID, BP, BQ, BK, WP, WQ)                         \
+#define HIPTK_H_TILE_V1V(TR, ID, BP, BQ, BK, WP, WQ, V)                     \
     HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 1, 1, false),     \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 1, false), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 1, false), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 1, 8, false), \
-        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 1, 8, false)
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, V, 1, false), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, V, 1, false), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 1, V, false), \
+        HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 1, V, false)
+#define HIPTK_H_TILE_V1(TR, ID, BP, BQ, BK, WP, WQ) HIPTK_H_TILE_V1V(TR, ID, BP, BQ, BK, WP, WQ, 8)

@@ -51,6 +51,8 @@ namespace hiptk
     const KernelEntry* entries_c32(int* count);
     const KernelEntry* entries_c64(int* count);
     const KernelEntry* entries_f64_as_f32(int* count);
+    const KernelEntry* entries_f32_as_f16(int* count);
+    const KernelEntry* entries_f32_as_bf16(int* count);
 
     // XCD-aware mapping of the linear workgroup id to an output tile.  Workgroups are
     // handed to the 8 XCDs round-robin, so ids that are congruent mod 8 share an L2.

@@ -27,7 +27,9 @@ namespace hiptk
                                           entries_f64,
                                           entries_c32,
                                           entries_c64,
-                                          entries_f64_as_f32};
+                                          entries_f64_as_f32,
+                                          entries_f32_as_f16,
+                                          entries_f32_as_bf16};
                 for(src_fn f : sources)
                 {
                     int                n = 0;
@@ -137,7 +139,9 @@ namespace hiptk
             {
             case HIPTK_F16: return launch_reduce<FinF16>(a, stream);
             case HIPTK_BF16: return launch_reduce<FinBF16>(a, stream);
-            case HIPTK_F32: return launch_reduce<FinWide<WTraitsF32>>(a, stream);
+            case HIPTK_F32:
+            case HIPTK_F32_AS_F16:
+            case HIPTK_F32_AS_BF16: return launch_reduce<FinWide<WTraitsF32>>(a, stream);
             case HIPTK_F64: return launch_reduce<FinWide<WTraitsF64>>(a, stream);
             case HIPTK_C32: return launch_reduce<FinWide<WTraitsC32>>(a, stream);
             case HIPTK_C64: return launch_reduce<FinWide<WTraitsC64>>(a, stream);

@@ -156,7 +156,7 @@ def scalar_ctype(compute, value):
     if compute == api.HIPTENSOR_COMPUTE_16F:
         return C.c_uint16(int(np.float16(value).view(np.uint16)))
     if compute == api.HIPTENSOR_COMPUTE_16BF:
-        return C.c_uint16(int(f32_to_bf16_bits(np.float32(value))))
+        return C.c_uint16(int(f32_to_bf16_bits(np.array([value], dtype=np.float32))[0]))
     raise ValueError(f"compute type {compute}")
 
 

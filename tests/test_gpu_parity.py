@@ -87,6 +87,21 @@ def test_tile_edges_and_k_tails(gpu_handle, oracle_mod, dtype):
         check(gpu_handle, oracle_mod, wl._rank4(dtype, cases.COMPUTE[dtype], m, n, k, a, b, f"edges_{dtype}_{m}_{n}_{k}"))
 
 
+@pytest.mark.parametrize("dtype,compute", [("f32", api.HIPTENSOR_COMPUTE_16F), ("f32", api.HIPTENSOR_COMPUTE_16BF),
+                                           ("f64", api.HIPTENSOR_COMPUTE_32F)])
+def test_mixed_compute_rows(gpu_handle, oracle_mod, dtype, compute):
+    """f32 data multiplied in f16 / bf16 (operands rounded when staged, f32 accumulate) and
+    f64 data multiplied in f32: the remaining type rows the reference registers
+    (library/src/contraction/contraction_solution_instances.cpp:82-160).  alpha / beta are
+    passed in the compute type, as the API specifies."""
+    for alpha, beta in ((1.5, 0.75), (0.5, None)):
+        for w in (cases.rank_case(3, dtype, alpha, beta), cases.rank_case(5, dtype, alpha, beta),
+                  wl._rank4(dtype, compute, (16, 6), (8, 10), (8, 9), alpha, beta, f"colmajor_{dtype}_{compute}"),
+                  cases.rank1_case(2, dtype, alpha, beta)):
+            w["compute"] = compute
+            check(gpu_handle, oracle_mod, w)
+
+
 def test_config5_layout_reduced(gpu_handle, oracle_mod):
     """The benchmark's rank-6 permuted / padded layout at reduced extents."""
     info = check(gpu_handle, oracle_mod, wl.config5(scale=2))
