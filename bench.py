@@ -163,6 +163,19 @@ def main():
                      "hbm_GBs_algorithmic": wl.algorithmic_bytes(w) / (r["kernel_ms"] * 1e-3) / 1e9},
         "device": {"name": prop.name, "cus": cus, "clock_ghz": clock_ghz},
     }
+    # what a loop of nothing but this type's MFMA instruction sustains on this device
+    import ctypes
+
+    from hiptensor_amd._lib import lib as _native
+    kcls = {"f16": 0, "bf16": 1, "f32": 2, "f64": 3, "c32": 4, "c64": 5}
+    ceil = {}
+    for label, rnd in (("constant_operands", 0), ("random_operands", 1)):
+        tf = ctypes.c_double(0)
+        if _native.hiptk_mfma_ceiling(kcls[w["dtype"]], rnd, ctypes.byref(tf)) == 0:
+            ceil[label] = tf.value
+    out["roofline"]["mfma_only_sustained_tflops"] = ceil
+    if ceil.get("random_operands"):
+        out["roofline"]["frac_of_sustained"] = tflops / ceil["random_operands"]
     if a.all:
         others = {}
         for name, cw in cfgs.items():
@@ -171,7 +184,10 @@ def main():
             steps = max(5, a.steps // 2)
             rr = measure(handle, cw, steps, a.warmup)
             tf = wl.flops(cw) / (rr["kernel_ms"] * 1e-3) / 1e12
+            tfc = ctypes.c_double(0)
+            sustained = tfc.value if _native.hiptk_mfma_ceiling(kcls[cw["dtype"]], 1, ctypes.byref(tfc)) == 0 else None
             others[name] = {"kernel_ms": rr["kernel_ms"], "tflops": tf, "frac_peak": tf / PEAK_TFLOPS[cw["dtype"]],
+                            "mfma_only_sustained_tflops": sustained,
                             "hbm_GBs_algorithmic": wl.algorithmic_bytes(cw) / (rr["kernel_ms"] * 1e-3) / 1e9,
                             "kernel": rr["info"]["kernel_name"], "split_k": rr["info"]["split_k"], "dtype": cw["dtype"]}
         out["others"] = others

@@ -344,7 +344,7 @@ namespace hiptk
               int  XV,
               int  YV,
               bool KAFF>
-    __global__ void __launch_bounds__(WP* WQ * 64) contract_h_kernel(const KArgs a)
+    __global__ void __launch_bounds__(WP* WQ * 64, 2) contract_h_kernel(const KArgs a)
     {
         constexpr int NT  = WP * WQ * 64;
         constexpr int WTP = BP / WP, WTQ = BQ / WQ;

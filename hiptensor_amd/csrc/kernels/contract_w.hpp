@@ -387,7 +387,7 @@ namespace hiptk
     };
 
     template <typename Tr, int BP, int BQ, int BK, int WP, int WQ>
-    __global__ void __launch_bounds__(WP* WQ * 64) contract_w_kernel(const KArgs a, int xmode, int ymode)
+    __global__ void __launch_bounds__(WP* WQ * 64, 2) contract_w_kernel(const KArgs a, int xmode, int ymode)
     {
         constexpr int NT   = WP * WQ * 64;
         constexpr int TILE = Tr::TILE;

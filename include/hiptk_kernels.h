@@ -114,6 +114,14 @@ int hiptk_contract(const hiptk_problem_t* prob,
                    void*                  stream,
                    int*                   hip_error);
 
+/* Calibration, no counterpart in the reference: the TFLOP/s a loop of nothing but the class's
+ * MFMA instruction sustains on the current device (one 4-wave workgroup per CU), with
+ * constant operands (random_operands = 0) or pseudo-random operands in [-1, 1) (1).  The
+ * clock the part holds under a full matrix-core load depends on the operand data, so the
+ * second figure is the practical ceiling for a contraction of random data.  Synchronous;
+ * allocates 4 KiB. */
+int hiptk_mfma_ceiling(int cls, int random_operands, double* tflops);
+
 #ifdef __cplusplus
 }
 #endif
