@@ -246,159 +246,138 @@ namespace hiptk
     };
 
     // ---- staging: global -> registers -> LDS tile[k][BR + PAD] ---------------------
+    //
+    // MODE (compile time) says which way an operand's contiguous vectors run.  Loads are
+    // never predicated: beyond K the k offset is 0 (the tables are zero padded), beyond
+    // the last row the row offset is that of a valid row, so every address is inside the
+    // tensor; values beyond K are replaced by zero after the load (TAIL tiles only).
+    // Unconditional loads let all of a tile's loads be in flight together.
 
-    template <typename Tr, int BR, int BK, int NT>
+    template <typename Tr, int MODE, int BR, int BK, int NT>
     struct WStager
     {
         typedef typename Tr::E E;
         typedef typename Tr::S S;
-        static constexpr int   V     = Tr::VMAX;
+        static constexpr int   V     = MODE == GATHER_SCALAR ? 1 : Tr::VMAX;
         static constexpr int   N     = BR * BK / NT; // elements per thread
+        static constexpr int   NV    = N / V; // vectors per thread
         static constexpr int   PAD   = (sizeof(S) >= 8 ? 2 : 4);
         static constexpr int   PITCH = BR + PAD;
         static constexpr int   ELEMS = BK * PITCH;
-        static_assert(BR * BK % NT == 0 && N % V == 0, "tile must split evenly over threads");
-        static_assert(NT % (BR / V) == 0 && NT % BK == 0 && NT % (BK / V) == 0, "thread mapping");
+        // threads along the fast direction of the mapping, and rows / k's covered per pass
+        static constexpr int PER  = MODE == GATHER_MN_VEC ? BR / V : (MODE == GATHER_K_VEC ? BK / V : BK);
+        static constexpr int STEP = NT / PER;
+        static_assert(BR * BK % NT == 0 && N % V == 0 && NV >= 1, "tile must split evenly over threads");
+        static_assert(NT % PER == 0, "thread mapping");
 
-        E       data[N];
-        int32_t off[N]; // varying-table offsets (k for MN vectors, rows otherwise)
-        int32_t fixed; // the other table's offset
-        int     mode, a, b;
-
-        __device__ inline void init(int mode_, const int32_t* rtab, int r0, int tid)
+        struct alignas(sizeof(E) * V) PackE
         {
-            mode = mode_;
-            if(mode == GATHER_MN_VEC)
-            {
-                constexpr int PER = BR / V;
-                a                 = tid % PER;
-                b                 = tid / PER;
-                fixed             = rtab[r0 + a * V];
-            }
-            else if(mode == GATHER_K_VEC)
-            {
-                constexpr int PER = BK / V, STEP = NT / PER;
-                a = tid % PER;
-                b = tid / PER;
-#pragma unroll
-                for(int i = 0; i < N / V; i++)
-                    off[i] = rtab[r0 + b + i * STEP];
-            }
+            E e[V];
+        };
+        struct alignas(sizeof(S) * V) PackS
+        {
+            S e[V];
+        };
+
+        PackE   data[NV];
+        int32_t roff[MODE == GATHER_MN_VEC ? 1 : NV]; // row-table offsets (loop invariant)
+        int32_t koff[MODE == GATHER_MN_VEC ? NV : 1]; // k-table offsets of the tile being fetched
+        int     a, b;
+
+        __device__ inline void init(const int32_t* rtab, int r0, int tid)
+        {
+            a = tid % PER;
+            b = tid / PER;
+            if constexpr(MODE == GATHER_MN_VEC)
+                roff[0] = rtab[r0 + a * V];
             else
             {
-                constexpr int STEP = NT / BK;
-                a                  = tid % BK;
-                b                  = tid / BK;
 #pragma unroll
-                for(int i = 0; i < N; i++)
-                    off[i] = rtab[r0 + b + i * STEP];
+                for(int i = 0; i < NV; i++)
+                    roff[i] = rtab[r0 + b + i * STEP];
             }
         }
 
         __device__ inline void load_koffs(const int32_t* ktab, int k0)
         {
-            if(mode == GATHER_MN_VEC)
+            if constexpr(MODE == GATHER_MN_VEC)
             {
-                constexpr int STEP = NT / (BR / V);
 #pragma unroll
-                for(int i = 0; i < N / V; i++)
-                    off[i] = ktab[k0 + b + i * STEP];
+                for(int i = 0; i < NV; i++)
+                    koff[i] = ktab[k0 + b + i * STEP];
             }
-            else if(mode == GATHER_K_VEC)
-                fixed = ktab[k0 + a * V];
             else
-                fixed = ktab[k0 + a];
+                koff[0] = ktab[k0 + a * V];
         }
 
-        template <int W>
-        static __device__ inline void vload(const E* p, bool ok, E* dst)
-        {
-            struct alignas(sizeof(E) * W) Pack
-            {
-                E e[W];
-            };
-            Pack v;
-#pragma unroll
-            for(int j = 0; j < W; j++)
-                v.e[j] = E{};
-            if(ok)
-                v = *(const Pack*)p;
-#pragma unroll
-            for(int j = 0; j < W; j++)
-                dst[j] = v.e[j];
-        }
-
+        template <bool TAIL>
         __device__ inline void fetch(const void* base, int k0, int K)
         {
             const E* bp = (const E*)base;
-            if(mode == GATHER_MN_VEC)
-            {
-                constexpr int STEP = NT / (BR / V);
 #pragma unroll
-                for(int i = 0; i < N / V; i++)
-                    vload<V>(bp + ((uint32_t)fixed + (uint32_t)off[i]),
-                             (k0 + b + i * STEP) < K,
-                             &data[i * V]);
-            }
-            else if(mode == GATHER_K_VEC)
+            for(int i = 0; i < NV; i++)
             {
-                const bool ok = (k0 + a * V) < K;
+                const int  k  = MODE == GATHER_MN_VEC ? k0 + b + i * STEP : k0 + a * V;
+                const bool ok = !TAIL || k < K;
+                const uint32_t off = MODE == GATHER_MN_VEC ? (uint32_t)roff[0] + (uint32_t)koff[i]
+                                                            : (uint32_t)roff[i] + (uint32_t)koff[0];
+                PackE v = *(const PackE*)(bp + off);
+                if(TAIL && !ok)
+                {
 #pragma unroll
-                for(int i = 0; i < N / V; i++)
-                    vload<V>(bp + ((uint32_t)off[i] + (uint32_t)fixed), ok, &data[i * V]);
-            }
-            else
-            {
-                const bool ok = (k0 + a) < K;
-#pragma unroll
-                for(int i = 0; i < N; i++)
-                    vload<1>(bp + ((uint32_t)off[i] + (uint32_t)fixed), ok, &data[i]);
+                    for(int j = 0; j < V; j++)
+                        v.e[j] = E{};
+                }
+                data[i] = v;
             }
         }
 
         __device__ inline void commit(S* lds)
         {
-            if(mode == GATHER_MN_VEC)
-            {
-                constexpr int STEP = NT / (BR / V);
 #pragma unroll
-                for(int i = 0; i < N / V; i++)
+            for(int i = 0; i < NV; i++)
+            {
+                if constexpr(MODE == GATHER_MN_VEC)
+                {
+                    PackS s;
 #pragma unroll
                     for(int j = 0; j < V; j++)
-                        lds[(b + i * STEP) * PITCH + a * V + j] = Tr::stage(data[i * V + j]);
-            }
-            else if(mode == GATHER_K_VEC)
-            {
-                constexpr int STEP = NT / (BK / V);
-#pragma unroll
-                for(int i = 0; i < N / V; i++)
+                        s.e[j] = Tr::stage(data[i].e[j]);
+                    *(PackS*)(lds + (b + i * STEP) * PITCH + a * V) = s;
+                }
+                else
+                {
 #pragma unroll
                     for(int j = 0; j < V; j++)
-                        lds[(a * V + j) * PITCH + b + i * STEP] = Tr::stage(data[i * V + j]);
-            }
-            else
-            {
-                constexpr int STEP = NT / BK;
-#pragma unroll
-                for(int i = 0; i < N; i++)
-                    lds[a * PITCH + b + i * STEP] = Tr::stage(data[i]);
+                        lds[(a * V + j) * PITCH + b + i * STEP] = Tr::stage(data[i].e[j]);
+                }
             }
         }
     };
 
-    template <typename Tr, int BP, int BQ, int BK, int WP, int WQ>
-    __global__ void __launch_bounds__(WP* WQ * 64, 2) contract_w_kernel(const KArgs a, int xmode, int ymode)
+    // Workgroup barrier that orders LDS traffic only: global loads that are still in
+    // flight (the next tile's gather) are not waited for.
+    __device__ inline void w_lds_barrier()
+    {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    }
+
+    template <typename Tr, int BP, int BQ, int BK, int WP, int WQ, int XM, int YM>
+    __global__ void __launch_bounds__(WP* WQ * 64, 2) contract_w_kernel(const KArgs a)
     {
         constexpr int NT   = WP * WQ * 64;
         constexpr int TILE = Tr::TILE;
         constexpr int WTP = BP / WP, WTQ = BQ / WQ;
         constexpr int TP = WTP / TILE, TQ = WTQ / TILE;
-        static_assert(WTP % TILE == 0 && WTQ % TILE == 0 && BK % Tr::KM == 0, "tile shape");
+        constexpr int KS = BK / Tr::KM;
+        static_assert(WTP % TILE == 0 && WTQ % TILE == 0 && BK % Tr::KM == 0 && KS >= 3, "tile shape");
         typedef typename Tr::S        S;
         typedef typename Tr::E        E;
         typedef typename Tr::O        O;
-        typedef WStager<Tr, BP, BK, NT> SX;
-        typedef WStager<Tr, BQ, BK, NT> SY;
+        typedef WStager<Tr, XM, BP, BK, NT> SX;
+        typedef WStager<Tr, YM, BQ, BK, NT> SY;
         constexpr int                 STAGE = SX::ELEMS + SY::ELEMS;
 
         extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
@@ -423,8 +402,8 @@ namespace hiptk
 
         SX sx;
         SY sy;
-        sx.init(xmode, a.xp, p0, tid);
-        sy.init(ymode, a.yq, q0, tid);
+        sx.init(a.xp, p0, tid);
+        sy.init(a.yq, q0, tid);
 
         typename Tr::Acc acc[TP][TQ];
 #pragma unroll
@@ -438,46 +417,109 @@ namespace hiptk
         const int xfo   = kslot * SX::PITCH + wp * WTP + row;
         const int yfo   = kslot * SY::PITCH + wq * WTQ + row;
 
+        // tiles below kt_full lie entirely inside K
+        const int kt_full = a.K / BK;
+
+        auto fetch_tile = [&](int t) {
+            if(t < kt_full)
+            {
+                sx.template fetch<false>(a.X, t * BK, a.K);
+                sy.template fetch<false>(a.Y, t * BK, a.K);
+            }
+            else
+            {
+                sx.template fetch<true>(a.X, t * BK, a.K);
+                sy.template fetch<true>(a.Y, t * BK, a.K);
+            }
+        };
+        auto compute = [&](const S* lx, const S* ly, int ks) {
+            typename Tr::XF xf[TP];
+            typename Tr::YF yf[TQ];
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+                xf[i] = Tr::prep_x(lx[xfo + ks * Tr::KM * SX::PITCH + i * TILE], lane);
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+                yf[j] = Tr::prep_y(ly[yfo + ks * Tr::KM * SY::PITCH + j * TILE], lane);
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+                    Tr::mma(xf[i], yf[j], acc[i][j]);
+        };
+
+        // Software pipeline over K tiles.  While tile t is being multiplied out of one LDS
+        // buffer, tile t+1 moves from registers into the other buffer and tile t+2 is
+        // gathered from global memory into those registers; one barrier per tile.
         if(kt_begin < kt_end)
         {
             sx.load_koffs(a.xk, kt_begin * BK);
             sy.load_koffs(a.yk, kt_begin * BK);
-            sx.fetch(a.X, kt_begin * BK, a.K);
-            sy.fetch(a.Y, kt_begin * BK, a.K);
+            fetch_tile(kt_begin);
+            sx.load_koffs(a.xk, (kt_begin + 1) * BK);
+            sy.load_koffs(a.yk, (kt_begin + 1) * BK);
+            sx.commit(lds);
+            sy.commit(lds + SX::ELEMS);
+            if(kt_begin + 1 < kt_end)
+            {
+                fetch_tile(kt_begin + 1);
+                sx.load_koffs(a.xk, (kt_begin + 2) * BK);
+                sy.load_koffs(a.yk, (kt_begin + 2) * BK);
+            }
+            w_lds_barrier();
         }
 
         int buf = 0;
-        for(int kt = kt_begin; kt < kt_end; kt++)
+        int kt  = kt_begin;
+        // steady state: tile kt+2 exists and is a full tile
+        const int steady_end = (kt_end < kt_full ? kt_end : kt_full) - 2;
+        for(; kt < steady_end; kt++)
         {
-            S* lx = lds + buf * STAGE;
-            S* ly = lx + SX::ELEMS;
-            sx.commit(lx);
-            sy.commit(ly);
-            __syncthreads();
+            const S* lx = lds + buf * STAGE;
+            const S* ly = lx + SX::ELEMS;
+            S*       nx = lds + (buf ^ 1) * STAGE;
+            S*       ny = nx + SX::ELEMS;
+#pragma unroll
+            for(int ks = 0; ks < KS; ks++)
+            {
+                compute(lx, ly, ks);
+                if(ks == 0)
+                    sx.commit(nx);
+                if(ks == 1)
+                    sy.commit(ny);
+                if(ks == 2)
+                {
+                    sx.template fetch<false>(a.X, (kt + 2) * BK, a.K);
+                    sy.template fetch<false>(a.Y, (kt + 2) * BK, a.K);
+                    sx.load_koffs(a.xk, (kt + 3) * BK);
+                    sy.load_koffs(a.yk, (kt + 3) * BK);
+                }
+            }
+            w_lds_barrier();
+            buf ^= 1;
+        }
+        // drain: at most the last three tiles (and every tile of a short K)
+        for(; kt < kt_end; kt++)
+        {
+            const S* lx = lds + buf * STAGE;
+            const S* ly = lx + SX::ELEMS;
+            S*       nx = lds + (buf ^ 1) * STAGE;
+            S*       ny = nx + SX::ELEMS;
+#pragma unroll
+            for(int ks = 0; ks < KS; ks++)
+                compute(lx, ly, ks);
             if(kt + 1 < kt_end)
             {
-                sx.load_koffs(a.xk, (kt + 1) * BK);
-                sy.load_koffs(a.yk, (kt + 1) * BK);
-                sx.fetch(a.X, (kt + 1) * BK, a.K);
-                sy.fetch(a.Y, (kt + 1) * BK, a.K);
+                sx.commit(nx);
+                sy.commit(ny);
+                if(kt + 2 < kt_end)
+                {
+                    fetch_tile(kt + 2);
+                    sx.load_koffs(a.xk, (kt + 3) * BK);
+                    sy.load_koffs(a.yk, (kt + 3) * BK);
+                }
             }
-#pragma unroll
-            for(int ks = 0; ks < BK / Tr::KM; ks++)
-            {
-                typename Tr::XF xf[TP];
-                typename Tr::YF yf[TQ];
-#pragma unroll
-                for(int i = 0; i < TP; i++)
-                    xf[i] = Tr::prep_x(lx[xfo + ks * Tr::KM * SX::PITCH + i * TILE], lane);
-#pragma unroll
-                for(int j = 0; j < TQ; j++)
-                    yf[j] = Tr::prep_y(ly[yfo + ks * Tr::KM * SY::PITCH + j * TILE], lane);
-#pragma unroll
-                for(int i = 0; i < TP; i++)
-#pragma unroll
-                    for(int j = 0; j < TQ; j++)
-                        Tr::mma(xf[i], yf[j], acc[i][j]);
-            }
+            w_lds_barrier();
             buf ^= 1;
         }
 
@@ -488,54 +530,61 @@ namespace hiptk
         {
             O* ws = (O*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
 #pragma unroll
-            for(int j = 0; j < TQ; j++)
-            {
-                const int q = qw + j * TILE;
-                if(q >= a.Q)
-                    continue;
-#pragma unroll
-                for(int i = 0; i < TP; i++)
-#pragma unroll
-                    for(int r = 0; r < Tr::NREG; r++)
-                    {
-                        const int p = pw + i * TILE + Tr::p_of(r, lane);
-                        if(p < a.P)
-                            ws[(size_t)p * a.Q + q] = Tr::get(acc[i][j], r);
-                    }
-            }
-            return;
-        }
-        E*         Dp  = (E*)a.D;
-        const E*   Cp  = (const E*)a.C;
-        const bool bil = a.bilinear != 0;
-#pragma unroll
-        for(int j = 0; j < TQ; j++)
-        {
-            const int q = qw + j * TILE;
-            if(q >= a.Q)
-                continue;
-            const uint32_t dqo = (uint32_t)a.dq[q];
-            const uint32_t cqo = bil ? (uint32_t)a.cq[q] : 0u;
-#pragma unroll
             for(int i = 0; i < TP; i++)
 #pragma unroll
                 for(int r = 0; r < Tr::NREG; r++)
                 {
                     const int p = pw + i * TILE + Tr::p_of(r, lane);
-                    if(p < a.P)
+                    if(p >= a.P)
+                        continue;
+                    O* wrow = ws + (size_t)p * a.Q;
+#pragma unroll
+                    for(int j = 0; j < TQ; j++)
                     {
-                        const E* cptr = bil ? Cp + ((uint32_t)a.cp[p] + cqo) : nullptr;
-                        Dp[(uint32_t)a.dp[p] + dqo]
-                            = Tr::finish(Tr::get(acc[i][j], r), a.alpha, a.beta, bil, cptr);
+                        const int q = qw + j * TILE;
+                        if(q < a.Q)
+                            wrow[q] = Tr::get(acc[i][j], r);
                     }
                 }
+            return;
         }
+        E*         Dp  = (E*)a.D;
+        const E*   Cp  = (const E*)a.C;
+        const bool bil = a.bilinear != 0;
+        uint32_t   dqo[TQ], cqo[TQ];
+#pragma unroll
+        for(int j = 0; j < TQ; j++)
+        {
+            // the q tables are padded with valid entries, so the lookup is safe beyond Q
+            dqo[j] = (uint32_t)a.dq[qw + j * TILE];
+            cqo[j] = bil ? (uint32_t)a.cq[qw + j * TILE] : 0u;
+        }
+#pragma unroll
+        for(int i = 0; i < TP; i++)
+#pragma unroll
+            for(int r = 0; r < Tr::NREG; r++)
+            {
+                const int p = pw + i * TILE + Tr::p_of(r, lane);
+                if(p >= a.P)
+                    continue;
+                const uint32_t dpo = (uint32_t)a.dp[p];
+                const uint32_t cpo = bil ? (uint32_t)a.cp[p] : 0u;
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+                {
+                    if(qw + j * TILE < a.Q)
+                    {
+                        const E* cptr = bil ? Cp + (cpo + cqo[j]) : nullptr;
+                        Dp[dpo + dqo[j]] = Tr::finish(Tr::get(acc[i][j], r), a.alpha, a.beta, bil, cptr);
+                    }
+                }
+            }
     }
 
     template <typename Tr, int BP, int BQ, int BK>
     constexpr int lds_bytes_w()
     {
-        return 2 * (WStager<Tr, BP, BK, 256>::ELEMS + WStager<Tr, BQ, BK, 256>::ELEMS)
+        return 2 * (WStager<Tr, 0, BP, BK, 256>::ELEMS + WStager<Tr, 0, BQ, BK, 256>::ELEMS)
                * (int)sizeof(typename Tr::S);
     }
 
@@ -544,13 +593,13 @@ namespace hiptk
     {
         static_assert(WP * WQ * 64 == 256, "wide kernels use 256 threads");
         constexpr int LDS  = lds_bytes_w<Tr, BP, BQ, BK>();
-        auto          kern = contract_w_kernel<Tr, BP, BQ, BK, WP, WQ>;
+        auto          kern = contract_w_kernel<Tr, BP, BQ, BK, WP, WQ, XM, YM>;
         static const hipError_t attr = hipFuncSetAttribute(
             (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         if(attr != hipSuccess)
             return (int)attr;
         dim3 grid(a.tiles_p * a.tiles_q, 1, a.split_k);
-        hipLaunchKernelGGL(kern, grid, dim3(256), LDS, stream, a, XM, YM);
+        hipLaunchKernelGGL(kern, grid, dim3(256), LDS, stream, a);
         return (int)hipGetLastError();
     }
 }
