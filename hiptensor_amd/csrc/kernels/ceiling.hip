@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <chrono>
+
 #include "hiptk_kernels.h"
 
 namespace
@@ -173,14 +175,22 @@ extern "C" int hiptk_mfma_ceiling(int cls, int random_operands, double* tflops)
         default: break;
         }
     };
-    launch(); // warm-up
+    launch(); // sets iters
     if(iters == 0)
     {
         (void)hipFree(sink);
         return HIPTK_ERR_ARG;
     }
     (void)hipDeviceSynchronize();
-    const int reps = 5;
+    // the clock governor takes tens of milliseconds of load to settle: run untimed for ~150 ms
+    const auto t0 = std::chrono::steady_clock::now();
+    while(std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() < 0.15)
+    {
+        for(int r = 0; r < 10; r++)
+            launch();
+        (void)hipDeviceSynchronize();
+    }
+    const int reps = 20;
     (void)hipEventRecord(e0, 0);
     for(int r = 0; r < reps; r++)
         launch();

@@ -4,7 +4,7 @@
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
-        HIPTK_W_TILE(WTraitsC32, 0, 128, 128, 8, 2, 2),
+        HIPTK_W_TILE(WTraitsC32, 0, 128, 128, 8, 2, 4),
         HIPTK_W_TILE(WTraitsC32, 1, 64, 64, 8, 2, 2),
     };
 

@@ -4,7 +4,7 @@
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
-        HIPTK_W_TILE(WTraitsF64AsF32, 0, 128, 128, 16, 2, 2),
+        HIPTK_W_TILE(WTraitsF64AsF32, 0, 128, 128, 16, 2, 4),
         HIPTK_W_TILE(WTraitsF64AsF32, 1, 64, 64, 16, 2, 2),
     };
 

@@ -24,6 +24,8 @@
 // lane-varying), so at a fixed register the 32 lanes of a half-wave write 32
 // consecutive q: the planner orients the problem so that q is D's contiguous index.
 #pragma once
+#include <type_traits>
+
 #include "kargs.h"
 
 namespace hiptk
@@ -343,8 +345,9 @@ namespace hiptk
               bool YKF,
               int  XV,
               int  YV,
-              bool KAFF>
-    __global__ void __launch_bounds__(WP* WQ * 64, 2) contract_h_kernel(const KArgs a)
+              bool KAFF,
+              bool PIPE>
+    __global__ void __launch_bounds__(WP* WQ * 64, ((BP / WP) * (BQ / WQ) > 128 * 64 ? 1 : 2)) contract_h_kernel(const KArgs a)
     {
         constexpr int NT  = WP * WQ * 64;
         constexpr int WTP = BP / WP, WTQ = BQ / WQ;
@@ -446,6 +449,102 @@ namespace hiptk
         int kt  = kt_begin;
         // steady state: tile kt+2 exists and is a full tile
         const int steady_end = (kt_end < kt_full ? kt_end : kt_full) - 2;
+        if constexpr(PIPE)
+        {
+            // Register-level pipeline for one wavefront per SIMD: the MFMA operands of
+            // k-substep s+1 are read from LDS while substep s is multiplied, across the tile
+            // boundary as well.  The tile's barrier sits between substeps KS-2 and KS-1: by
+            // then every wave has issued its last reads of the current buffer and finished
+            // writing the next one, so substep KS-1 overlaps the first operand reads of the
+            // next tile.  sched_group_barrier pins the interleaving of MFMA, LDS and global
+            // instructions that the compiler would otherwise bunch together.
+            static_assert(KS >= 4 && KS % 2 == 0, "pipelined loop needs an even number of k-substeps");
+            constexpr int RX = TP * (XKF ? 1 : 2), RY = TQ * (YKF ? 1 : 2); // LDS reads per substep
+            constexpr int NM = TP * TQ; // MFMAs per substep
+            u32x4_t       xf[2][TP], yf[2][TQ];
+            auto load_frags = [&](const uint16_t* lx, const uint16_t* ly, int ks, int slot) {
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+                    xf[slot][i] = frag_load<XKF, LX::PITCH>(lx, xbase, i * 32, ks);
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+                    yf[slot][j] = frag_load<YKF, LY::PITCH>(ly, ybase, j * 32, ks);
+            };
+            auto mma = [&](int slot) {
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+#pragma unroll
+                    for(int j = 0; j < TQ; j++)
+                        acc[i][j] = Tr::mfma(xf[slot][i], yf[slot][j], acc[i][j]);
+            };
+            // NM MFMAs with the substep's LDS reads spread over the first half of them and
+            // `extra` instructions of class `mask` (LDS writes or global loads) over the rest
+            auto interleave = [&](auto mask_c, auto extra_c) {
+                constexpr int mask  = decltype(mask_c)::value;
+                constexpr int extra = decltype(extra_c)::value;
+                constexpr int H     = NM / 2;
+                constexpr int RPM   = (RX + RY + H - 1) / H;
+                constexpr int EPM   = (extra + (NM - H) - 1) / (NM - H);
+#pragma unroll
+                for(int m = 0; m < H; m++)
+                {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
+                }
+#pragma unroll
+                for(int m = H; m < NM; m++)
+                {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if constexpr(extra > 0)
+                        __builtin_amdgcn_sched_group_barrier(mask, EPM, 0);
+                }
+            };
+            typedef std::integral_constant<int, 0x200> DsWrite;
+            typedef std::integral_constant<int, 0x020> VmemRead;
+            if(kt < steady_end)
+                load_frags(lds, lds + LX::ELEMS, 0, 0);
+            for(; kt < steady_end; kt++)
+            {
+                const uint16_t* lx = lds + buf * STAGE;
+                const uint16_t* ly = lx + LX::ELEMS;
+                uint16_t*       nx = lds + (buf ^ 1) * STAGE;
+                uint16_t*       ny = nx + LX::ELEMS;
+#pragma unroll
+                for(int ks = 0; ks < KS; ks++)
+                {
+                    if(ks == KS - 1)
+                    {
+                        lds_barrier();
+                        load_frags(nx, ny, 0, (ks + 1) & 1);
+                    }
+                    else
+                        load_frags(lx, ly, ks + 1, (ks + 1) & 1);
+                    mma(ks & 1);
+                    if(ks == 0)
+                    {
+                        sx.commit(nx);
+                        interleave(DsWrite{}, std::integral_constant<int, decltype(sx)::N>{});
+                    }
+                    else if(ks == 1)
+                    {
+                        sy.commit(ny);
+                        interleave(DsWrite{}, std::integral_constant<int, decltype(sy)::N>{});
+                    }
+                    else if(ks == 2)
+                    {
+                        sx.template fetch<false>(a.X, (kt + 2) * BK, a.K, a.xk_stride);
+                        sy.template fetch<false>(a.Y, (kt + 2) * BK, a.K, a.yk_stride);
+                        sx.load_koffs(a.xk, (kt + 3) * BK);
+                        sy.load_koffs(a.yk, (kt + 3) * BK);
+                        interleave(VmemRead{}, std::integral_constant<int, decltype(sx)::N + decltype(sy)::N>{});
+                    }
+                    else
+                        interleave(DsWrite{}, std::integral_constant<int, 0>{});
+                }
+                buf ^= 1;
+            }
+        }
+        else
         for(; kt < steady_end; kt++)
         {
             const uint16_t* lx = lds + buf * STAGE;
@@ -456,15 +555,18 @@ namespace hiptk
             for(int ks = 0; ks < KS; ks++)
             {
                 compute(lx, ly, ks);
+                // registers of an operand are refilled right after they are stored, so a
+                // gather has a whole tile's worth of MFMA time to arrive
                 if(ks == 0)
-                    sx.commit(nx);
-                if(ks == (KS > 1 ? 1 : 0))
-                    sy.commit(ny);
-                if(ks == (KS > 2 ? 2 : KS - 1))
                 {
+                    sx.commit(nx);
                     sx.template fetch<false>(a.X, (kt + 2) * BK, a.K, a.xk_stride);
-                    sy.template fetch<false>(a.Y, (kt + 2) * BK, a.K, a.yk_stride);
                     sx.load_koffs(a.xk, (kt + 3) * BK);
+                }
+                if(ks == (KS > 1 ? 1 : 0))
+                {
+                    sy.commit(ny);
+                    sy.template fetch<false>(a.Y, (kt + 2) * BK, a.K, a.yk_stride);
                     sy.load_koffs(a.yk, (kt + 3) * BK);
                 }
             }
@@ -627,13 +729,14 @@ namespace hiptk
               bool YKF,
               int  XV,
               int  YV,
-              bool KAFF>
+              bool KAFF,
+              bool PIPE>
     int launch_h(const KArgs& a, hipStream_t stream)
     {
         typedef TileLds<XKF, BP, BK> LX;
         typedef TileLds<YKF, BQ, BK> LY;
         constexpr int                LDS = 2 * (LX::ELEMS + LY::ELEMS) * 2;
-        auto kern = contract_h_kernel<Tr, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF>;
+        auto kern = contract_h_kernel<Tr, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF, PIPE>;
         static const hipError_t attr = hipFuncSetAttribute(
             (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
         if(attr != hipSuccess)
@@ -657,7 +760,16 @@ namespace hiptk
         TR::CLS, ID, XKF, YKF, XV, YV, KAFF, BP, BQ, BK, WP *WQ * 64,                       \
             hiptk::lds_bytes_h<BP, BQ, BK, XKF, YKF>(),                                     \
             #TR "_" #BP "x" #BQ "x" #BK "_x" #XKF #XV "_y" #YKF #YV "_kaff" #KAFF,          \
-            &hiptk::launch_h<hiptk::TR, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF>         \
+            &hiptk::launch_h<hiptk::TR, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF, false>  \
+    }
+
+// The same with the register-level pipeline (one wavefront per SIMD, accumulators in AGPRs).
+#define HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF)                  \
+    {                                                                                       \
+        TR::CLS, ID, XKF, YKF, XV, YV, KAFF, BP, BQ, BK, WP *WQ * 64,                       \
+            hiptk::lds_bytes_h<BP, BQ, BK, XKF, YKF>(),                                     \
+            #TR "_" #BP "x" #BQ "x" #BK "_x" #XKF #XV "_y" #YKF #YV "_kaff" #KAFF "_pipe",  \
+            &hiptk::launch_h<hiptk::TR, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF, true>   \
     }
 
 // The four layout combinations of a tile whose operands are both gathered V wide.

@@ -483,15 +483,18 @@ namespace hiptk
             for(int ks = 0; ks < KS; ks++)
             {
                 compute(lx, ly, ks);
+                // registers of an operand are refilled right after they are stored, so a
+                // gather has a whole tile's worth of MFMA time to arrive
                 if(ks == 0)
-                    sx.commit(nx);
-                if(ks == 1)
-                    sy.commit(ny);
-                if(ks == 2)
                 {
+                    sx.commit(nx);
                     sx.template fetch<false>(a.X, (kt + 2) * BK, a.K);
-                    sy.template fetch<false>(a.Y, (kt + 2) * BK, a.K);
                     sx.load_koffs(a.xk, (kt + 3) * BK);
+                }
+                if(ks == 1)
+                {
+                    sy.commit(ny);
+                    sy.template fetch<false>(a.Y, (kt + 2) * BK, a.K);
                     sy.load_koffs(a.yk, (kt + 3) * BK);
                 }
             }
@@ -591,7 +594,6 @@ namespace hiptk
     template <typename Tr, int BP, int BQ, int BK, int WP, int WQ, int XM, int YM>
     int launch_w(const KArgs& a, hipStream_t stream)
     {
-        static_assert(WP * WQ * 64 == 256, "wide kernels use 256 threads");
         constexpr int LDS  = lds_bytes_w<Tr, BP, BQ, BK>();
         auto          kern = contract_w_kernel<Tr, BP, BQ, BK, WP, WQ, XM, YM>;
         static const hipError_t attr = hipFuncSetAttribute(
@@ -599,7 +601,7 @@ namespace hiptk
         if(attr != hipSuccess)
             return (int)attr;
         dim3 grid(a.tiles_p * a.tiles_q, 1, a.split_k);
-        hipLaunchKernelGGL(kern, grid, dim3(256), LDS, stream, a);
+        hipLaunchKernelGGL(kern, grid, dim3(WP * WQ * 64), LDS, stream, a);
         return (int)hipGetLastError();
     }
 }
@@ -609,7 +611,7 @@ namespace hiptk
     {                                                                                          \
         hiptk::TR::CLS, ID, (XM != hiptk::GATHER_MN_VEC), (YM != hiptk::GATHER_MN_VEC),        \
             (XM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX),                                \
-            (YM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX), 0, BP, BQ, BK, 256,               \
+            (YM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX), 0, BP, BQ, BK, WP *WQ * 64,      \
             hiptk::lds_bytes_w<hiptk::TR, BP, BQ, BK>(), #TR "_" #BP "x" #BQ "x" #BK "_" #XM #YM, \
             &hiptk::launch_w<hiptk::TR, BP, BQ, BK, WP, WQ, XM, YM>                            \
     }

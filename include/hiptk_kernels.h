@@ -118,8 +118,9 @@ int hiptk_contract(const hiptk_problem_t* prob,
  * MFMA instruction sustains on the current device (one 4-wave workgroup per CU), with
  * constant operands (random_operands = 0) or pseudo-random operands in [-1, 1) (1).  The
  * clock the part holds under a full matrix-core load depends on the operand data, so the
- * second figure is the practical ceiling for a contraction of random data.  Synchronous;
- * allocates 4 KiB. */
+ * second figure is the practical ceiling for a contraction of random data.  Synchronous:
+ * loads the device for about 150 ms first so that its clock has settled, then times 20
+ * launches; allocates 4 KiB. */
 int hiptk_mfma_ceiling(int cls, int random_operands, double* tflops);
 
 #ifdef __cplusplus
