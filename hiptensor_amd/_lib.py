@@ -75,6 +75,7 @@ _SIGS = {
     "hiptensorAmdPlanInfo": (C.c_int, [vp, C.POINTER(PlanInfo)]),
     "hiptensorAmdPlanTable": (C.c_int64, [vp, C.c_int, i32p, C.c_int64]),
     "hiptk_mfma_ceiling": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_double)]),
+    "hiptk_tile_count": (C.c_int, [C.c_int]),
 }
 for _name, (_res, _args) in _SIGS.items():
     _fn = getattr(lib, _name)

@@ -658,7 +658,9 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
 
     const auto             t0 = std::chrono::steady_clock::now();
     const hipta::ProblemIn in = problemFromDesc(*desc);
-    const std::string      key = planKey(in, (int)find->mSelectionAlgorithm, workspaceSize);
+    // HIPTENSOR_AMD_FORCE_KERNEL="tile[,splitK]" pins the kernel choice (testing / tuning aid)
+    const char*            force = std::getenv("HIPTENSOR_AMD_FORCE_KERNEL");
+    const std::string      key = planKey(in, (int)find->mSelectionAlgorithm, workspaceSize) + (force ? std::string("|force=") + force : std::string());
     PlanState*             st  = h->lookup(key);
     if(!st)
     {
@@ -713,6 +715,21 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
             pick = hipta::time_choices(*h, v, ranked, top, trace);
             if(!trace.empty())
                 log.heuristics(fn, trace.c_str());
+        }
+        if(force)
+        {
+            int       tile = -1, split = 0;
+            const int got = std::sscanf(force, "%d,%d", &tile, &split);
+            size_t    hit = ranked.size();
+            for(size_t i = 0; i < ranked.size() && hit == ranked.size(); i++)
+                if(got >= 1 && ranked[i].sol->tile_id == tile && (got < 2 || ranked[i].split_k == split))
+                    hit = i;
+            if(hit == ranked.size())
+            {
+                log.errorf(fn, "HIPTENSOR_AMD_FORCE_KERNEL=%s matches no candidate (%s)", force, hiptensorGetErrorString(HIPTENSOR_STATUS_EXECUTION_FAILED));
+                return HIPTENSOR_STATUS_EXECUTION_FAILED;
+            }
+            pick = hit;
         }
         const hipta::Choice& c = ranked[pick];
         fresh->magic           = PlanState::MAGIC;

@@ -14,6 +14,10 @@ namespace hiptk
         // the variants whose column operand is contiguous along k are built
         HIPTK_H_ENTRY(TraitsBF16, 7, 256, 192, 64, 4, 2, true, true, 8, 8, false),
         HIPTK_H_ENTRY(TraitsBF16, 7, 256, 192, 64, 4, 2, false, true, 8, 8, false),
+        // four wavefronts (one per SIMD, accumulators in AGPRs) with the register-level pipeline
+        HIPTK_HP_TILE_V8(TraitsBF16, 8, 256, 256, 64, 2, 2, false),
+        HIPTK_HP_ENTRY(TraitsBF16, 9, 256, 192, 64, 2, 2, true, true, 8, 8, false),
+        HIPTK_HP_ENTRY(TraitsBF16, 9, 256, 192, 64, 2, 2, false, true, 8, 8, false),
     };
 
     const KernelEntry* entries_bf16_vec(int* count)

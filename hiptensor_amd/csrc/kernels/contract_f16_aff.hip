@@ -14,8 +14,10 @@ namespace hiptk
         // the variants whose column operand is contiguous along k are built
         HIPTK_H_ENTRY(TraitsF16, 7, 256, 192, 64, 4, 2, true, true, 8, 8, true),
         HIPTK_H_ENTRY(TraitsF16, 7, 256, 192, 64, 4, 2, false, true, 8, 8, true),
-        // 256 x 256 on four wavefronts (128 x 128 each, accumulators in AGPRs), register pipeline
-        HIPTK_HP_ENTRY(TraitsF16, 8, 256, 256, 64, 2, 2, false, false, 8, 8, true),
+        // four wavefronts (one per SIMD, accumulators in AGPRs) with the register-level pipeline
+        HIPTK_HP_TILE_V8(TraitsF16, 8, 256, 256, 64, 2, 2, true),
+        HIPTK_HP_ENTRY(TraitsF16, 9, 256, 192, 64, 2, 2, true, true, 8, 8, true),
+        HIPTK_HP_ENTRY(TraitsF16, 9, 256, 192, 64, 2, 2, false, true, 8, 8, true),
     };
 
     const KernelEntry* entries_f16_aff(int* count)

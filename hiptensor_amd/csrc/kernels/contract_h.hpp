@@ -779,6 +779,11 @@ namespace hiptk
         HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, V, V, KAFF),    \
         HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, V, V, KAFF)
 #define HIPTK_H_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ, KAFF) HIPTK_H_TILE_VV(TR, ID, BP, BQ, BK, WP, WQ, 8, KAFF)
+#define HIPTK_HP_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ, KAFF)                      \
+    HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 8, KAFF),         \
+        HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 8, 8, KAFF),    \
+        HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 8, KAFF),    \
+        HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, 8, 8, KAFF)
 
 // Combinations in which at least one operand is a scalar gather (always staged k-fast).
 #define HIPTK_H_TILE_V1V(TR, ID, BP, BQ, BK, WP, WQ, V)                     \

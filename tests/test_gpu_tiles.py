@@ -1,0 +1,91 @@
+"""GPU parity of every instantiated tile: each tile configuration of each kernel class is
+pinned through HIPTENSOR_AMD_FORCE_KERNEL (without and with split-K) and checked against the
+CPU oracle, on layouts that cover the row-fast, k-fast and mixed operand gathers.  The
+default selection exercises only a few tiles; this covers the rest, including their steady
+state (K spans several K tiles), K tails and partial tiles in M and N."""
+import os
+
+import pytest
+
+import cases
+import gpu_util
+from hiptensor_amd import api
+from hiptensor_amd import workloads as wl
+from hiptensor_amd._lib import lib
+
+pytestmark = pytest.mark.gpu
+
+ROWS = [("f16", None), ("bf16", None), ("f32", None), ("f64", None), ("c32", None), ("c64", None),
+        ("f32", api.HIPTENSOR_COMPUTE_16F), ("f32", api.HIPTENSOR_COMPUTE_16BF), ("f64", api.HIPTENSOR_COMPUTE_32F)]
+
+
+def layouts(dtype, compute, big):
+    """Row-fast (packed column-major), k-fast and mixed problems; extents are multiples of
+    the widest vector so the vectorised kernels are the ones selected."""
+    m, n, k = ((40, 9), (24, 13), (16, 27)) if big else ((40, 5), (24, 7), (16, 9))
+    a, b = (1.1 + 1.2j, 2.2 + 2.3j) if dtype.startswith("c") else (1.5, 0.75)
+    ext = {0: m[0], 1: m[1], 10: n[0], 11: n[1], 20: k[0], 21: k[1]}
+    out = [wl._rank4(dtype, compute, m, n, k, a, b, f"tiles_rowfast_{dtype}"),
+           wl.make_workload(dtype, compute, [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], ext, a, None,
+                            name=f"tiles_kfast_{dtype}"),
+           wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], ext, a, b,
+                            name=f"tiles_mixed_{dtype}")]
+    # K modes in a different order in A and B: they cannot fuse into one stride (table-driven k offsets)
+    out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 21, 20], [0, 1, 10, 11],
+                                ext, a, b, name=f"tiles_ktable_{dtype}"))
+    # odd extents: scalar gathers on every operand
+    odd = {0: 7, 1: 23, 10: 5, 11: 29, 20: 3, 21: 37 if big else 21}
+    out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], odd, a, b,
+                                name=f"tiles_scalar_{dtype}"))
+    return out
+
+
+@pytest.mark.parametrize("dtype,compute", ROWS)
+def test_every_tile_of_the_class(gpu_handle, oracle_mod, dtype, compute):
+    compute = cases.COMPUTE[dtype] if compute is None else compute
+    big = dtype in ("f16", "bf16") or compute in (api.HIPTENSOR_COMPUTE_16F, api.HIPTENSOR_COMPUTE_16BF)
+    ws_ = layouts(dtype, compute, big)
+    probe = wl.Contraction(gpu_handle, ws_[0])
+    cls = probe.info["kernel_class"]
+    probe.close()
+    ntiles = lib.hiptk_tile_count(cls)
+    assert ntiles >= 2
+    covered = {}
+    try:
+        for w in ws_:
+            inp = wl.host_inputs(w)
+            exp = cases.logical_view(w, oracle_mod.contract(w, inp["A"], inp["B"], inp["C"]))
+            for tile in range(ntiles):
+                for split in (1, 2):
+                    os.environ["HIPTENSOR_AMD_FORCE_KERNEL"] = f"{tile},{split}"
+                    print(f"[case] {w['name']} compute={compute} tile={tile} split={split}", flush=True)
+                    try:
+                        got, info = gpu_util.run_gpu(gpu_handle, w, inp, pref=api.HIPTENSOR_WORKSPACE_MAX, return_info=True)
+                    except api.HiptensorError as e:
+                        # the tile is not instantiated for this layout (or the id is unused)
+                        assert e.status == api.HIPTENSOR_STATUS_EXECUTION_FAILED, e
+                        continue
+                    assert info["split_k"] == split
+                    cases.assert_parity(w, cases.logical_view(w, got), exp, info["kernel_name"])
+                    covered.setdefault(tile, set()).add(info["kernel_name"])
+    finally:
+        os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
+    # every tile id that has a kernel at all must have run on at least one layout
+    missing = [t for t in range(ntiles) if t not in covered and _tile_exists(cls, t)]
+    assert not missing, f"tiles never exercised: {missing}"
+    print("covered:", {t: sorted(v) for t, v in covered.items()}, flush=True)
+
+
+def _tile_exists(cls, tile):
+    import ctypes
+
+    class TileInfo(ctypes.Structure):
+        _fields_ = [("tile_id", ctypes.c_int32), ("bp", ctypes.c_int32), ("bq", ctypes.c_int32),
+                    ("bk", ctypes.c_int32), ("threads", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
+                    ("name", ctypes.c_char * 64)]
+
+    fn = lib.hiptk_tile_info
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(TileInfo)]
+    ti = TileInfo()
+    return fn(cls, tile, ctypes.byref(ti)) == 0
