@@ -713,8 +713,15 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
                 top = (size_t)std::max(1, std::atoi(e));
             std::string trace;
             pick = hipta::time_choices(*h, v, ranked, top, trace);
-            if(!trace.empty())
-                log.heuristics(fn, trace.c_str());
+            // one log line per timed candidate
+            for(size_t b = 0; b < trace.size();)
+            {
+                size_t e = trace.find("; ", b);
+                if(e == std::string::npos)
+                    e = trace.size();
+                log.heuristics(fn, trace.substr(b, e - b).c_str());
+                b = e + 2;
+            }
         }
         if(force)
         {

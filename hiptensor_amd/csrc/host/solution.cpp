@@ -110,12 +110,12 @@ namespace hipta
 
     namespace
     {
-        // Measured on MI355X with this library's kernels, as fractions of the class's
-        // nominal MFMA peak per CU: `alone` is what one workgroup of the tile sustains when
-        // it has a CU to itself (latency bound), `full` what a CU sustains with as many of
-        // them resident as fit.  (The f64 figures are against the published 128 flop/clk/CU;
-        // a loop of nothing but v_mfma_f64_16x16x4_f64 sustains 0.46 of that on this part,
-        // so 0.45 is the ceiling there.)
+        // Measured on MI355X with this library's kernels at the device's sustained clock and
+        // with random operands, as fractions of the class's nominal MFMA peak per CU
+        // (2.4 GHz x flop/clk/CU): `alone` is what one workgroup of the tile sustains when it
+        // has a CU to itself (latency bound), `full` what a CU sustains with as many of them
+        // resident as fit.  For orientation, a loop of nothing but MFMA instructions on random
+        // operands sustains 0.65 (f16), 0.71 (bf16), 0.98 (f32) and 0.86 (f64) of nominal.
         struct TileRate
         {
             double alone, full;
@@ -129,14 +129,17 @@ namespace hipta
             case HIPTK_BF16:
             case HIPTK_F32_AS_F16:
             case HIPTK_F32_AS_BF16:
-                return area >= 65536   ? TileRate{0.35, 0.35}
-                       : area >= 49152 ? TileRate{0.34, 0.34}
-                       : area >= 32768 ? TileRate{0.30, 0.30}
-                       : area >= 16384 ? TileRate{0.18, 0.29}
-                                       : TileRate{0.07, 0.20};
+                return area >= 65536   ? TileRate{0.44, 0.44}
+                       : area >= 49152 ? TileRate{0.40, 0.40}
+                       : area >= 32768 ? TileRate{0.38, 0.38}
+                       : area >= 16384 ? TileRate{0.233, 0.325}
+                                       : TileRate{0.107, 0.21};
             case HIPTK_F64:
-            case HIPTK_C64: return area >= 16384 ? TileRate{0.385, 0.42} : TileRate{0.20, 0.45};
-            default: return area >= 16384 ? TileRate{0.45, 0.50} : TileRate{0.24, 0.60};
+            case HIPTK_C64:
+                return area >= 16384  ? TileRate{0.76, 0.76}
+                       : area >= 4096 ? TileRate{0.45, 0.78}
+                                      : TileRate{0.12, 0.69};
+            default: return area >= 16384 ? TileRate{0.74, 0.74} : TileRate{0.45, 0.72};
             }
         }
     }
@@ -155,7 +158,15 @@ namespace hipta
         const double per_cu  = std::ceil(wgs / dev.cus); // workgroups the busiest CU runs
         const double sharing = std::min<double>(resident, per_cu);
         TileRate     r       = tile_rate(v.cls, s.bp * s.bq);
-        if(v.x_vec == 1 || v.y_vec == 1)
+        if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152)
+        {
+            // the four-wave register-pipelined form of the large tiles: a little faster in
+            // its main loop, slower in the epilogue that reads C
+            const double f = v.bilinear ? 0.97 : 1.02;
+            r.alone *= f;
+            r.full *= f;
+        }
+        if((v.x_vec == 1 || v.y_vec == 1) && class_max_vec(v.cls) > 1)
         {
             r.alone *= 0.35; // scalar gathers are issue bound
             r.full *= 0.35;
@@ -169,7 +180,7 @@ namespace hipta
                              * v.elem_bytes;
         us = std::max(us, bytes / (dev.hbm_gbs * 1e3 * 0.6));
         // launch, and prologue + epilogue of every round of workgroups on a CU
-        us += 3.0 + 1.5 * std::ceil(per_cu / sharing);
+        us += 2.0 + 1.0 * std::ceil(per_cu / sharing);
         if(split > 1)
         {
             const double ws = (double)split * v.P * v.Q * class_acc_bytes(v.cls);

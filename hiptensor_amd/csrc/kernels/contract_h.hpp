@@ -364,6 +364,9 @@ namespace hiptk
         const int wave = tid >> 6;
         const int wp   = wave / WQ;
         const int wq   = wave % WQ;
+#ifdef HIPTK_CLOCK_PROBE
+        const long long cp_c0 = clock64(), cp_w0 = wall_clock64();
+#endif
 
         int tp, tq;
         tile_coords(blockIdx.x, a.tiles_p, a.tiles_q, tp, tq);
@@ -520,23 +523,21 @@ namespace hiptk
                     else
                         load_frags(lx, ly, ks + 1, (ks + 1) & 1);
                     mma(ks & 1);
+                    // an operand's staging registers are refilled right after they are stored:
+                    // the gather of tile kt+2 then has a whole tile of MFMA time to arrive
                     if(ks == 0)
                     {
                         sx.commit(nx);
+                        sx.template fetch<false>(a.X, (kt + 2) * BK, a.K, a.xk_stride);
+                        sx.load_koffs(a.xk, (kt + 3) * BK);
                         interleave(DsWrite{}, std::integral_constant<int, decltype(sx)::N>{});
                     }
                     else if(ks == 1)
                     {
                         sy.commit(ny);
-                        interleave(DsWrite{}, std::integral_constant<int, decltype(sy)::N>{});
-                    }
-                    else if(ks == 2)
-                    {
-                        sx.template fetch<false>(a.X, (kt + 2) * BK, a.K, a.xk_stride);
                         sy.template fetch<false>(a.Y, (kt + 2) * BK, a.K, a.yk_stride);
-                        sx.load_koffs(a.xk, (kt + 3) * BK);
                         sy.load_koffs(a.yk, (kt + 3) * BK);
-                        interleave(VmemRead{}, std::integral_constant<int, decltype(sx)::N + decltype(sy)::N>{});
+                        interleave(DsWrite{}, std::integral_constant<int, decltype(sy)::N>{});
                     }
                     else
                         interleave(DsWrite{}, std::integral_constant<int, 0>{});
@@ -599,6 +600,14 @@ namespace hiptk
         }
 
         // ---- epilogue ----
+#ifdef HIPTK_CLOCK_PROBE
+        if(a.ws && a.split_k == 1 && tid == 0 && blockIdx.x < 256)
+        {
+            long long* o = (long long*)a.ws + 2 * blockIdx.x;
+            o[0]         = clock64() - cp_c0;
+            o[1]         = wall_clock64() - cp_w0;
+        }
+#endif
         const float alpha = (float)a.alpha[0];
         const float beta  = (float)a.beta[0];
         if(a.split_k > 1)
@@ -634,11 +643,50 @@ namespace hiptk
             // wave's accumulators through LDS (the operand buffers are free now) so that a
             // lane ends up with 8 consecutive q of one row and moves them as one 16-byte
             // access; 16 lanes cover 256 contiguous bytes of a row.
-            constexpr int EP = WTQ + 4; // floats per staged row
+            constexpr int EP   = WTQ + 4; // floats per staged row
+            constexpr int VPR  = WTQ / 8; // 8-element vectors per staged row
+            constexpr int NVEC = (32 * WTQ / 8) / 64; // vectors per lane and slab
             static_assert(32 * EP * 4 * WP * WQ <= 2 * STAGE * 2, "epilogue staging must fit the operand buffers");
             float*    st = (float*)lds + wave * (32 * EP);
             const int pw = p0 + wp * WTP;
             const int qw = q0 + wq * WTQ;
+            const bool bil = a.bilinear != 0;
+            // Offsets and C values of a slab are fetched while the slab before it is being
+            // written, so that table look-ups, C loads and D stores of different vectors are
+            // all in flight together instead of one dependent round trip per vector.  (The
+            // compiler cannot hoist them itself: D may alias C.)  A lane reads every C element
+            // before it writes the D element at the same place, so exact aliasing stays valid.
+            uint32_t dqo[NVEC], cqo[NVEC];
+            bool     qok[NVEC];
+#pragma unroll
+            for(int v = 0; v < NVEC; v++)
+            {
+                const int q = qw + ((v * 64 + lane) % VPR) * 8;
+                qok[v]      = q < a.Q;
+                dqo[v]      = qok[v] ? (uint32_t)a.dq[q] : 0u;
+                cqo[v]      = (qok[v] && bil) ? (uint32_t)a.cq[q] : 0u;
+            }
+            struct Slab
+            {
+                u32x4_t  c[NVEC];
+                uint32_t doff[NVEC];
+                bool     ok[NVEC];
+            };
+            Slab sl[2];
+            auto prefetch = [&](int i, Slab& s) {
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    const int p = pw + i * 32 + (v * 64 + lane) / VPR;
+                    s.ok[v]     = qok[v] && p < a.P;
+                    s.doff[v]   = s.ok[v] ? (uint32_t)a.dp[p] + dqo[v] : 0u;
+                    u32x4_t c4  = {0u, 0u, 0u, 0u};
+                    if(s.ok[v] && bil)
+                        c4 = *(const u32x4_t*)(Cp + ((uint32_t)a.cp[p] + cqo[v]));
+                    s.c[v] = c4;
+                }
+            };
+            prefetch(0, sl[0]);
 #pragma unroll
             for(int i = 0; i < TP; i++)
             {
@@ -647,26 +695,25 @@ namespace hiptk
 #pragma unroll
                     for(int r = 0; r < 16; r++)
                         st[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
+                if(i + 1 < TP)
+                    prefetch(i + 1, sl[(i + 1) & 1]);
                 wave_lds_fence();
+                const Slab& cur = sl[i & 1];
 #pragma unroll
-                for(int v = 0; v < (32 * WTQ / 8) / 64; v++)
+                for(int v = 0; v < NVEC; v++)
                 {
-                    constexpr int VPR  = WTQ / 8; // 8-element vectors per staged row
-                    const int     slot = v * 64 + lane;
-                    const int     row  = slot / VPR;
-                    const int     qv   = (slot % VPR) * 8;
-                    const int p = pw + i * 32 + row;
-                    const int q = qw + qv;
-                    if(p < a.P && q < a.Q)
+                    const int slot = v * 64 + lane;
+                    const int row  = slot / VPR;
+                    const int qv   = (slot % VPR) * 8;
+                    if(cur.ok[v])
                     {
-                        const float*   src = st + row * EP + qv;
-                        const f32x4_t  lo  = *(const f32x4_t*)src;
-                        const f32x4_t  hi  = *(const f32x4_t*)(src + 4);
-                        float          v8[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        const uint32_t doff  = (uint32_t)a.dp[p] + (uint32_t)a.dq[q];
-                        if(a.bilinear)
+                        const float*  src   = st + row * EP + qv;
+                        const f32x4_t lo    = *(const f32x4_t*)src;
+                        const f32x4_t hi    = *(const f32x4_t*)(src + 4);
+                        float         v8[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        if(bil)
                         {
-                            const u32x4_t c4 = *(const u32x4_t*)(Cp + ((uint32_t)a.cp[p] + (uint32_t)a.cq[q]));
+                            const u32x4_t c4 = cur.c[v];
 #pragma unroll
                             for(int e = 0; e < 8; e++)
                             {
@@ -684,7 +731,7 @@ namespace hiptk
 #pragma unroll
                         for(int e = 0; e < 4; e++)
                             o[e] = (uint32_t)Tr::from_f32(v8[2 * e]) | ((uint32_t)Tr::from_f32(v8[2 * e + 1]) << 16);
-                        *(u32x4_t*)(Dp + doff) = o;
+                        *(u32x4_t*)(Dp + cur.doff[v]) = o;
                     }
                 }
                 wave_lds_fence();

@@ -123,6 +123,12 @@ int hiptk_contract(const hiptk_problem_t* prob,
  * launches; allocates 4 KiB. */
 int hiptk_mfma_ceiling(int cls, int random_operands, double* tflops);
 
+/* Fills `bytes` (a multiple of 4) of device memory with pseudo-random finite elements of the
+ * class's storage type, magnitudes in [0.5, 1) and random signs, on `stream`.  No counterpart
+ * in the reference: the measured kernel selection times its candidates on such data, since
+ * the clock this device sustains depends on the operand values. */
+int hiptk_fill_pattern(void* dst, uint64_t bytes, int cls, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
