@@ -403,19 +403,23 @@ namespace hipta
         }
 
         // ---- offset tables ----
-        auto pad256 = [](int64_t n) { return (size_t)((n + 255) / 256 * 256); };
+        // Row / column tables cover every index a tile may overhang to: the largest tile edge is
+        // 256 and need not divide 256 (192-wide tiles), so one extra 256 beyond the rounded
+        // extent; the pad value 0 is the offset of row 0, a valid element.  The k tables get
+        // the same: the kernels read k offsets up to three K tiles ahead.
+        auto padded = [](int64_t n) { return (size_t)((n + 255) / 256 * 256 + 256); };
         int64_t mxp, mxk, myq, myk, mcp, mcq, mdp, mdq;
         bool    ok = true;
-        ok &= make_table(v.pdims, v.P, pad256(v.P), [](const Dim& d) { return d.sx; }, v.xp, mxp);
-        ok &= make_table(v.kdims, v.K, pad256(v.K) + 256, [](const Dim& d) { return d.sx; }, v.xk, mxk);
-        ok &= make_table(v.qdims, v.Q, pad256(v.Q), [](const Dim& d) { return d.sy; }, v.yq, myq);
-        ok &= make_table(v.kdims, v.K, pad256(v.K) + 256, [](const Dim& d) { return d.sy; }, v.yk, myk);
-        ok &= make_table(v.pdims, v.P, pad256(v.P), [](const Dim& d) { return d.sd; }, v.dp, mdp);
-        ok &= make_table(v.qdims, v.Q, pad256(v.Q), [](const Dim& d) { return d.sd; }, v.dq, mdq);
+        ok &= make_table(v.pdims, v.P, padded(v.P), [](const Dim& d) { return d.sx; }, v.xp, mxp);
+        ok &= make_table(v.kdims, v.K, padded(v.K), [](const Dim& d) { return d.sx; }, v.xk, mxk);
+        ok &= make_table(v.qdims, v.Q, padded(v.Q), [](const Dim& d) { return d.sy; }, v.yq, myq);
+        ok &= make_table(v.kdims, v.K, padded(v.K), [](const Dim& d) { return d.sy; }, v.yk, myk);
+        ok &= make_table(v.pdims, v.P, padded(v.P), [](const Dim& d) { return d.sd; }, v.dp, mdp);
+        ok &= make_table(v.qdims, v.Q, padded(v.Q), [](const Dim& d) { return d.sd; }, v.dq, mdq);
         if(in.bilinear)
         {
-            ok &= make_table(v.pdims, v.P, pad256(v.P), [](const Dim& d) { return d.sc; }, v.cp, mcp);
-            ok &= make_table(v.qdims, v.Q, pad256(v.Q), [](const Dim& d) { return d.sc; }, v.cq, mcq);
+            ok &= make_table(v.pdims, v.P, padded(v.P), [](const Dim& d) { return d.sc; }, v.cp, mcp);
+            ok &= make_table(v.qdims, v.Q, padded(v.Q), [](const Dim& d) { return d.sc; }, v.cq, mcq);
         }
         else
             mcp = mcq = 0;

@@ -70,9 +70,11 @@ typedef struct hiptk_problem
     int32_t tile_id; /* index into the class's tile list                      */
     int32_t split_k; /* >= 1; > 1 needs workspace                             */
     int64_t P, Q, K; /* GEMM view extents (rows, columns, reduction)          */
-    /* offset tables, element units.  xp / cp / dp hold P entries padded up to a
-     * multiple of 256 with valid offsets; yq / cq / dq likewise for Q; xk / yk
-     * hold K entries padded with zeros up to a multiple of 256.               */
+    /* offset tables, element units.  xp / cp / dp hold P entries followed by valid
+     * offsets (e.g. 0) up to roundup(P, 256) + 256 entries, so that a tile that
+     * overhangs P reads something harmless; yq / cq / dq likewise for Q; xk / yk
+     * hold K entries followed by zeros up to roundup(K, 256) + 256 entries (the
+     * kernels read k offsets up to three K tiles ahead).                         */
     const int32_t *xp, *xk, *yq, *yk, *cp, *cq, *dp, *dq;
     int32_t x_kfast; /* 1: X vectors run along k, 0: along p                   */
     int32_t y_kfast; /* 1: Y vectors run along k, 0: along q                   */

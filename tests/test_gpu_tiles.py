@@ -33,6 +33,12 @@ def layouts(dtype, compute, big):
     # K modes in a different order in A and B: they cannot fuse into one stride (table-driven k offsets)
     out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 21, 20], [0, 1, 10, 11],
                                 ext, a, b, name=f"tiles_ktable_{dtype}"))
+    # N = 256: a 192-wide tile overhangs the column tables beyond the next multiple of 256
+    ov = {0: 40, 1: 5, 10: 32, 11: 8, 20: 16, 21: 9}
+    out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], ov, a, b,
+                                name=f"tiles_overhang_{dtype}"))
+    out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [0, 1, 10, 11], ov, a, None,
+                                name=f"tiles_overhang_p_{dtype}"))
     # odd extents: scalar gathers on every operand
     odd = {0: 7, 1: 23, 10: 5, 11: 29, 20: 3, 21: 37 if big else 21}
     out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], odd, a, b,
