@@ -135,3 +135,47 @@ def test_concurrent_execution_of_one_plan(gpu_handle, oracle_mod):
     for o in outs:
         cases.assert_parity(w, o.cpu().numpy().view(np.float16), exp, "threads")
     c.close()
+
+
+def test_contraction_inside_a_hip_graph(gpu_handle, oracle_mod):
+    """hiptensorContraction only enqueues kernels on the caller's stream (no allocation, no
+    memset, no synchronisation), so it can be captured into a HIP graph: single-pass and
+    split-K (two kernels + workspace) plans are captured, then replayed three times with new
+    operand values written between the replays; every replay must equal the eager result."""
+    import torch
+
+    for w in (wl.config1(), wl._rank4("f16", cases.COMPUTE["f16"], (16, 12), (8, 20), (8, 24), 1.0, 0.5, "graph_f16")):
+        inp = wl.host_inputs(w)
+        c = wl.Contraction(gpu_handle, w, pref=api.HIPTENSOR_WORKSPACE_RECOMMENDED)
+        A, B, Cd = (gpu_util.to_device(inp[k]) for k in ("A", "B", "C"))
+        D = gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"]))
+        De = torch.empty_like(D)
+        ws = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+        wsp = ws.data_ptr() if c.workspace_bytes else None
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):  # warm-up outside the capture (first launch sets function attributes)
+            assert c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(), wsp, side.cuda_stream) == 0
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            st = c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(), wsp, torch.cuda.current_stream().cuda_stream)
+        assert st == 0
+        rng = np.random.default_rng(7)
+        for rep in range(3):
+            newA = inp["A"].copy()
+            rng.shuffle(newA)
+            A.copy_(gpu_util.to_device(newA))
+            D.copy_(gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"])))
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), De.data_ptr(), wsp, torch.cuda.current_stream().cuda_stream) == 0
+            torch.cuda.synchronize()
+            got = D.cpu().numpy().view(wl.NP_STORE[w["dtype"]])
+            eager = De.cpu().numpy().view(wl.NP_STORE[w["dtype"]])
+            assert np.array_equal(got.view(np.uint8), eager.view(np.uint8)), f"{w['name']} replay {rep} differs from eager"
+            exp = oracle_mod.contract(w, newA, inp["B"], inp["C"])
+            cases.assert_parity(w, got, exp, f"graph replay {rep}")
+        c.close()
