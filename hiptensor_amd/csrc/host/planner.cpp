@@ -366,11 +366,15 @@ namespace hipta
                 vk = vector_width(v.kdims[0].len, strides_except(rows, v.kdims, use_x, &v.kdims[0]), align, v.elem_bytes, maxv);
             if(!rows.empty() && (use_x ? rows[0].sx : rows[0].sy) == 1)
                 vr = vector_width(rows[0].len, strides_except(rows, v.kdims, use_x, &rows[0]), align, v.elem_bytes, maxv);
-            // the kernels are instantiated for full-width vectors and for scalars
-            if(vk < maxv)
-                vk = 1;
-            if(vr < maxv)
-                vr = 1;
+            // the wide classes are instantiated for full-width vectors and for scalars; the
+            // 16-bit classes also for 8- and 4-byte vectors (narrowed jointly below)
+            if(maxv != 8)
+            {
+                if(vk < maxv)
+                    vk = 1;
+                if(vr < maxv)
+                    vr = 1;
+            }
             if(vr > vk)
             {
                 kfast = 0;
@@ -384,6 +388,28 @@ namespace hipta
         };
         pick(true, v.pdims, Xt.align, v.x_kfast, v.x_vec);
         pick(false, v.qdims, Yt.align, v.y_kfast, v.y_vec);
+        if(maxv == 8 && !(v.x_vec == 8 && v.y_vec == 8))
+        {
+            // 16-bit kernels exist for (8,8), (4,4), (2,2), (1,8), (8,1) and (1,1) elements per
+            // vector of (X, Y): narrow the pair to the widest of those both operands admit.  A
+            // narrower vector along the same direction is always valid.
+            if(v.x_vec >= 2 && v.y_vec >= 2)
+                v.x_vec = v.y_vec = std::min(v.x_vec, v.y_vec);
+            else
+            {
+                // scalar gathers are staged k-fast
+                if(v.x_vec < 8)
+                {
+                    v.x_vec   = 1;
+                    v.x_kfast = 1;
+                }
+                if(v.y_vec < 8)
+                {
+                    v.y_vec   = 1;
+                    v.y_kfast = 1;
+                }
+            }
+        }
         v.cd_vec = 1;
         if(!v.qdims.empty() && v.qdims[0].sd == 1 && (!in.bilinear || v.qdims[0].sc == 1))
         {

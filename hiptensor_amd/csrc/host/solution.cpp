@@ -166,10 +166,15 @@ namespace hipta
             r.alone *= f;
             r.full *= f;
         }
-        if((v.x_vec == 1 || v.y_vec == 1) && class_max_vec(v.cls) > 1)
+        if(class_max_vec(v.cls) > 1)
         {
-            r.alone *= 0.35; // scalar gathers are issue bound
-            r.full *= 0.35;
+            // narrower gathers are issue bound: measured on 2040^3 f16 problems whose runs
+            // admit 16 / 8 / 4 / 2 bytes per load: 456 / 395 / 209 / 114 TFLOP/s
+            const int    vmin = std::min(v.x_vec, v.y_vec);
+            const int    full = class_max_vec(v.cls);
+            const double f    = vmin >= full ? 1.0 : vmin * 2 >= full ? 0.87 : vmin * 4 >= full && vmin > 1 ? 0.45 : 0.25;
+            r.alone *= f;
+            r.full *= f;
         }
         const double frac     = std::min(sharing * r.alone, r.full);
         const double flops_wg = class_flops_per_mac(v.cls) * (double)s.bp * s.bq * kper;

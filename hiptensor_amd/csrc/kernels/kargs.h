@@ -46,6 +46,10 @@ namespace hiptk
     const KernelEntry* entries_f16_gen(int* count);
     const KernelEntry* entries_bf16_vec(int* count);
     const KernelEntry* entries_bf16_gen(int* count);
+    const KernelEntry* entries_f16_v4(int* count);
+    const KernelEntry* entries_f16_v2(int* count);
+    const KernelEntry* entries_bf16_v4(int* count);
+    const KernelEntry* entries_bf16_v2(int* count);
     const KernelEntry* entries_f32(int* count);
     const KernelEntry* entries_f64(int* count);
     const KernelEntry* entries_c32(int* count);

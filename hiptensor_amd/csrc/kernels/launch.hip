@@ -23,6 +23,10 @@ namespace hiptk
                                           entries_f16_gen,
                                           entries_bf16_vec,
                                           entries_bf16_gen,
+                                          entries_f16_v4,
+                                          entries_f16_v2,
+                                          entries_bf16_v4,
+                                          entries_bf16_v2,
                                           entries_f32,
                                           entries_f64,
                                           entries_c32,

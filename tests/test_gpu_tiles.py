@@ -39,6 +39,16 @@ def layouts(dtype, compute, big):
                                 name=f"tiles_overhang_{dtype}"))
     out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [0, 1, 10, 11], ov, a, None,
                                 name=f"tiles_overhang_p_{dtype}"))
+    if big:
+        # runs that admit only 8-byte and 4-byte vectors (row-fast, k-fast and mixed)
+        for tag, e0 in (("v4", 12), ("v2", 10)):
+            ev = {0: e0, 1: 9, 10: e0, 11: 13, 20: e0, 21: 27}
+            out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ev, a, b,
+                                        name=f"tiles_{tag}_rowfast_{dtype}"))
+            out.append(wl.make_workload(dtype, compute, [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], ev, a, None,
+                                        name=f"tiles_{tag}_kfast_{dtype}"))
+            out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], ev, a, b,
+                                        name=f"tiles_{tag}_mixed_{dtype}"))
     # odd extents: scalar gathers on every operand
     odd = {0: 7, 1: 23, 10: 5, 11: 29, 20: 3, 21: 37 if big else 21}
     out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], odd, a, b,

@@ -105,7 +105,25 @@ def test_vector_width_follows_runs_and_alignment(host_handle):
     ext[0], ext[1] = 12, 5  # the fused M run has 60 elements: not a multiple of 8
     w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
     info, _ = plan(host_handle, w)
-    assert info["y_vec"] == 1 and info["x_vec"] == 8
+    # 16-bit kernels exist for (8,8), (4,4), (2,2), (8,1), (1,8), (1,1): the pair is narrowed jointly
+    assert (info["x_vec"], info["y_vec"]) == (4, 4)
+    ext[0], ext[1] = 10, 3  # runs of 30 elements: 4-byte vectors
+    w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"]) == (2, 2)
+    ext[0], ext[1] = 5, 3  # odd run: that operand is a scalar gather (staged k-fast), the other keeps 16 bytes
+    w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"], info["y_kfast"]) == (8, 1, 1)
+    ext[10], ext[11] = 12, 3  # ... and a 4-element run beside a scalar operand falls to scalar as well
+    w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"], info["x_kfast"], info["y_kfast"]) == (1, 1, 1, 1)
+    # the wide classes have full-width or scalar kernels only
+    ext = {0: 6, 1: 5, 10: 8, 11: 10, 20: 16, 21: 5}
+    w = wl.make_workload("f32", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"]) == (4, 1)
 
 
 def test_extent_one_modes_and_missing_groups(host_handle):
