@@ -132,7 +132,7 @@ namespace hipta
                 return area >= 65536   ? TileRate{0.44, 0.44}
                        : area >= 49152 ? TileRate{0.40, 0.40}
                        : area >= 32768 ? TileRate{0.38, 0.38}
-                       : area >= 16384 ? TileRate{0.233, 0.325}
+                       : area >= 16384 ? TileRate{0.265, 0.315}
                                        : TileRate{0.107, 0.21};
             case HIPTK_F64:
             case HIPTK_C64:
@@ -149,11 +149,9 @@ namespace hipta
         const double tiles  = std::ceil((double)v.P / s.bp) * std::ceil((double)v.Q / s.bq);
         const double ktiles = std::ceil((double)v.K / s.bk);
         const double kper   = std::ceil(ktiles / split) * s.bk;
-        // workgroups that fit on one CU at a time (LDS bound; the 256 x 256 tile also fills
-        // the register file on its own)
-        int resident = std::max(1, std::min(4, dev.lds_per_cu / std::max(1, s.lds_bytes)));
-        if(s.threads >= 512)
-            resident = 1;
+        // workgroups that fit on one CU at a time: bound by LDS and by 16 wavefronts per CU
+        // (kernels are compiled for at least two waves per SIMD, none for more than four)
+        int resident = std::max(1, std::min({4, dev.lds_per_cu / std::max(1, s.lds_bytes), 1024 / std::max(64, s.threads)}));
         const double wgs     = tiles * split;
         const double per_cu  = std::ceil(wgs / dev.cus); // workgroups the busiest CU runs
         const double sharing = std::min<double>(resident, per_cu);

@@ -6,7 +6,7 @@ namespace hiptk
 {
     static const KernelEntry k_entries[] = {
         HIPTK_H_TILE_V8(TraitsF16, 0, 256, 256, 64, 2, 4, true),
-        HIPTK_H_TILE_V8(TraitsF16, 1, 128, 128, 64, 2, 2, true),
+        HIPTK_H_TILE_V8(TraitsF16, 1, 128, 128, 64, 2, 4, true),
         HIPTK_H_TILE_V8(TraitsF16, 2, 64, 64, 64, 2, 2, true),
         HIPTK_H_TILE_V8(TraitsF16, 5, 256, 128, 64, 4, 2, true),
         HIPTK_H_TILE_V8(TraitsF16, 6, 128, 256, 64, 2, 4, true),
