@@ -280,9 +280,10 @@ class Contraction:
         bil = w["beta"] is not None
         self.dC = chk(api.hiptensorInitTensorDescriptor(handle, w["lens"]["D"], w["strides"]["C"], t), "descC") if bil else None
         m = w["modes"]
+        al = align if isinstance(align, dict) else {t: align for t in "ABCD"}  # bytes, per tensor
         self.desc = chk(api.hiptensorInitContractionDescriptor(
-            handle, self.dA, m["A"], align, self.dB, m["B"], align,
-            self.dC, m["D"] if bil else None, align if bil else 0, self.dD, m["D"], align, w["compute"]), "contraction desc")
+            handle, self.dA, m["A"], al["A"], self.dB, m["B"], al["B"],
+            self.dC, m["D"] if bil else None, al["C"] if bil else 0, self.dD, m["D"], al["D"], w["compute"]), "contraction desc")
         self.find = chk(api.hiptensorInitContractionFind(handle, algo), "find")
         self.workspace_bytes = chk(api.hiptensorContractionGetWorkspaceSize(handle, self.desc, self.find, pref), "workspace")
         if workspace_limit is not None:

@@ -179,3 +179,57 @@ def test_contraction_inside_a_hip_graph(gpu_handle, oracle_mod):
             exp = oracle_mod.contract(w, newA, inp["B"], inp["C"])
             cases.assert_parity(w, got, exp, f"graph replay {rep}")
         c.close()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32", "f64"])
+def test_pointer_alignment_drives_the_vector_width(gpu_handle, oracle_mod, dtype):
+    """Operands at addresses that are only 8-, 4- or 2-byte aligned: the alignment reported by
+    hiptensorGetAlignmentRequirement goes into the descriptor, the planner narrows the gathers
+    to it (16-bit classes: 8 -> 4 -> 2 -> 1 elements; wide classes: full width or scalar),
+    and the result still matches the oracle."""
+    import torch
+
+    a, b = 1.5, 0.75
+    w = wl._rank4(dtype, cases.COMPUTE[dtype], (16, 6), (8, 10), (8, 9), a, b, f"misaligned_{dtype}")
+    inp = wl.host_inputs(w)
+    exp = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
+    eb = wl.ELEM_BYTES[dtype]
+    seen = set()
+    for shift in (0, 8, 4, 2):
+        if shift % eb:
+            continue
+        bufs = {}
+        for k in ("A", "B", "C"):
+            raw = torch.zeros(inp[k].nbytes + 64, dtype=torch.uint8, device="cuda")
+            base = (-raw.data_ptr()) % 16 + shift  # exactly `shift` beyond a 16-byte boundary
+            view = raw[base:base + inp[k].nbytes]
+            view.copy_(gpu_util.to_device(inp[k]))
+            bufs[k] = (raw, view)
+        nanD = wl.nan_buffer(dtype, inp["spanD"])
+        rawD = torch.zeros(nanD.nbytes + 64, dtype=torch.uint8, device="cuda")
+        baseD = (-rawD.data_ptr()) % 16 + shift
+        viewD = rawD[baseD:baseD + nanD.nbytes]
+        viewD.copy_(gpu_util.to_device(nanD))
+        probe = wl.Contraction(gpu_handle, w)
+        al = {}
+        for k, (d, ptr) in {"A": (probe.dA, bufs["A"][1].data_ptr()), "B": (probe.dB, bufs["B"][1].data_ptr()),
+                            "C": (probe.dC, bufs["C"][1].data_ptr()), "D": (probe.dD, viewD.data_ptr())}.items():
+            al[k] = api.check(api.hiptensorGetAlignmentRequirement(gpu_handle, ptr, d), "alignment")
+            assert al[k] == (16 if shift == 0 else shift), (k, shift, al[k])
+        probe.close()
+        c = wl.Contraction(gpu_handle, w, align=al)
+        full = {"f16": 8, "f32": 4, "f64": 2}[dtype]
+        want = max(1, min(full, (16 if shift == 0 else shift) // eb))
+        if dtype != "f16" and want < full:
+            want = 1
+        assert (c.info["x_vec"], c.info["y_vec"]) == (want, want), (shift, c.info)
+        seen.add(want)
+        ws = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+        st = c.run(bufs["A"][1].data_ptr(), bufs["B"][1].data_ptr(), bufs["C"][1].data_ptr(), viewD.data_ptr(),
+                   ws.data_ptr() if c.workspace_bytes else None, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert st == 0
+        got = viewD.cpu().numpy().view(wl.NP_STORE[dtype])
+        cases.assert_parity(w, got, exp, f"shift {shift} {c.info['kernel_name']}")
+        c.close()
+    assert len(seen) >= 2
