@@ -47,17 +47,10 @@ namespace hiptk
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
 
+    // f32 -> bf16, round to nearest even: v_cvt_pk_bf16_f32 on gfx950 (NaNs come out quiet)
     __device__ inline uint16_t f32_to_bf16_rne(float f)
     {
-        uint32_t x = __float_as_uint(f);
-        if((~x & 0x7F800000u) == 0)
-        {
-            if(x & 0xFFFFu)
-                x |= 0x10000u;
-        }
-        else
-            x += 0x7FFFu + ((x >> 16) & 1u);
-        return (uint16_t)(x >> 16);
+        return __builtin_bit_cast(uint16_t, (__bf16)f);
     }
 
     struct TraitsF16
