@@ -139,7 +139,8 @@ namespace hipta
                 return area >= 16384  ? TileRate{0.76, 0.76}
                        : area >= 4096 ? TileRate{0.45, 0.78}
                                       : TileRate{0.12, 0.69};
-            default: return area >= 16384 ? TileRate{0.74, 0.74} : TileRate{0.45, 0.72};
+            case HIPTK_C32: return area >= 16384 ? TileRate{0.78, 0.78} : TileRate{0.48, 0.77};
+            default: return area >= 16384 ? TileRate{0.73, 0.73} : TileRate{0.36, 0.66};
             }
         }
     }
@@ -160,7 +161,8 @@ namespace hipta
         {
             // the four-wave register-pipelined form of the large tiles: a little faster in
             // its main loop, slower in the epilogue that reads C
-            const double f = v.bilinear ? 0.97 : 1.02;
+            // (and its longer prologue only pays off over many K tiles)
+            const double f = kper / s.bk < 24 ? 0.9 : v.bilinear ? 0.97 : 1.02;
             r.alone *= f;
             r.full *= f;
         }
@@ -183,11 +185,16 @@ namespace hipta
                              * v.elem_bytes;
         us = std::max(us, bytes / (dev.hbm_gbs * 1e3 * 0.6));
         // launch, and prologue + epilogue of every round of workgroups on a CU
-        us += 2.0 + 1.0 * std::ceil(per_cu / sharing);
+        // (a workgroup's epilogue moves its output tile, and C, at about 30 GB/s per CU)
+        const double tile_io = (double)s.bp * s.bq * v.elem_bytes * (v.bilinear ? 2.0 : 1.0) / 30e3;
+        us += 2.0 + (1.0 + tile_io) * std::ceil(per_cu / sharing);
         if(split > 1)
         {
             const double ws = (double)split * v.P * v.Q * class_acc_bytes(v.cls);
-            us += 2.0 * ws / (dev.hbm_gbs * 1e3 * 0.6) + 3.0; // partials out and back, second launch
+            // partials out and back, second launch; partials that fit the 256 MiB last-level
+            // cache never reach HBM
+            const double bw = ws <= 160e6 ? dev.hbm_gbs * 1e3 * 1.0 : dev.hbm_gbs * 1e3 * 0.6;
+            us += 2.0 * ws / bw + 3.0 + 0.12 * split; // the reduction walks the slices one after another
         }
         return us;
     }
