@@ -202,6 +202,12 @@ def main():
                             "mfma_only_sustained_tflops": sustained,
                             "hbm_GBs_algorithmic": wl.algorithmic_bytes(cw) / (rr["kernel_ms"] * 1e-3) / 1e9,
                             "kernel": rr["info"]["kernel_name"], "split_k": rr["info"]["split_k"], "dtype": cw["dtype"]}
+        if not a.no_cpu:
+            # the reference's CPU contraction beside the other configurations too: in full where
+            # that takes seconds, on a slab for the rank-6 problem
+            for name in ("cfg1", "cfg3", "cfg4", "cfg5"):
+                if name in others:
+                    others[name]["cpu_baseline"] = cpu_baseline(cfgs[name])
         out["others"] = others
     if a.copy_calibration:
         src = torch.ones(1 << 28, dtype=torch.uint8, device="cuda")
