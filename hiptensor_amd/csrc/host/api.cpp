@@ -759,6 +759,11 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         p.y_vec                = v.y_vec;
         p.cd_vec               = v.cd_vec;
         p.k_affine             = v.k_affine;
+        p.cd_affine = v.cd_affine;
+        p.dp_stride = (int32_t)v.dp_stride;
+        p.dq_stride = (int32_t)v.dq_stride;
+        p.cp_stride = (int32_t)v.cp_stride;
+        p.cq_stride = (int32_t)v.cq_stride;
         p.xk_stride            = (int32_t)v.xk_stride;
         p.yk_stride            = (int32_t)v.yk_stride;
         fresh->kernel_name     = hiptk_kernel_name(&p);

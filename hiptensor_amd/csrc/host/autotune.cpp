@@ -83,6 +83,11 @@ namespace hipta
         p.y_vec   = v.y_vec;
         p.cd_vec  = v.cd_vec;
         p.k_affine  = v.k_affine;
+        p.cd_affine = v.cd_affine;
+        p.dp_stride = (int32_t)v.dp_stride;
+        p.dq_stride = (int32_t)v.dq_stride;
+        p.cp_stride = (int32_t)v.cp_stride;
+        p.cq_stride = (int32_t)v.cq_stride;
         p.xk_stride = (int32_t)v.xk_stride;
         p.yk_stride = (int32_t)v.yk_stride;
         p.xp      = base + offs[0];

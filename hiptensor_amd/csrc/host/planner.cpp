@@ -348,6 +348,18 @@ namespace hipta
                 v.k_affine = 0;
         }
 
+        if(v.pdims.size() <= 1 && v.qdims.size() <= 1)
+        {
+            v.cd_affine = 1;
+            v.dp_stride = v.pdims.empty() ? 0 : v.pdims[0].sd;
+            v.cp_stride = v.pdims.empty() ? 0 : v.pdims[0].sc;
+            v.dq_stride = v.qdims.empty() ? 0 : v.qdims[0].sd;
+            v.cq_stride = v.qdims.empty() ? 0 : v.qdims[0].sc;
+            for(int64_t st : {v.dp_stride, v.dq_stride, v.cp_stride, v.cq_stride})
+                if(st > 0x7FFFFFFFll)
+                    v.cd_affine = 0;
+        }
+
         // ---- gather direction and vector width per operand ----
         const int maxv = class_max_vec(v.cls);
         const TensorIn& Xt = v.swapped ? B : A;

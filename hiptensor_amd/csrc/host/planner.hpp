@@ -58,6 +58,9 @@ namespace hipta
         // the K modes fused into (at most) one: k offsets are k * stride
         int     k_affine = 0;
         int64_t xk_stride = 0, yk_stride = 0;
+        // P and Q each fused into (at most) one dim in C and D: offsets are index * stride
+        int     cd_affine = 0;
+        int64_t dp_stride = 0, dq_stride = 0, cp_stride = 0, cq_stride = 0;
         int elem_bytes = 0;
         // bytes each tensor spans in memory (1 + sum (len-1)*stride elements)
         int64_t spanA = 0, spanB = 0, spanC = 0, spanD = 0;

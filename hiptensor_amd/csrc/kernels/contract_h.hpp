@@ -358,6 +358,8 @@ namespace hiptk
         const int wp   = wave / WQ;
         const int wq   = wave % WQ;
 #ifdef HIPTK_CLOCK_PROBE
+        // diagnostic build: shader-clock cycles of the main loop and 100 MHz wall-clock stamps
+        // of the kernel's stages go to the workspace (8 x int64 per workgroup, first 256)
         const long long cp_c0 = clock64(), cp_w0 = wall_clock64();
 #endif
 
@@ -441,6 +443,9 @@ namespace hiptk
             lds_barrier();
         }
 
+#ifdef HIPTK_CLOCK_PROBE
+        const long long cp_c1 = clock64(), cp_w1 = wall_clock64();
+#endif
         int buf = 0;
         int kt  = kt_begin;
         // steady state: tile kt+2 exists and is a full tile
@@ -594,12 +599,21 @@ namespace hiptk
 
         // ---- epilogue ----
 #ifdef HIPTK_CLOCK_PROBE
-        if(a.ws && a.split_k == 1 && tid == 0 && blockIdx.x < 256)
-        {
-            long long* o = (long long*)a.ws + 2 * blockIdx.x;
-            o[0]         = clock64() - cp_c0;
-            o[1]         = wall_clock64() - cp_w0;
-        }
+        const long long cp_c2 = clock64(), cp_w2 = wall_clock64();
+        auto            probe_out = [&]() {
+            __builtin_amdgcn_s_waitcnt(0);
+            if(a.ws && a.split_k == 1 && tid == 0 && blockIdx.x < 256)
+            {
+                long long* o = (long long*)a.ws + 8 * blockIdx.x;
+                o[0]         = cp_c2 - cp_c1; // main loop, shader cycles
+                o[1]         = cp_w2 - cp_w1; // main loop, wall ticks
+                o[2]         = cp_w0;
+                o[3]         = cp_w1;
+                o[4]         = cp_w2;
+                o[5]         = wall_clock64();
+                o[6]         = cp_c1 - cp_c0;
+            }
+        };
 #endif
         const float alpha = (float)a.alpha[0];
         const float beta  = (float)a.beta[0];
@@ -640,10 +654,10 @@ namespace hiptk
             constexpr int VPR  = WTQ / 8; // 8-element vectors per staged row
             constexpr int NVEC = (32 * WTQ / 8) / 64; // vectors per lane and slab
             static_assert(32 * EP * 4 * WP * WQ <= 2 * STAGE * 2, "epilogue staging must fit the operand buffers");
-            float*    st = (float*)lds + wave * (32 * EP);
             const int pw = p0 + wp * WTP;
             const int qw = q0 + wq * WTQ;
             const bool bil = a.bilinear != 0;
+            const bool aff = a.cd_affine != 0;
             // Offsets and C values of a slab are fetched while the slab before it is being
             // written, so that table look-ups, C loads and D stores of different vectors are
             // all in flight together instead of one dependent round trip per vector.  (The
@@ -656,8 +670,10 @@ namespace hiptk
             {
                 const int q = qw + ((v * 64 + lane) % VPR) * 8;
                 qok[v]      = q < a.Q;
-                dqo[v]      = qok[v] ? (uint32_t)a.dq[q] : 0u;
-                cqo[v]      = (qok[v] && bil) ? (uint32_t)a.cq[q] : 0u;
+                // affine C / D (every benchmark-style packed layout): offsets are computed, so the
+                // epilogue starts without a round trip to the offset tables
+                dqo[v] = !qok[v] ? 0u : aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
+                cqo[v] = !(qok[v] && bil) ? 0u : aff ? (uint32_t)q * (uint32_t)a.cq_stride : (uint32_t)a.cq[q];
             }
             struct Slab
             {
@@ -672,63 +688,102 @@ namespace hiptk
                 {
                     const int p = pw + i * 32 + (v * 64 + lane) / VPR;
                     s.ok[v]     = qok[v] && p < a.P;
-                    s.doff[v]   = s.ok[v] ? (uint32_t)a.dp[p] + dqo[v] : 0u;
+                    s.doff[v]   = !s.ok[v] ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
                     u32x4_t c4  = {0u, 0u, 0u, 0u};
                     if(s.ok[v] && bil)
-                        c4 = *(const u32x4_t*)(Cp + ((uint32_t)a.cp[p] + cqo[v]));
+                        c4 = *(const u32x4_t*)(Cp + ((aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p]) + cqo[v]));
                     s.c[v] = c4;
                 }
             };
-            prefetch(0, sl[0]);
-#pragma unroll
-            for(int i = 0; i < TP; i++)
-            {
+            // Two staging buffers per wave when the operand buffers have room for them: slab
+            // i+1 is written to LDS while slab i is read back, converted and stored.
+            constexpr bool DB = 2 * 32 * EP * 4 * WP * WQ <= 2 * STAGE * 2;
+            float* const   st0 = (float*)lds + wave * ((DB ? 2 : 1) * 32 * EP);
+            auto write_slab = [&](int i, float* dst) {
 #pragma unroll
                 for(int j = 0; j < TQ; j++)
 #pragma unroll
                     for(int r = 0; r < 16; r++)
-                        st[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
-                if(i + 1 < TP)
-                    prefetch(i + 1, sl[(i + 1) & 1]);
+                        dst[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
+            };
+            prefetch(0, sl[0]);
+            if constexpr(DB)
+            {
+                write_slab(0, st0);
                 wave_lds_fence();
+            }
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+            {
+                const float* cur_st = st0 + (DB ? (i & 1) * 32 * EP : 0);
+                if constexpr(DB)
+                {
+                    if(i + 1 < TP)
+                    {
+                        prefetch(i + 1, sl[(i + 1) & 1]);
+                        write_slab(i + 1, st0 + ((i + 1) & 1) * 32 * EP);
+                    }
+                }
+                else
+                {
+                    write_slab(i, st0);
+                    if(i + 1 < TP)
+                        prefetch(i + 1, sl[(i + 1) & 1]);
+                    wave_lds_fence();
+                }
                 const Slab& cur = sl[i & 1];
+                // all of the slab's vectors are read from LDS before any is converted and stored
+                f32x4_t lo[NVEC], hi[NVEC];
 #pragma unroll
                 for(int v = 0; v < NVEC; v++)
                 {
-                    const int slot = v * 64 + lane;
-                    const int row  = slot / VPR;
-                    const int qv   = (slot % VPR) * 8;
-                    if(cur.ok[v])
-                    {
-                        const float*  src   = st + row * EP + qv;
-                        const f32x4_t lo    = *(const f32x4_t*)src;
-                        const f32x4_t hi    = *(const f32x4_t*)(src + 4);
-                        float         v8[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        if(bil)
-                        {
-                            const u32x4_t c4 = cur.c[v];
-#pragma unroll
-                            for(int e = 0; e < 8; e++)
-                            {
-                                const uint16_t cb = (uint16_t)(c4[e >> 1] >> ((e & 1) * 16));
-                                v8[e]             = alpha * v8[e] + beta * Tr::to_f32(cb);
-                            }
-                        }
-                        else
-                        {
-#pragma unroll
-                            for(int e = 0; e < 8; e++)
-                                v8[e] = alpha * v8[e];
-                        }
-                        u32x4_t o;
-#pragma unroll
-                        for(int e = 0; e < 4; e++)
-                            o[e] = (uint32_t)Tr::from_f32(v8[2 * e]) | ((uint32_t)Tr::from_f32(v8[2 * e + 1]) << 16);
-                        *(u32x4_t*)(Dp + cur.doff[v]) = o;
-                    }
+                    const int    slot = v * 64 + lane;
+                    const float* src  = cur_st + (slot / VPR) * EP + (slot % VPR) * 8;
+                    lo[v]             = *(const f32x4_t*)src;
+                    hi[v]             = *(const f32x4_t*)(src + 4);
                 }
+                u32x4_t o[NVEC];
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    float v8[8] = {lo[v][0], lo[v][1], lo[v][2], lo[v][3], hi[v][0], hi[v][1], hi[v][2], hi[v][3]};
+                    if(bil)
+                    {
+                        const u32x4_t c4 = cur.c[v];
+#pragma unroll
+                        for(int e = 0; e < 8; e++)
+                        {
+                            const uint16_t cb = (uint16_t)(c4[e >> 1] >> ((e & 1) * 16));
+                            v8[e]             = alpha * v8[e] + beta * Tr::to_f32(cb);
+                        }
+                    }
+                    else
+                    {
+#pragma unroll
+                        for(int e = 0; e < 8; e++)
+                            v8[e] = alpha * v8[e];
+                    }
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        o[v][e] = (uint32_t)Tr::from_f32(v8[2 * e]) | ((uint32_t)Tr::from_f32(v8[2 * e + 1]) << 16);
+                }
+                // Loads and stores share one in-order counter, so waiting for a load also waits
+                // for every store issued before it.  The next slab's prefetch is therefore
+                // awaited here, before this slab's stores are issued: the only stores it can
+                // wait for are the previous slab's, a whole slab old, and this slab's stores
+                // then drain while the next slab is converted.
+                // (With computed offsets and no C there are no loads, and nothing to wait for.)
+                if(bil || !aff)
+                    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                    if(cur.ok[v])
+                        *(u32x4_t*)(Dp + cur.doff[v]) = o[v];
                 wave_lds_fence();
             }
+#ifdef HIPTK_CLOCK_PROBE
+            probe_out();
+#endif
             return;
         }
         {

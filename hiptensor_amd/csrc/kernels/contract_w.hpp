@@ -554,13 +554,15 @@ namespace hiptk
         E*         Dp  = (E*)a.D;
         const E*   Cp  = (const E*)a.C;
         const bool bil = a.bilinear != 0;
+        const bool aff = a.cd_affine != 0; // C / D offsets are index * stride: no table lookups
         uint32_t   dqo[TQ], cqo[TQ];
 #pragma unroll
         for(int j = 0; j < TQ; j++)
         {
             // the q tables are padded with valid entries, so the lookup is safe beyond Q
-            dqo[j] = (uint32_t)a.dq[qw + j * TILE];
-            cqo[j] = bil ? (uint32_t)a.cq[qw + j * TILE] : 0u;
+            const int q = qw + j * TILE;
+            dqo[j]      = aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
+            cqo[j]      = !bil ? 0u : aff ? (uint32_t)q * (uint32_t)a.cq_stride : (uint32_t)a.cq[q];
         }
 #pragma unroll
         for(int i = 0; i < TP; i++)
@@ -570,8 +572,8 @@ namespace hiptk
                 const int p = pw + i * TILE + Tr::p_of(r, lane);
                 if(p >= a.P)
                     continue;
-                const uint32_t dpo = (uint32_t)a.dp[p];
-                const uint32_t cpo = bil ? (uint32_t)a.cp[p] : 0u;
+                const uint32_t dpo = aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p];
+                const uint32_t cpo = !bil ? 0u : aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p];
 #pragma unroll
                 for(int j = 0; j < TQ; j++)
                 {

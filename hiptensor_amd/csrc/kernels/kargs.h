@@ -22,6 +22,8 @@ namespace hiptk
         int32_t bilinear;
         int32_t tiles_p, tiles_q;
         int32_t xk_stride, yk_stride; // element stride of k when the K modes fused into one
+        int32_t cd_affine; // 1: C / D offsets are p * stride + q * stride, no table lookups
+        int32_t dp_stride, dq_stride, cp_stride, cq_stride;
         int32_t cd_vec; // contiguous elements along q shared by C and D
         double  alpha[2], beta[2];
     };

@@ -272,6 +272,11 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
     a.Q  = (int32_t)prob->Q;
     a.K  = (int32_t)prob->K;
     a.bilinear  = bil ? 1 : 0;
+    a.cd_affine = prob->cd_affine;
+    a.dp_stride = prob->dp_stride;
+    a.dq_stride = prob->dq_stride;
+    a.cp_stride = prob->cp_stride;
+    a.cq_stride = prob->cq_stride;
     a.xk_stride = prob->xk_stride;
     a.yk_stride = prob->yk_stride;
     a.cd_vec    = prob->cd_vec;

@@ -85,7 +85,10 @@ typedef struct hiptk_problem
                          a kernel that multiplies instead of reading xk / yk is used when
                          one is instantiated (the tables must still be valid)          */
     int32_t xk_stride, yk_stride;
-    int32_t reserved;
+    int32_t cd_affine; /* 1: dp[p] == p * dp_stride, dq[q] == q * dq_stride (and likewise cp / cq
+                          for a bilinear problem) for all p < P, q < Q: the epilogue then computes
+                          offsets instead of reading the tables (which must still be valid)      */
+    int32_t dp_stride, dq_stride, cp_stride, cq_stride;
 } hiptk_problem_t;
 
 /* Number of tile configurations of a class, and their description. */
