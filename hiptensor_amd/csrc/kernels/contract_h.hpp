@@ -643,6 +643,103 @@ namespace hiptk
         typedef typename Tr::out_t out_t;
         out_t*       Dp = (out_t*)a.D;
         const out_t* Cp = (const out_t*)a.C;
+        if constexpr(sizeof(out_t) == 2 && WTQ >= 128) // (measured: a gain only for the wide wave tiles)
+        if(a.cd_vec == 8 && !a.bilinear)
+        {
+            // Scale with D contiguous along q in runs of 8.  The results are converted to their
+            // 16-bit type in the accumulator layout (lane = column q, 4 consecutive registers =
+            // 4 consecutive rows p) and transposed through LDS at half the f32 volume: a slab is
+            // staged as [q][32 rows + 4] halves with one ds_write_b64 per 4 registers, and read
+            // back with the transposing ds_read_b64_tr_b16, which hands every lane 4 consecutive
+            // q of one row; two of them make the 16-byte store.  A 16-lane group covers 4 rows x
+            // 32 q, a store instruction 4 rows x 256 contiguous bytes (8 x 128 for 64-wide wave
+            // tiles).  The 72-byte column pitch keeps both the writes and the reads conflict free.
+            constexpr int PH   = 36; // halves per staged column: 32 rows + pad
+            constexpr int NVEC = (32 * WTQ / 8) / 64; // 16-byte stores per lane and slab
+            constexpr int QB   = WTQ / 32; // 32-column blocks per wave tile
+            static_assert(2 * WTQ * PH * 2 * WP * WQ <= 2 * STAGE * 2, "epilogue staging must fit the operand buffers");
+            typedef short4_t __attribute__((address_space(3))) * lds_s4_ptr;
+            uint16_t* const st0 = lds + wave * (2 * WTQ * PH);
+            const int       pw  = p0 + wp * WTP;
+            const int       qw  = q0 + wq * WTQ;
+            const bool      aff = a.cd_affine != 0;
+            const int       L   = lane & 15;
+            const int       G   = lane >> 4;
+            // this lane's row within a slab and first column, per store vector
+            int      prow[NVEC], qcol[NVEC];
+            uint32_t dqo[NVEC];
+            bool     qok[NVEC];
+#pragma unroll
+            for(int v = 0; v < NVEC; v++)
+            {
+                const int u = v * 4 + G; // (row quad, column block) unit of this 16-lane group
+                prow[v]     = 4 * (u / QB) + (L & 3);
+                qcol[v]     = 32 * (u % QB) + 8 * (L >> 2);
+                const int q = qw + qcol[v];
+                qok[v]      = q < a.Q;
+                dqo[v]      = !qok[v] ? 0u : aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
+            }
+            uint32_t doff[2][NVEC];
+            auto     offsets = [&](int i, uint32_t (&d)[NVEC]) {
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    const int p = pw + i * 32 + prow[v];
+                    d[v] = !(qok[v] && p < a.P) ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
+                }
+            };
+            auto write_slab = [&](int i, uint16_t* dst) {
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+#pragma unroll
+                    for(int g = 0; g < 4; g++)
+                    {
+                        u32x2_t w;
+                        w[0] = (uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g]) | ((uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 1]) << 16);
+                        w[1] = (uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 2]) | ((uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 3]) << 16);
+                        *(u32x2_t*)(dst + (j * 32 + (lane & 31)) * PH + 8 * g + 4 * (lane >> 5)) = w;
+                    }
+            };
+            offsets(0, doff[0]);
+            write_slab(0, st0);
+            wave_lds_fence();
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+            {
+                const uint16_t* cur = st0 + (i & 1) * (WTQ * PH);
+                if(i + 1 < TP)
+                {
+                    offsets(i + 1, doff[(i + 1) & 1]);
+                    write_slab(i + 1, st0 + ((i + 1) & 1) * (WTQ * PH));
+                }
+                u32x4_t o[NVEC];
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    // the word this lane supplies: column qcol-block + 8 * (L % 4) + L / 4, the group's 4 rows
+                    const int       u   = v * 4 + G;
+                    const uint16_t* src = cur + (32 * (u % QB) + 8 * (L & 3) + (L >> 2)) * PH + 4 * (u / QB);
+                    const short4_t  lo  = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(src));
+                    const short4_t  hi  = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(src + 4 * PH));
+                    const u32x2_t   l2  = __builtin_bit_cast(u32x2_t, lo);
+                    const u32x2_t   h2  = __builtin_bit_cast(u32x2_t, hi);
+                    o[v]                = u32x4_t{l2[0], l2[1], h2[0], h2[1]};
+                }
+                // table-driven offsets are loads: await the next slab's before this slab's stores
+                // go out (loads and stores share one in-order counter)
+                if(!aff)
+                    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                    if(qok[v] && pw + i * 32 + prow[v] < a.P)
+                        *(u32x4_t*)(Dp + doff[i & 1][v]) = o[v];
+                wave_lds_fence();
+            }
+#ifdef HIPTK_CLOCK_PROBE
+            probe_out();
+#endif
+            return;
+        }
         if constexpr(sizeof(out_t) == 2)
         if(a.cd_vec == 8)
         {
