@@ -333,9 +333,10 @@ namespace hipta
         v.P = extent(v.pdims);
         v.Q = extent(v.qdims);
         v.K = extent(v.kdims);
-        if(v.P > 0x7FFFFF00ll || v.Q > 0x7FFFFF00ll || v.K > 0x7FFFFF00ll)
+        // every folded extent gets an int32 offset table on the host and on the device
+        if(v.P > (1ll << 28) || v.Q > (1ll << 28) || v.K > (1ll << 28))
         {
-            why = "a folded extent exceeds 2^31";
+            why = "a folded extent exceeds 2^28 (offset tables would not fit)";
             return PlanStatus::UNSUPPORTED_SHAPE;
         }
 

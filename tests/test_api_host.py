@@ -199,3 +199,13 @@ def test_logger_api(host_handle, tmp_path):
     import re
     assert re.match(r"^\[\d+\]\[\d{4}-\d\d-\d\d \d\d:\d\d:\d\d\]\[hipTensor\]\[Error\]\[\w+\] ", line)
     assert api.hiptensorGetHiprtVersion() != 0
+
+
+def test_folded_extent_limit(host_handle):
+    """Extents whose offset tables could not be held are refused at plan time, not attempted."""
+    from hiptensor_amd import workloads as wl
+
+    w = wl.make_workload("f32", api.HIPTENSOR_COMPUTE_32F, [0, 20], [10, 20], [0, 10], {0: 2, 10: 2, 20: (1 << 28) + 8}, 1.0, None)
+    with pytest.raises(api.HiptensorError) as e:
+        wl.Contraction(host_handle, w)
+    assert e.value.status == api.HIPTENSOR_STATUS_NOT_SUPPORTED
