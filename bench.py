@@ -131,6 +131,8 @@ def main():
     ap.add_argument("--workload", default="cfg2_f16_scale")
     ap.add_argument("--all", action="store_true", help="also time every other configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--pcie", action="store_true",
+                    help="also time the step with operands copied from, and the result to, pinned host memory")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run 3 plain device copies of 256 MiB (a kernel of known traffic, to scale "
                          "the profiler's FETCH_SIZE / WRITE_SIZE counters by)")
@@ -209,6 +211,44 @@ def main():
                 if name in others:
                     others[name]["cpu_baseline"] = cpu_baseline(cfgs[name])
         out["others"] = others
+    if a.pcie:
+        # the same call with operands starting and the result ending in pinned host memory
+        # (never `value`: the API takes device pointers, so this is the application's own copying)
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        import numpy as np
+
+        inp = wl.host_inputs(w, nan_gaps=False)
+        hA = torch.from_numpy(inp["A"].view(np.uint8).copy()).pin_memory()
+        hB = torch.from_numpy(inp["B"].view(np.uint8).copy()).pin_memory()
+        hC = torch.from_numpy(inp["C"].view(np.uint8).copy()).pin_memory() if inp["C"] is not None else None
+        nD = inp["spanD"] * wl.ELEM_BYTES[w["dtype"]]
+        hD = torch.empty(nD, dtype=torch.uint8).pin_memory()
+        dA, dB, dD = torch.empty_like(hA, device="cuda"), torch.empty_like(hB, device="cuda"), torch.empty(nD, dtype=torch.uint8, device="cuda")
+        dC = torch.empty_like(hC, device="cuda") if hC is not None else None
+        c = wl.Contraction(handle, w)
+        wsb = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+        stream = torch.cuda.current_stream()
+
+        def once():
+            dA.copy_(hA, non_blocking=True)
+            dB.copy_(hB, non_blocking=True)
+            if dC is not None:
+                dC.copy_(hC, non_blocking=True)
+            assert c.run(dA.data_ptr(), dB.data_ptr(), dC.data_ptr() if dC is not None else None, dD.data_ptr(),
+                         wsb.data_ptr() if c.workspace_bytes else None, stream.cuda_stream) == 0
+            hD.copy_(dD, non_blocking=True)
+
+        for _ in range(3):
+            once()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            once()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 100.0
+        c.close()
+        out["pcie_inclusive"] = {"ms_per_step": ms, "tflops": fl / (ms * 1e-3) / 1e12,
+                                 "host_bytes_moved": int(hA.numel() + hB.numel() + (hC.numel() if hC is not None else 0) + nD)}
     if a.copy_calibration:
         src = torch.ones(1 << 28, dtype=torch.uint8, device="cuda")
         dst = torch.empty_like(src)
