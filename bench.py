@@ -32,7 +32,7 @@ HBM_PEAK_GBS = 8000.0
 # raw readings and the copy-kernel scale factors).  Keyed by (workload, kernel); null otherwise.
 MEASURED_TRAFFIC_BYTES = {
     ("cfg2_f16_scale_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue"): (2.0 * 98533.9 + 1.0 * 32768.0) * 1024,
-    ("cfg2_f16_scale_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue_pipe"): (2.0 * 98563.0 + 1.0 * 32768.0) * 1024,
+    ("cfg2_f16_scale_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue_pipe2x2"): (2.0 * 98563.0 + 1.0 * 32768.0) * 1024,
 }
 
 

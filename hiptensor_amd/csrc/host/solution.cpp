@@ -159,10 +159,10 @@ namespace hipta
         TileRate     r       = tile_rate(v.cls, s.bp * s.bq);
         if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152)
         {
-            // the four-wave register-pipelined form of the large tiles: a little faster in
-            // its main loop, slower in the epilogue that reads C
-            // (and its longer prologue only pays off over many K tiles)
-            const double f = kper / s.bk < 24 ? 0.9 : v.bilinear ? 0.97 : 1.02;
+            // the four-wave form of the 256 x 256 tile (one wave per SIMD): level with the
+            // eight-wave form over a long K without C, behind it in the epilogue that reads C
+            // and over a short K
+            const double f = kper / s.bk < 24 ? 0.9 : v.bilinear ? 0.95 : 1.005;
             r.alone *= f;
             r.full *= f;
         }

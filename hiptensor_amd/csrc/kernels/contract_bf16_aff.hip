@@ -5,19 +5,17 @@
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
-        HIPTK_H_TILE_V8(TraitsBF16, 0, 256, 256, 64, 2, 4, true),
-        HIPTK_H_TILE_V8(TraitsBF16, 1, 128, 128, 64, 2, 4, true),
+        HIPTK_HP_TILE_V8(TraitsBF16, 0, 256, 256, 64, 2, 4, true),
+        HIPTK_HP_TILE_V8(TraitsBF16, 1, 128, 128, 64, 2, 4, true),
         HIPTK_H_TILE_V8(TraitsBF16, 2, 64, 64, 64, 2, 2, true),
-        HIPTK_H_TILE_V8(TraitsBF16, 5, 256, 128, 64, 4, 2, true),
-        HIPTK_H_TILE_V8(TraitsBF16, 6, 128, 256, 64, 2, 4, true),
+        HIPTK_HP_TILE_V8(TraitsBF16, 5, 256, 128, 64, 4, 2, true),
+        HIPTK_HP_TILE_V8(TraitsBF16, 6, 128, 256, 64, 2, 4, true),
         // 256 x 192: the 24 row vectors of a 192-row tile do not divide the workgroup, so only
         // the variants whose column operand is contiguous along k are built
-        HIPTK_H_ENTRY(TraitsBF16, 7, 256, 192, 64, 4, 2, true, true, 8, 8, true),
-        HIPTK_H_ENTRY(TraitsBF16, 7, 256, 192, 64, 4, 2, false, true, 8, 8, true),
-        // four wavefronts (one per SIMD, accumulators in AGPRs) with the register-level pipeline
+        HIPTK_HP_ENTRY(TraitsBF16, 7, 256, 192, 64, 4, 2, true, true, 8, 8, true),
+        HIPTK_HP_ENTRY(TraitsBF16, 7, 256, 192, 64, 4, 2, false, true, 8, 8, true),
+        // 256 x 256 on four wavefronts (one per SIMD, wave tile 128 x 128, accumulators in AGPRs)
         HIPTK_HP_TILE_V8(TraitsBF16, 8, 256, 256, 64, 2, 2, true),
-        HIPTK_HP_ENTRY(TraitsBF16, 9, 256, 192, 64, 2, 2, true, true, 8, 8, true),
-        HIPTK_HP_ENTRY(TraitsBF16, 9, 256, 192, 64, 2, 2, false, true, 8, 8, true),
     };
 
     const KernelEntry* entries_bf16_aff(int* count)

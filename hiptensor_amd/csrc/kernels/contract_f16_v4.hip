@@ -6,7 +6,7 @@ namespace hiptk
 {
     static const KernelEntry k_entries[] = {
         HIPTK_H_TILE_VV(TraitsF16, 0, 256, 256, 64, 2, 4, 4, false),
-        HIPTK_H_TILE_VV(TraitsF16, 1, 128, 128, 64, 2, 4, 4, false),
+        HIPTK_HP_TILE_VV(TraitsF16, 1, 128, 128, 64, 2, 4, 4, false),
         HIPTK_H_TILE_VV(TraitsF16, 2, 64, 64, 64, 2, 2, 4, false),
     };
 

@@ -6,7 +6,7 @@
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
-        HIPTK_H_TILE_VV(TraitsF32AsF16, 0, 128, 128, 64, 2, 4, 4, false),
+        HIPTK_HP_TILE_VV(TraitsF32AsF16, 0, 128, 128, 64, 2, 4, 4, false),
         HIPTK_H_TILE_VV(TraitsF32AsF16, 1, 64, 64, 64, 2, 2, 4, false),
         HIPTK_H_TILE_V1V(TraitsF32AsF16, 2, 128, 128, 32, 2, 2, 4),
         HIPTK_H_TILE_V1V(TraitsF32AsF16, 3, 64, 64, 32, 2, 2, 4),

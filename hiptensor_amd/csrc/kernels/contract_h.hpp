@@ -960,7 +960,7 @@ namespace hiptk
     {                                                                                       \
         TR::CLS, ID, XKF, YKF, XV, YV, KAFF, BP, BQ, BK, WP *WQ * 64,                       \
             hiptk::lds_bytes_h<BP, BQ, BK, XKF, YKF>(),                                     \
-            #TR "_" #BP "x" #BQ "x" #BK "_x" #XKF #XV "_y" #YKF #YV "_kaff" #KAFF "_pipe",  \
+            #TR "_" #BP "x" #BQ "x" #BK "_x" #XKF #XV "_y" #YKF #YV "_kaff" #KAFF "_pipe" #WP "x" #WQ, \
             &hiptk::launch_h<hiptk::TR, BP, BQ, BK, WP, WQ, XKF, YKF, XV, YV, KAFF, true>   \
     }
 
@@ -971,11 +971,12 @@ namespace hiptk
         HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, V, V, KAFF),    \
         HIPTK_H_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, V, V, KAFF)
 #define HIPTK_H_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ, KAFF) HIPTK_H_TILE_VV(TR, ID, BP, BQ, BK, WP, WQ, 8, KAFF)
-#define HIPTK_HP_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ, KAFF)                      \
-    HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, 8, 8, KAFF),         \
-        HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, 8, 8, KAFF),    \
-        HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, 8, 8, KAFF),    \
-        HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, 8, 8, KAFF)
+#define HIPTK_HP_TILE_VV(TR, ID, BP, BQ, BK, WP, WQ, V, KAFF)                   \
+    HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, true, V, V, KAFF),         \
+        HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, true, false, V, V, KAFF),    \
+        HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, true, V, V, KAFF),    \
+        HIPTK_HP_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, false, false, V, V, KAFF)
+#define HIPTK_HP_TILE_V8(TR, ID, BP, BQ, BK, WP, WQ, KAFF) HIPTK_HP_TILE_VV(TR, ID, BP, BQ, BK, WP, WQ, 8, KAFF)
 
 // Combinations in which at least one operand is a scalar gather (always staged k-fast).
 #define HIPTK_H_TILE_V1V(TR, ID, BP, BQ, BK, WP, WQ, V)                     \
