@@ -643,7 +643,8 @@ namespace hiptk
         typedef typename Tr::out_t out_t;
         out_t*       Dp = (out_t*)a.D;
         const out_t* Cp = (const out_t*)a.C;
-        if constexpr(sizeof(out_t) == 2 && WTQ >= 128) // (measured: a gain only for the wide wave tiles)
+        // (measured: a gain only for the wide wave tiles; and the staging has to fit)
+        if constexpr(sizeof(out_t) == 2 && WTQ >= 128 && 2 * WTQ * 36 * 2 * WP * WQ <= 2 * STAGE * 2)
         if(a.cd_vec == 8 && !a.bilinear)
         {
             // Scale with D contiguous along q in runs of 8.  The results are converted to their
