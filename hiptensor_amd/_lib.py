@@ -45,6 +45,16 @@ class PlanInfo(C.Structure):
     ]
 
 
+class PermutationInfo(C.Structure):
+    _fields_ = [
+        ("fused_rank", C.c_int32), ("extent", C.c_int32 * 6),
+        ("a_stride", C.c_int32 * 6), ("b_stride", C.c_int32 * 6),
+        ("kernel", C.c_int32), ("mode_i", C.c_int32), ("mode_j", C.c_int32),
+        ("tile", C.c_int32), ("vec_r", C.c_int32), ("vec_w", C.c_int32),
+        ("empty", C.c_int32), ("kernel_name", C.c_char * 96),
+    ]
+
+
 LOGGER_CALLBACK = C.CFUNCTYPE(None, C.c_int32, C.c_char_p, C.c_char_p)
 
 _SIGS = {
@@ -66,6 +76,8 @@ _SIGS = {
     "hiptensorAmdInitContractionPlan": (C.c_int, [vp, C.POINTER(vp), vp, vp, C.c_uint64]),
     "hiptensorAmdDestroyContractionPlan": (C.c_int, [vp]),
     "hiptensorAmdContraction": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, C.c_uint64, vp]),
+    "hiptensorAmdPermutation": (C.c_int, [vp, vp, vp, vp, i32p, vp, vp, i32p, C.c_int, vp]),
+    "hiptensorAmdPermutationInfo": (C.c_int, [vp, i32p, vp, i32p, vp, vp, C.POINTER(PermutationInfo)]),
     "hiptensorAmdLoggerSetCallback": (C.c_int, [LOGGER_CALLBACK]),
     "hiptensorAmdLoggerOpenFile": (C.c_int, [C.c_char_p]),
     "hiptensorAmdLoggerSetLevel": (C.c_int, [C.c_int]),

@@ -1,4 +1,4 @@
-"""Python mirror of the hipTensor 1.4 contraction API.
+"""Python mirror of the hipTensor 1.4 contraction and permutation API.
 
 Function names, argument order and status codes are those of
 library/include/hiptensor/hiptensor.hpp:41-228 in the reference; every call goes
@@ -166,6 +166,31 @@ def hiptensorContraction(handle, plan, alpha, A, B, beta, C_, D, workspace, work
     return lib.hiptensorAmdContraction(
         handle, plan, ap, _vp(A), _vp(B), bp, _vp(C_), _vp(D), _vp(workspace), int(workspaceSize), _vp(stream)
     )
+
+
+def hiptensorPermutation(handle, alpha, A, descA, modeA, B, descB, modeB, typeScalar, stream):
+    """alpha: ctypes scalar of typeScalar (or None); A, B: device addresses (int or None)."""
+    ap = C.cast(C.pointer(alpha), C.c_void_p) if alpha is not None else None
+    return lib.hiptensorAmdPermutation(
+        handle, ap, _vp(A), descA, _i32(modeA), _vp(B), descB, _i32(modeB), int(typeScalar), _vp(stream)
+    )
+
+
+# kernel ids of the permutation path (HIPTK_PERM_* in include/hiptk_kernels.h)
+PERM_COPY, PERM_TILED, PERM_ROWS, PERM_GATHER = 0, 1, 2, 3
+
+
+def permutationInfo(descA, modeA, descB, modeB, A=0, B=0):
+    """What hiptensorPermutation would launch (no device needed): (status, dict)."""
+    info = _lib.PermutationInfo()
+    st = lib.hiptensorAmdPermutationInfo(descA, _i32(modeA), descB, _i32(modeB), _vp(A), _vp(B), C.byref(info))
+    if st != 0:
+        return st, None
+    out = {name: getattr(info, name) for name, _ in _lib.PermutationInfo._fields_}
+    for k in ("extent", "a_stride", "b_stride"):
+        out[k] = list(out[k])[: info.fused_rank]
+    out["kernel_name"] = info.kernel_name.decode()
+    return st, out
 
 
 def _vp(x):

@@ -11,6 +11,14 @@ namespace hipta
 {
     hiptensorStatus_t createHostOnlyHandle(hiptensorHandle_t** handle);
     const PlanState*  planState(const hiptensorContractionPlan_t* plan);
+    hiptensorStatus_t planPermutation(const hiptensorTensorDescriptor_t* descA,
+                                      const int32_t                      modeA[],
+                                      const hiptensorTensorDescriptor_t* descB,
+                                      const int32_t                      modeB[],
+                                      const void*                        A,
+                                      const void*                        B,
+                                      hiptk_permute_t&                   out,
+                                      bool&                              empty);
 }
 
 namespace
@@ -200,6 +208,66 @@ extern "C" int hiptensorAmdContraction(const void* handle,
                                      workspace,
                                      workspaceSize,
                                      (hipStream_t)stream);
+}
+
+extern "C" int hiptensorAmdPermutation(const void*    handle,
+                                       const void*    alpha,
+                                       const void*    A,
+                                       const void*    descA,
+                                       const int32_t* modeA,
+                                       void*          B,
+                                       const void*    descB,
+                                       const int32_t* modeB,
+                                       int            typeScalar,
+                                       void*          stream)
+{
+    return (int)hiptensorPermutation((const hiptensorHandle_t*)handle,
+                                     alpha,
+                                     A,
+                                     (const hiptensorTensorDescriptor_t*)descA,
+                                     modeA,
+                                     B,
+                                     (const hiptensorTensorDescriptor_t*)descB,
+                                     modeB,
+                                     (hipDataType)typeScalar,
+                                     (hipStream_t)stream);
+}
+
+extern "C" int hiptensorAmdPermutationInfo(const void*                    descA,
+                                           const int32_t*                 modeA,
+                                           const void*                    descB,
+                                           const int32_t*                 modeB,
+                                           const void*                    A,
+                                           const void*                    B,
+                                           hiptensorAmdPermutationInfo_t* out)
+{
+    if(!descA || !modeA || !descB || !modeB || !out)
+        return (int)HIPTENSOR_STATUS_NOT_INITIALIZED;
+    const auto* dA = (const hiptensorTensorDescriptor_t*)descA;
+    const auto* dB = (const hiptensorTensorDescriptor_t*)descB;
+    std::memset(out, 0, sizeof(*out));
+    hiptk_permute_t p;
+    bool            empty = false;
+    auto            st    = hipta::planPermutation(dA, modeA, dB, modeB, A, B, p, empty);
+    if(st != HIPTENSOR_STATUS_SUCCESS)
+        return (int)st;
+    out->fused_rank = p.rank;
+    for(int d = 0; d < 6; ++d)
+    {
+        out->extent[d]   = p.extent[d];
+        out->a_stride[d] = p.a_stride[d];
+        out->b_stride[d] = p.b_stride[d];
+    }
+    out->kernel = p.kernel;
+    out->mode_i = p.mode_i;
+    out->mode_j = p.mode_j;
+    out->tile   = p.tile;
+    out->vec_r  = p.vec_r;
+    out->vec_w  = p.vec_w;
+    out->empty  = empty ? 1 : 0;
+    if(!empty)
+        std::strncpy(out->kernel_name, hiptk_permute_kernel_name(&p), sizeof(out->kernel_name) - 1);
+    return 0;
 }
 
 extern "C" int hiptensorAmdLoggerSetCallback(hiptensorAmdLoggerCallback_t callback)

@@ -1,0 +1,218 @@
+#include "permute_plan.hpp"
+
+#include <algorithm>
+#include <cstring>
+
+namespace hipta
+{
+    namespace
+    {
+        struct Tile
+        {
+            int ti, tj;
+        };
+        // the kernel layer's tile shapes (elements): square, long along i, long along j
+        constexpr Tile TILES4[3] = {{64, 64}, {256, 16}, {16, 256}};
+        constexpr Tile TILES2[3] = {{128, 128}, {512, 32}, {32, 512}};
+
+        bool alignedTo(const void* p, int64_t bytes)
+        {
+            return (reinterpret_cast<uintptr_t>(p) % (uintptr_t)bytes) == 0;
+        }
+
+        // Largest vector (elements) not above cap that divides `extent` and every stride in
+        // `others`, and that the address is aligned for.
+        int pickVec(int elem_bytes, int cap, int64_t extent, const std::vector<int64_t>& others, const void* p, bool copy)
+        {
+            const int cands4[] = {4, 2, 1}, cands2[] = {8, 2, 1}, candsCopy2[] = {8, 4, 2, 1};
+            const int* c;
+            int        n;
+            if(elem_bytes == 4)
+                c = cands4, n = 3;
+            else if(copy)
+                c = candsCopy2, n = 4;
+            else
+                c = cands2, n = 3;
+            for(int k = 0; k < n; ++k)
+            {
+                const int v = c[k];
+                if(v > cap || extent % v != 0 || !alignedTo(p, (int64_t)v * elem_bytes))
+                    continue;
+                bool ok = true;
+                for(int64_t s : others)
+                    ok = ok && (s % v == 0);
+                if(ok)
+                    return v;
+            }
+            return 1;
+        }
+
+        // Share of a tile grid's lanes that fall inside the extents.
+        double coverage(int64_t e, int t)
+        {
+            const int64_t tiles = (e + t - 1) / t;
+            return (double)e / (double)(tiles * t);
+        }
+
+        int pickTile(int elem_bytes, int64_t e_i, int64_t e_j, const int order[3])
+        {
+            const Tile* ts   = elem_bytes == 4 ? TILES4 : TILES2;
+            int         best = order[0];
+            double      bc   = -1.0;
+            for(int k = 0; k < 3; ++k)
+            {
+                const int    t = order[k];
+                const double c = coverage(e_i, ts[t].ti) * coverage(e_j, ts[t].tj);
+                if(c > bc + 1e-9)
+                    bc = c, best = t;
+            }
+            return best;
+        }
+    }
+
+    PermuteStatus plan_permutation(const PermuteIn& in, const PermuteTuning& tune, hiptk_permute_t& out)
+    {
+        std::memset(&out, 0, sizeof(out));
+        const size_t rank = in.lenA.size();
+        if(in.lenB.size() != rank || in.modeA.size() != rank || in.modeB.size() != rank)
+            return PermuteStatus::BAD_RANK;
+
+        // position of each B mode in A; every label once on both sides, lengths agree
+        std::vector<int> posInA(rank, -1);
+        std::vector<bool> used(rank, false);
+        for(size_t k = 0; k < rank; ++k)
+        {
+            for(size_t i = 0; i < rank; ++i)
+                if(in.modeA[i] == in.modeB[k] && !used[i])
+                {
+                    posInA[k] = (int)i;
+                    break;
+                }
+            if(posInA[k] < 0 || in.lenB[k] != in.lenA[posInA[k]])
+                return PermuteStatus::BAD_MODES;
+            used[posInA[k]] = true;
+        }
+        int64_t count = 1;
+        for(size_t i = 0; i < rank; ++i)
+        {
+            if(in.lenA[i] < 0)
+                return PermuteStatus::BAD_MODES;
+            if(in.lenA[i] == 0)
+                return PermuteStatus::EMPTY;
+            count *= in.lenA[i];
+            if(count >= (int64_t(1) << 31))
+                return PermuteStatus::TOO_LARGE;
+        }
+
+        // packed strides, first listed mode fastest; B's stride carried to A's order
+        std::vector<int64_t> bInA(rank, 0);
+        {
+            int64_t s = 1;
+            for(size_t k = 0; k < rank; ++k)
+            {
+                bInA[posInA[k]] = s;
+                s *= in.lenB[k];
+            }
+        }
+        // drop extent-1 modes, fuse neighbours of A that are neighbours in B in the same order
+        std::vector<int64_t> ext, as, bs;
+        {
+            int64_t s = 1;
+            for(size_t i = 0; i < rank; ++i)
+            {
+                const int64_t e = in.lenA[i];
+                if(e != 1)
+                {
+                    if(!ext.empty() && bInA[i] == bs.back() * ext.back())
+                        ext.back() *= e;
+                    else
+                    {
+                        ext.push_back(e);
+                        as.push_back(s);
+                        bs.push_back(bInA[i]);
+                    }
+                }
+                s *= e;
+            }
+            if(ext.empty())
+            {
+                ext.push_back(1);
+                as.push_back(1);
+                bs.push_back(1);
+            }
+        }
+        const int r    = (int)ext.size();
+        out.elem_bytes = in.elem_bytes;
+        out.rank       = r;
+        for(int d = 0; d < r; ++d)
+        {
+            out.extent[d]   = (int32_t)ext[d];
+            out.a_stride[d] = (int32_t)as[d];
+            out.b_stride[d] = (int32_t)bs[d];
+        }
+        out.vec_r = out.vec_w = 1;
+        const int cap         = std::max(1, tune.max_vec);
+
+        if(r == 1)
+        {
+            out.kernel = HIPTK_PERM_COPY;
+            const int v = std::min(pickVec(in.elem_bytes, cap, ext[0], {}, in.A, true),
+                                   pickVec(in.elem_bytes, cap, ext[0], {}, in.B, true));
+            out.vec_r = out.vec_w = v;
+            return PermuteStatus::OK;
+        }
+
+        int jB = 0; // B's fastest mode
+        for(int d = 0; d < r; ++d)
+            if(bs[d] == 1)
+                jB = d;
+
+        // layout-admissible kernels: TILED needs differing fastest modes, ROWS a shared one
+        const bool shared = jB == 0;
+        int        kernel;
+        if(tune.kernel == HIPTK_PERM_GATHER)
+            kernel = HIPTK_PERM_GATHER;
+        else if(tune.kernel == HIPTK_PERM_TILED || tune.kernel == HIPTK_PERM_ROWS)
+            kernel = shared ? HIPTK_PERM_ROWS : HIPTK_PERM_TILED;
+        else if(count <= 16384)
+            kernel = HIPTK_PERM_GATHER; // a launch's worth of latency either way
+        else if(shared)
+            kernel = ext[0] >= 16 ? HIPTK_PERM_ROWS : HIPTK_PERM_GATHER;
+        else
+            kernel = (ext[0] >= 16 && ext[jB] >= 16) ? HIPTK_PERM_TILED : HIPTK_PERM_GATHER;
+        out.kernel = kernel;
+        if(kernel == HIPTK_PERM_GATHER)
+            return PermuteStatus::OK;
+
+        out.mode_i = 0;
+        std::vector<int64_t> aOthers(as.begin() + 1, as.end());
+        const int            vr = pickVec(in.elem_bytes, cap, ext[0], aOthers, in.A, false);
+        if(kernel == HIPTK_PERM_TILED)
+        {
+            out.mode_j = jB;
+            std::vector<int64_t> bOthers;
+            for(int d = 0; d < r; ++d)
+                if(d != jB)
+                    bOthers.push_back(bs[d]);
+            out.vec_r         = vr;
+            out.vec_w         = pickVec(in.elem_bytes, cap, ext[jB], bOthers, in.B, false);
+            const int order[] = {0, 1, 2};
+            out.tile          = tune.tile >= 0 && tune.tile <= 2 ? tune.tile : pickTile(in.elem_bytes, ext[0], ext[jB], order);
+        }
+        else
+        {
+            // second tile mode: the one B walks next, so that stores sweep B in order
+            int mj = 1;
+            for(int d = 1; d < r; ++d)
+                if(bs[d] < bs[mj])
+                    mj = d;
+            out.mode_j = mj;
+            std::vector<int64_t> bOthers(bs.begin() + 1, bs.end());
+            const int            vw = pickVec(in.elem_bytes, cap, ext[0], bOthers, in.B, false);
+            out.vec_r = out.vec_w = std::min(vr, vw);
+            const int order[]     = {1, 0, 2};
+            out.tile              = tune.tile >= 0 && tune.tile <= 2 ? tune.tile : pickTile(in.elem_bytes, ext[0], ext[mj], order);
+        }
+        return PermuteStatus::OK;
+    }
+}

@@ -1,0 +1,502 @@
+// Tensor permutation kernels, B[perm(index)] = opB(alpha * opA(A[index])), and their launcher.
+//
+// The work is a stream of bytes through HBM, so the kernels are built around memory
+// coalescing, not arithmetic:
+//   * COPY    one fused mode left: a scaled vector copy.
+//   * TILED   A's fastest mode i and B's fastest mode j differ.  A workgroup moves a
+//             two-dimensional tile of those two modes: it reads rows along i (contiguous in A),
+//             applies the element operation, parks the tile in LDS, and writes it out along j
+//             (contiguous in B).  The other modes only choose the tile's base offsets, once per
+//             workgroup on the scalar unit.
+//   * ROWS    A and B share the fastest mode: runs of it are contiguous on both sides and go
+//             from registers straight back to memory, no LDS.
+//   * GATHER  one thread per element of B; covers tiny tensors and awkward extents.
+// Element operation per Composable Kernel's UnaryCombinedOp<Aop, Scale, Bop>
+// (ck/tensor_operation/gpu/element/combined_element_wise_operation.hpp:14-32): every step is
+// rounded to the element type; for f16 alpha is rounded to half first
+// (unary_element_wise_operation.hpp:647-651).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+
+#include "hiptk_kernels.h"
+
+namespace hiptk
+{
+    namespace
+    {
+        constexpr int PERM_THREADS = 256;
+        constexpr int PERM_BATCH   = HIPTK_PERM_MAX_RANK - 2;
+
+        struct PArgs
+        {
+            const void* A;
+            void*       B;
+            uint32_t    e_i, e_j; // extents of the two tile modes
+            uint32_t    a_j; // A stride of mode j (mode i has stride 1 in A)
+            uint32_t    b_i, b_j; // B strides (TILED: b_j == 1, ROWS: b_i == 1)
+            uint32_t    nt_i, nt_j; // tiles along i and j
+            int32_t     nb; // modes that only pick the tile's base
+            uint32_t    bext[PERM_BATCH], ba[PERM_BATCH], bb[PERM_BATCH];
+            float       alpha;
+            int32_t     op_a, op_b;
+        };
+
+        struct GArgs
+        {
+            const void* A;
+            void*       B;
+            uint32_t    n;
+            int32_t     rank;
+            uint32_t    ext[HIPTK_PERM_MAX_RANK]; // in B's order, fastest first
+            uint32_t    astr[HIPTK_PERM_MAX_RANK];
+            float       alpha;
+            int32_t     op_a, op_b;
+        };
+
+        template <typename T, int V>
+        struct alignas(sizeof(T) * V) Vec
+        {
+            T v[V];
+        };
+
+        template <typename T>
+        __device__ inline T element_op(T x, T alpha, int op_a, int op_b)
+        {
+            T y = x;
+            if(op_a)
+                y = y * y;
+            y = alpha * y;
+            if(op_b)
+                y = y * y;
+            return y;
+        }
+
+        template <typename T, int TI, int TJ, int VR, int VW, bool TRANSPOSE>
+        __global__ __launch_bounds__(PERM_THREADS) void permute_tile_kernel(PArgs a)
+        {
+            constexpr int NT    = PERM_THREADS;
+            constexpr int PITCH = TI + 1; // odd pitch: column reads spread over the banks
+            constexpr int VPR   = TI / VR; // vectors per tile row
+            constexpr int NRV   = VPR * TJ / NT; // vectors per thread, read side
+            static_assert(TI % VR == 0 && (VPR * TJ) % NT == 0 && NRV >= 1, "read shape");
+            __shared__ T tile[TRANSPOSE ? TJ * PITCH : 1];
+
+            const T* __restrict__ A = static_cast<const T*>(a.A);
+            T* __restrict__ B       = static_cast<T*>(a.B);
+            const int tid           = threadIdx.x;
+
+            uint32_t       blk = blockIdx.x;
+            const uint32_t ti  = blk % a.nt_i;
+            blk /= a.nt_i;
+            const uint32_t tj = blk % a.nt_j;
+            blk /= a.nt_j;
+            uint32_t aoff = 0, boff = 0;
+            for(int d = 0; d < a.nb; ++d)
+            {
+                const uint32_t c = blk % a.bext[d];
+                blk /= a.bext[d];
+                aoff += c * a.ba[d];
+                boff += c * a.bb[d];
+            }
+            const uint32_t i0 = ti * TI, j0 = tj * TJ;
+            aoff += i0 + j0 * a.a_j;
+            boff += i0 * a.b_i + j0 * a.b_j;
+
+            const T alpha = static_cast<T>(a.alpha);
+
+            Vec<T, VR> r[NRV];
+#pragma unroll
+            for(int k = 0; k < NRV; ++k)
+            {
+                const uint32_t v = tid + k * NT, iv = v % VPR, j = v / VPR;
+                const bool     ok = (i0 + iv * VR < a.e_i) && (j0 + j < a.e_j);
+                r[k]              = Vec<T, VR>{};
+                if(ok)
+                    r[k] = *reinterpret_cast<const Vec<T, VR>*>(A + aoff + iv * VR + j * a.a_j);
+            }
+#pragma unroll
+            for(int k = 0; k < NRV; ++k)
+            {
+                const uint32_t v = tid + k * NT, iv = v % VPR, j = v / VPR;
+#pragma unroll
+                for(int e = 0; e < VR; ++e)
+                    r[k].v[e] = element_op(r[k].v[e], alpha, a.op_a, a.op_b);
+                if constexpr(TRANSPOSE)
+                {
+#pragma unroll
+                    for(int e = 0; e < VR; ++e)
+                        tile[j * PITCH + iv * VR + e] = r[k].v[e];
+                }
+                else
+                {
+                    const bool ok = (i0 + iv * VR < a.e_i) && (j0 + j < a.e_j);
+                    if(ok)
+                        *reinterpret_cast<Vec<T, VR>*>(B + boff + iv * VR + j * a.b_j) = r[k];
+                }
+            }
+            if constexpr(TRANSPOSE)
+            {
+                constexpr int VPC = TJ / VW; // vectors per tile column
+                constexpr int NWV = VPC * TI / NT;
+                static_assert(TJ % VW == 0 && (VPC * TI) % NT == 0 && NWV >= 1, "write shape");
+                __syncthreads();
+#pragma unroll
+                for(int k = 0; k < NWV; ++k)
+                {
+                    const uint32_t v = tid + k * NT, jv = v % VPC, i = v / VPC;
+                    const bool     ok = (j0 + jv * VW < a.e_j) && (i0 + i < a.e_i);
+                    Vec<T, VW>     o;
+#pragma unroll
+                    for(int e = 0; e < VW; ++e)
+                        o.v[e] = tile[(jv * VW + e) * PITCH + i];
+                    if(ok)
+                        *reinterpret_cast<Vec<T, VW>*>(B + boff + jv * VW + i * a.b_i) = o;
+                }
+            }
+        }
+
+        template <typename T, int V>
+        __global__ __launch_bounds__(PERM_THREADS) void permute_copy_kernel(
+            const void* Av, void* Bv, uint32_t nvec, float alphaF, int op_a, int op_b)
+        {
+            constexpr int U = 4;
+            const auto*   A = static_cast<const Vec<T, V>*>(Av);
+            auto*         B = static_cast<Vec<T, V>*>(Bv);
+            const T       alpha = static_cast<T>(alphaF);
+            const uint32_t base = blockIdx.x * (PERM_THREADS * U) + threadIdx.x;
+            Vec<T, V>      r[U];
+#pragma unroll
+            for(int u = 0; u < U; ++u)
+            {
+                const uint32_t idx = base + u * PERM_THREADS;
+                r[u]               = Vec<T, V>{};
+                if(idx < nvec)
+                    r[u] = A[idx];
+            }
+#pragma unroll
+            for(int u = 0; u < U; ++u)
+            {
+                const uint32_t idx = base + u * PERM_THREADS;
+#pragma unroll
+                for(int e = 0; e < V; ++e)
+                    r[u].v[e] = element_op(r[u].v[e], alpha, op_a, op_b);
+                if(idx < nvec)
+                    B[idx] = r[u];
+            }
+        }
+
+        template <typename T>
+        __global__ __launch_bounds__(PERM_THREADS) void permute_gather_kernel(GArgs g)
+        {
+            const uint32_t idx = blockIdx.x * PERM_THREADS + threadIdx.x;
+            if(idx >= g.n)
+                return;
+            uint32_t rem = idx, aoff = 0;
+            for(int d = 0; d < g.rank; ++d)
+            {
+                const uint32_t c = rem % g.ext[d];
+                rem /= g.ext[d];
+                aoff += c * g.astr[d];
+            }
+            const T alpha               = static_cast<T>(g.alpha);
+            static_cast<T*>(g.B)[idx] = element_op(static_cast<const T*>(g.A)[aoff], alpha, g.op_a, g.op_b);
+        }
+
+        // ---------------------------------------------------------------- host side
+
+        struct TileShape
+        {
+            int ti, tj;
+        };
+        // element tiles per element size: square, long along i, long along j
+        constexpr TileShape TILES4[3] = {{64, 64}, {256, 16}, {16, 256}};
+        constexpr TileShape TILES2[3] = {{128, 128}, {512, 32}, {32, 512}};
+
+        template <typename T, int TI, int TJ, int VR, int VW, bool TR>
+        int launch_tile(const PArgs& a, uint32_t grid, hipStream_t s)
+        {
+            hipLaunchKernelGGL((permute_tile_kernel<T, TI, TJ, VR, VW, TR>), dim3(grid), dim3(PERM_THREADS), 0, s, a);
+            return (int)hipGetLastError();
+        }
+
+        template <typename T, int TI, int TJ, int VMAX>
+        int launch_tile_vec(bool transpose, int vr, int vw, const PArgs& a, uint32_t grid, hipStream_t s)
+        {
+#define HIPTK_PERM_CASE(R, W)                                           \
+    if(vr == R && vw == W)                                              \
+        return transpose ? launch_tile<T, TI, TJ, R, W, true>(a, grid, s) \
+                         : (R == W ? launch_tile<T, TI, TJ, R, R, false>(a, grid, s) : -1);
+            HIPTK_PERM_CASE(1, 1)
+            HIPTK_PERM_CASE(1, 2)
+            HIPTK_PERM_CASE(1, VMAX)
+            HIPTK_PERM_CASE(2, 1)
+            HIPTK_PERM_CASE(2, 2)
+            HIPTK_PERM_CASE(2, VMAX)
+            HIPTK_PERM_CASE(VMAX, 1)
+            HIPTK_PERM_CASE(VMAX, 2)
+            HIPTK_PERM_CASE(VMAX, VMAX)
+#undef HIPTK_PERM_CASE
+            return -1;
+        }
+
+        template <typename T, int VMAX>
+        int launch_tile_shape(int tile, bool transpose, int vr, int vw, const PArgs& a, uint32_t grid, hipStream_t s)
+        {
+            constexpr const TileShape* TS = sizeof(T) == 4 ? TILES4 : TILES2;
+            switch(tile)
+            {
+            case 0: return launch_tile_vec<T, TS[0].ti, TS[0].tj, VMAX>(transpose, vr, vw, a, grid, s);
+            case 1: return launch_tile_vec<T, TS[1].ti, TS[1].tj, VMAX>(transpose, vr, vw, a, grid, s);
+            case 2: return launch_tile_vec<T, TS[2].ti, TS[2].tj, VMAX>(transpose, vr, vw, a, grid, s);
+            default: return -1;
+            }
+        }
+
+        template <typename T>
+        int launch_copy(int vec, const void* A, void* B, uint32_t n, float alpha, int oa, int ob, hipStream_t s)
+        {
+            const uint32_t nvec = n / vec;
+            const uint32_t grid = (nvec + PERM_THREADS * 4 - 1) / (PERM_THREADS * 4);
+#define HIPTK_COPY_CASE(V)                                                                                           \
+    if(vec == V)                                                                                                     \
+    {                                                                                                                \
+        hipLaunchKernelGGL((permute_copy_kernel<T, V>), dim3(grid), dim3(PERM_THREADS), 0, s, A, B, nvec, alpha, oa, ob); \
+        return (int)hipGetLastError();                                                                               \
+    }
+            HIPTK_COPY_CASE(1)
+            HIPTK_COPY_CASE(2)
+            HIPTK_COPY_CASE(4)
+            if constexpr(sizeof(T) == 2)
+            {
+                HIPTK_COPY_CASE(8)
+            }
+#undef HIPTK_COPY_CASE
+            return -1;
+        }
+
+        bool vec_allowed(int elem_bytes, int v)
+        {
+            return v == 1 || v == 2 || (elem_bytes == 4 ? v == 4 : v == 8);
+        }
+        bool copy_vec_allowed(int elem_bytes, int v)
+        {
+            return v == 1 || v == 2 || v == 4 || (elem_bytes == 2 && v == 8);
+        }
+
+        bool aligned(const void* p, int bytes)
+        {
+            return (reinterpret_cast<uintptr_t>(p) % (uintptr_t)bytes) == 0;
+        }
+
+        // Shape checks shared by the name query and the launcher.
+        bool well_formed(const hiptk_permute_t* p, int64_t* count)
+        {
+            if(!p || (p->elem_bytes != 2 && p->elem_bytes != 4) || p->rank < 1 || p->rank > HIPTK_PERM_MAX_RANK)
+                return false;
+            if((p->op_a | p->op_b) & ~1)
+                return false;
+            int64_t n = 1;
+            for(int d = 0; d < p->rank; ++d)
+            {
+                if(p->extent[d] < 1 || p->a_stride[d] < 1 || p->b_stride[d] < 1)
+                    return false;
+                n *= p->extent[d];
+                if(n >= (int64_t(1) << 31))
+                    return false;
+            }
+            // A is packed in the order given
+            int64_t s = 1;
+            for(int d = 0; d < p->rank; ++d)
+            {
+                if(p->a_stride[d] != s)
+                    return false;
+                s *= p->extent[d];
+            }
+            // B is packed in some order of the same modes
+            int order[HIPTK_PERM_MAX_RANK];
+            for(int d = 0; d < p->rank; ++d)
+                order[d] = d;
+            std::sort(order, order + p->rank, [p](int x, int y) {
+                return p->b_stride[x] != p->b_stride[y] ? p->b_stride[x] < p->b_stride[y] : x < y;
+            });
+            s = 1;
+            for(int d = 0; d < p->rank; ++d)
+            {
+                if(p->b_stride[order[d]] != s)
+                    return false;
+                s *= p->extent[order[d]];
+            }
+            *count = n;
+            return true;
+        }
+
+        const char* type_tag(int elem_bytes)
+        {
+            return elem_bytes == 4 ? "f32" : "f16";
+        }
+    }
+}
+
+extern "C" const char* hiptk_permute_kernel_name(const hiptk_permute_t* p)
+{
+    using namespace hiptk;
+    static thread_local char name[96];
+    name[0]   = 0;
+    int64_t n = 0;
+    if(!well_formed(p, &n))
+        return name;
+    switch(p->kernel)
+    {
+    case HIPTK_PERM_COPY:
+        if(p->rank == 1 && copy_vec_allowed(p->elem_bytes, p->vec_r))
+            snprintf(name, sizeof(name), "permute_copy_%s_v%d", type_tag(p->elem_bytes), p->vec_r);
+        break;
+    case HIPTK_PERM_TILED:
+    case HIPTK_PERM_ROWS:
+    {
+        if(p->tile < 0 || p->tile > 2 || !vec_allowed(p->elem_bytes, p->vec_r) || !vec_allowed(p->elem_bytes, p->vec_w))
+            break;
+        if(p->kernel == HIPTK_PERM_ROWS && p->vec_r != p->vec_w)
+            break;
+        const TileShape t = (p->elem_bytes == 4 ? TILES4 : TILES2)[p->tile];
+        snprintf(name,
+                 sizeof(name),
+                 "permute_%s_%s_%dx%d_r%d_w%d",
+                 p->kernel == HIPTK_PERM_TILED ? "tiled" : "rows",
+                 type_tag(p->elem_bytes),
+                 t.ti,
+                 t.tj,
+                 p->vec_r,
+                 p->vec_w);
+        break;
+    }
+    case HIPTK_PERM_GATHER: snprintf(name, sizeof(name), "permute_gather_%s", type_tag(p->elem_bytes)); break;
+    default: break;
+    }
+    return name;
+}
+
+extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, void* stream, int* hip_error)
+{
+    using namespace hiptk;
+    if(hip_error)
+        *hip_error = 0;
+    int64_t n = 0;
+    if(!well_formed(p, &n) || !A || !B)
+        return HIPTK_ERR_ARG;
+    if(!aligned(A, p->elem_bytes) || !aligned(B, p->elem_bytes))
+        return HIPTK_ERR_ARG;
+    hipStream_t s  = static_cast<hipStream_t>(stream);
+    int         rc = -1;
+
+    if(p->kernel == HIPTK_PERM_COPY)
+    {
+        const int v = p->vec_r;
+        if(p->rank != 1 || !copy_vec_allowed(p->elem_bytes, v))
+            return HIPTK_ERR_NO_KERNEL;
+        if(n % v != 0 || !aligned(A, v * p->elem_bytes) || !aligned(B, v * p->elem_bytes))
+            return HIPTK_ERR_ARG;
+        rc = p->elem_bytes == 4 ? launch_copy<float>(v, A, B, (uint32_t)n, p->alpha, p->op_a, p->op_b, s)
+                                : launch_copy<_Float16>(v, A, B, (uint32_t)n, p->alpha, p->op_a, p->op_b, s);
+    }
+    else if(p->kernel == HIPTK_PERM_GATHER)
+    {
+        GArgs g;
+        memset(&g, 0, sizeof(g));
+        g.A     = A;
+        g.B     = B;
+        g.n     = (uint32_t)n;
+        g.rank  = p->rank;
+        g.alpha = p->alpha;
+        g.op_a  = p->op_a;
+        g.op_b  = p->op_b;
+        int order[HIPTK_PERM_MAX_RANK];
+        for(int d = 0; d < p->rank; ++d)
+            order[d] = d;
+        std::sort(order, order + p->rank, [p](int x, int y) {
+            return p->b_stride[x] != p->b_stride[y] ? p->b_stride[x] < p->b_stride[y] : x < y;
+        });
+        for(int d = 0; d < p->rank; ++d)
+        {
+            g.ext[d]  = (uint32_t)p->extent[order[d]];
+            g.astr[d] = (uint32_t)p->a_stride[order[d]];
+        }
+        const uint32_t grid = (uint32_t)((n + PERM_THREADS - 1) / PERM_THREADS);
+        if(p->elem_bytes == 4)
+            hipLaunchKernelGGL((permute_gather_kernel<float>), dim3(grid), dim3(PERM_THREADS), 0, s, g);
+        else
+            hipLaunchKernelGGL((permute_gather_kernel<_Float16>), dim3(grid), dim3(PERM_THREADS), 0, s, g);
+        rc = (int)hipGetLastError();
+    }
+    else if(p->kernel == HIPTK_PERM_TILED || p->kernel == HIPTK_PERM_ROWS)
+    {
+        const bool transpose = p->kernel == HIPTK_PERM_TILED;
+        const int  mi = p->mode_i, mj = p->mode_j;
+        if(p->rank < 2 || mi != 0 || mj < 1 || mj >= p->rank || p->tile < 0 || p->tile > 2)
+            return HIPTK_ERR_ARG;
+        if(!vec_allowed(p->elem_bytes, p->vec_r) || !vec_allowed(p->elem_bytes, p->vec_w))
+            return HIPTK_ERR_NO_KERNEL;
+        if(!transpose && p->vec_r != p->vec_w)
+            return HIPTK_ERR_NO_KERNEL;
+        // the layout each kernel assumes
+        if(transpose ? p->b_stride[mj] != 1 : p->b_stride[0] != 1)
+            return HIPTK_ERR_ARG;
+        // what the vector widths assume: whole vectors inside the extents, every other
+        // stride and both base pointers multiples of the vector
+        const int vr = p->vec_r, vw = p->vec_w;
+        if(p->extent[0] % vr != 0 || !aligned(A, vr * p->elem_bytes))
+            return HIPTK_ERR_ARG;
+        for(int d = 1; d < p->rank; ++d)
+            if(p->a_stride[d] % vr != 0)
+                return HIPTK_ERR_ARG;
+        const int wmode = transpose ? mj : 0; // the mode stores run along
+        if(p->extent[wmode] % vw != 0 || !aligned(B, vw * p->elem_bytes))
+            return HIPTK_ERR_ARG;
+        for(int d = 0; d < p->rank; ++d)
+            if(d != wmode && p->b_stride[d] % vw != 0)
+                return HIPTK_ERR_ARG;
+
+        const TileShape t = (p->elem_bytes == 4 ? TILES4 : TILES2)[p->tile];
+        PArgs           a;
+        memset(&a, 0, sizeof(a));
+        a.A     = A;
+        a.B     = B;
+        a.e_i   = (uint32_t)p->extent[0];
+        a.e_j   = (uint32_t)p->extent[mj];
+        a.a_j   = (uint32_t)p->a_stride[mj];
+        a.b_i   = (uint32_t)p->b_stride[0];
+        a.b_j   = (uint32_t)p->b_stride[mj];
+        a.nt_i  = (a.e_i + t.ti - 1) / t.ti;
+        a.nt_j  = (a.e_j + t.tj - 1) / t.tj;
+        a.alpha = p->alpha;
+        a.op_a  = p->op_a;
+        a.op_b  = p->op_b;
+        int64_t grid = (int64_t)a.nt_i * a.nt_j;
+        for(int d = 1; d < p->rank; ++d)
+        {
+            if(d == mj)
+                continue;
+            a.bext[a.nb] = (uint32_t)p->extent[d];
+            a.ba[a.nb]   = (uint32_t)p->a_stride[d];
+            a.bb[a.nb]   = (uint32_t)p->b_stride[d];
+            ++a.nb;
+            grid *= p->extent[d];
+        }
+        if(grid >= (int64_t(1) << 31))
+            return HIPTK_ERR_ARG;
+        rc = p->elem_bytes == 4 ? launch_tile_shape<float, 4>(p->tile, transpose, vr, vw, a, (uint32_t)grid, s)
+                                : launch_tile_shape<_Float16, 8>(p->tile, transpose, vr, vw, a, (uint32_t)grid, s);
+    }
+    else
+        return HIPTK_ERR_NO_KERNEL;
+
+    if(rc == -1)
+        return HIPTK_ERR_NO_KERNEL;
+    if(hip_error)
+        *hip_error = rc;
+    return rc == 0 ? HIPTK_OK : HIPTK_ERR_LAUNCH;
+}

@@ -1,4 +1,5 @@
-"""Benchmark / test workloads of the contraction path and their seeded inputs.
+"""Benchmark / test workloads of the contraction path (and of the permutation beside it)
+and their seeded inputs.
 
 A workload is a plain dict:
   dtype    "f16" | "bf16" | "f32" | "f64" | "c32" | "c64"
@@ -305,3 +306,58 @@ class Contraction:
         api.destroy("contraction", self.desc)
         for d in (self.dA, self.dB, self.dC, self.dD):
             api.destroy("tensor", d)
+
+
+# ---------------------------------------------------------------------------
+# Permutation workloads: B[modes permuted] = opB(alpha * opA(A)).
+# Both tensors are packed with the first listed mode fastest, the layout the reference's
+# permutation assumes (library/src/permutation/permutation_solution_impl.hpp:125-128).
+# ---------------------------------------------------------------------------
+
+def permutation(dtype, lens, perm, alpha=1.0, scalar=None, opA=api.HIPTENSOR_OP_IDENTITY,
+                opB=api.HIPTENSOR_OP_IDENTITY, name=""):
+    """`perm` as in the reference's test files ("Permuted Dims"): mode k of B is mode perm[k]
+    of A.  `scalar` is the type alpha is passed as ("f16" / "f32", default: the data type)."""
+    modesA = list(range(100, 100 + len(lens)))
+    return {
+        "kind": "permutation", "name": name or f"perm_{dtype}_{'x'.join(map(str, lens))}_{''.join(map(str, perm))}",
+        "dtype": dtype, "scalar": scalar or dtype, "alpha": float(alpha), "opA": int(opA), "opB": int(opB),
+        "perm": list(perm), "lensA": list(lens), "modesA": modesA,
+        "lensB": [lens[p] for p in perm], "modesB": [modesA[p] for p in perm],
+    }
+
+
+def permutation_input(w, seed=SEED_A):
+    """Packed host tensor A with the seeded values in [-1, 1)."""
+    n = int(np.prod(w["lensA"])) if w["lensA"] else 1
+    return gen_values(n, seed).astype(NP_STORE[w["dtype"]])
+
+
+def permutation_alpha(w):
+    """ctypes scalar holding alpha in the layout of the scalar type."""
+    if w["scalar"] == "f16":
+        return C.c_uint16(int(np.float16(w["alpha"]).view(np.uint16)))
+    return C.c_float(w["alpha"])
+
+
+class Permutation:
+    """Descriptors for one permutation workload, through the public API."""
+
+    def __init__(self, handle, w):
+        self.handle, self.w = handle, w
+        t = HIP_TYPE[w["dtype"]]
+        self.dA = api.check(api.hiptensorInitTensorDescriptor(handle, w["lensA"], None, t, w["opA"]), "descA")
+        self.dB = api.check(api.hiptensorInitTensorDescriptor(handle, w["lensB"], None, t, w["opB"]), "descB")
+        self.alpha = permutation_alpha(w)
+
+    def info(self, A=0, B=0):
+        return api.check(api.permutationInfo(self.dA, self.w["modesA"], self.dB, self.w["modesB"], A, B), "permutationInfo")
+
+    def run(self, A, B, stream=0):
+        """A, B: device addresses (ints)."""
+        return api.hiptensorPermutation(self.handle, self.alpha, A, self.dA, self.w["modesA"], B, self.dB,
+                                        self.w["modesB"], HIP_TYPE[self.w["scalar"]], stream or None)
+
+    def close(self):
+        api.destroy("tensor", self.dA)
+        api.destroy("tensor", self.dB)

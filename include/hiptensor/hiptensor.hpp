@@ -1,4 +1,4 @@
-// Public entry points of the contraction path.
+// Public entry points of the contraction path and of the tensor permutation beside it.
 //
 // Declarations are source-compatible with hipTensor 1.4's
 // library/include/hiptensor/hiptensor.hpp (line numbers cited per function), so a
@@ -7,8 +7,7 @@
 // std::vector members, exactly as in the reference; a flat extern "C" flavour of
 // the same calls lives in <hiptensor_amd.h>.
 //
-// hiptensorPermutation and hiptensorReduction (hiptensor.hpp:85-100, 230-300) are
-// not part of the contraction path and are not provided.
+// hiptensorReduction (hiptensor.hpp:230-300) is not part of this path and is not provided.
 #ifndef HIPTENSOR_API_HPP
 #define HIPTENSOR_API_HPP
 
@@ -35,6 +34,23 @@ hiptensorStatus_t hiptensorInitTensorDescriptor(const hiptensorHandle_t*     han
 
 // Name of a status code.                                           [hiptensor.hpp:71]
 const char* hiptensorGetErrorString(const hiptensorStatus_t error);
+
+// B[perm(index)] = opB(alpha * opA(A[index])) for f16 or f32 tensors of 2 to 6 modes; modeB is
+// a reordering of modeA.  As in the reference, both tensors are taken as packed with their
+// FIRST listed mode fastest, whatever strides the descriptors hold, and the unary operator
+// HIPTENSOR_OP_SQRT squares its argument.  alpha is a host pointer to one scalar of
+// typeScalar (HIP_R_16F or HIP_R_32F).  Enqueued on `stream`, returns without synchronising.
+//                                                              [hiptensor.hpp:89-98]
+hiptensorStatus_t hiptensorPermutation(const hiptensorHandle_t*           handle,
+                                       const void*                        alpha,
+                                       const void*                        A,
+                                       const hiptensorTensorDescriptor_t* descA,
+                                       const int32_t                      modeA[],
+                                       void*                              B,
+                                       const hiptensorTensorDescriptor_t* descB,
+                                       const int32_t                      modeB[],
+                                       const hipDataType                  typeScalar,
+                                       const hipStream_t                  stream);
 
 // Largest power-of-two alignment (element size .. 16 bytes) of `ptr`.
 //                                                            [hiptensor.hpp:108-111]

@@ -1,5 +1,6 @@
 /*
- * Flat C ABI of the contraction path (extern "C", plain pointers and sizes).
+ * Flat C ABI of the contraction path and of the tensor permutation (extern "C", plain
+ * pointers and sizes).
  *
  * The reference's public functions take C++ structs with std::vector members
  * (library/include/hiptensor/hiptensor_types.hpp:177-227), so they cannot be bound
@@ -91,6 +92,40 @@ int hiptensorAmdContraction(const void* handle,
                             void*       workspace,
                             uint64_t    workspaceSize,
                             void*       stream);
+
+/* hiptensorPermutation; typeScalar is a hipDataType, stream a hipStream_t  (hiptensor.hpp:89-98) */
+int hiptensorAmdPermutation(const void*    handle,
+                            const void*    alpha,
+                            const void*    A,
+                            const void*    descA,
+                            const int32_t* modeA,
+                            void*          B,
+                            const void*    descB,
+                            const int32_t* modeB,
+                            int            typeScalar,
+                            void*          stream);
+
+/* What hiptensorAmdPermutation would launch for these descriptors, mode lists and addresses
+ * (only the alignment of A and B is looked at; nothing is read or launched, no device is
+ * needed).  Returns the status the call would return before launching.  No counterpart in
+ * the reference. */
+typedef struct hiptensorAmdPermutationInfo
+{
+    int32_t fused_rank;   /* modes left after extent-1 modes are dropped and neighbours fused */
+    int32_t extent[6];    /* fused extents in A's order, fastest first                        */
+    int32_t a_stride[6], b_stride[6];
+    int32_t kernel;       /* HIPTK_PERM_COPY / TILED / ROWS / GATHER                          */
+    int32_t mode_i, mode_j, tile, vec_r, vec_w;
+    int32_t empty;        /* 1: an extent is zero, nothing would be launched                  */
+    char    kernel_name[96];
+} hiptensorAmdPermutationInfo_t;
+int hiptensorAmdPermutationInfo(const void*                    descA,
+                                const int32_t*                 modeA,
+                                const void*                    descB,
+                                const int32_t*                 modeB,
+                                const void*                    A,
+                                const void*                    B,
+                                hiptensorAmdPermutationInfo_t* out);
 
 /* logger control                                                     (hiptensor.hpp:308-343) */
 typedef void (*hiptensorAmdLoggerCallback_t)(int32_t logContext, const char* funcName, const char* msg);

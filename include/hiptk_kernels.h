@@ -134,6 +134,50 @@ int hiptk_mfma_ceiling(int cls, int random_operands, double* tflops);
  * the clock this device sustains depends on the operand values. */
 int hiptk_fill_pattern(void* dst, uint64_t bytes, int cls, void* stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Tensor permutation, B[perm(index)] = opB(alpha * opA(A[index])).  Takes the place of the
+ * Composable Kernel DeviceElementwise objects the reference drives for this operation
+ * (library/src/permutation/permutation_solution_impl.hpp:134-152,
+ * library/src/permutation/permutation_solution.cpp).  The problem arrives with modes already
+ * fused: extent / a_stride / b_stride are listed in A's order, a_stride[0] == 1.
+ * ------------------------------------------------------------------------------------------ */
+enum
+{
+    HIPTK_PERM_COPY   = 0, /* one fused mode: a scaled copy                                      */
+    HIPTK_PERM_TILED  = 1, /* A's fastest mode (mode_i) and B's fastest mode (mode_j) differ:
+                              two-dimensional tiles of those two modes go through LDS, read along
+                              mode_i and written along mode_j                                     */
+    HIPTK_PERM_ROWS   = 2, /* both tensors share the fastest mode (mode_i == 0): runs of that mode
+                              are copied, tiles span it and one further mode (mode_j)             */
+    HIPTK_PERM_GATHER = 3  /* one thread per element of B, any layout                             */
+};
+
+#define HIPTK_PERM_MAX_RANK 6
+
+typedef struct hiptk_permute
+{
+    int32_t elem_bytes; /* 2: f16, 4: f32                                                        */
+    int32_t rank;       /* fused modes, 1..6                                                      */
+    int32_t extent[HIPTK_PERM_MAX_RANK];
+    int32_t a_stride[HIPTK_PERM_MAX_RANK]; /* elements                                            */
+    int32_t b_stride[HIPTK_PERM_MAX_RANK];
+    int32_t op_a, op_b; /* 0: identity, 1: square                                                 */
+    float   alpha;      /* multiplies in float for f32, rounded to half first for f16             */
+    int32_t kernel;     /* HIPTK_PERM_*                                                           */
+    int32_t mode_i, mode_j; /* TILED / ROWS: positions (in this struct's order) of the two tile modes */
+    int32_t tile;       /* TILED / ROWS: 0 square, 1 long along mode_i, 2 long along mode_j       */
+    int32_t vec_r;      /* elements per global load (1, 2, 4; 8 for f16)                          */
+    int32_t vec_w;      /* elements per global store                                              */
+} hiptk_permute_t;
+
+/* Name of the kernel a problem selects ("" if the combination is not instantiated). */
+const char* hiptk_permute_kernel_name(const hiptk_permute_t* prob);
+
+/* Enqueue on `stream`.  The launcher checks, before anything is launched, that the problem is
+ * well formed and that A, B and every stride meet the alignment vec_r / vec_w ask for;
+ * the two tensors hold fewer than 2^31 elements each.  Returns a HIPTK_* code. */
+int hiptk_permute(const hiptk_permute_t* prob, const void* A, void* B, void* stream, int* hip_error);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,4 +1,4 @@
-"""CPU oracle of the contraction path.  TEST INFRASTRUCTURE ONLY.
+"""CPU oracle of the contraction and permutation paths.  TEST INFRASTRUCTURE ONLY.
 
 Only tests, the smoke check and the cpu_baseline leg of the benchmark may import this
 package; the product (hiptensor_amd) never does.
@@ -6,6 +6,8 @@ package; the product (hiptensor_amd) never does.
   contract(w, A, B, C, ...)       the C restatement in contraction_oracle.c
   ref_contract(w, A, B, C)        the reference's own CPU contraction, compiled from its
                                   sources by build_ref.sh into _ref/ (None if not built)
+  permute(w, A)                   the C restatement in permutation_oracle.c
+  ref_permute(w, A)               the reference's own CPU permutation (None if not built)
 """
 import ctypes as C
 import os
@@ -55,6 +57,8 @@ def lib():
         _lib.oracle_bf16_to_f32.argtypes = [C.c_uint16]
         _lib.oracle_gen_value.restype = C.c_float
         _lib.oracle_gen_value.argtypes = [C.c_uint32]
+        _lib.oracle_permutation.restype = C.c_int
+        _lib.oracle_permutation.argtypes = [C.c_int, C.c_int] + [C.c_void_p] * 3 + [C.c_int] + [C.c_void_p] * 4 + [C.c_int] * 2
     return _lib
 
 
@@ -69,6 +73,9 @@ def ref_lib():
             + [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p] * 2
             + [C.c_int] + [C.c_void_p] * 5 + [C.c_int] * 4
         )
+        if hasattr(_ref, "ref_permutation"):
+            _ref.ref_permutation.restype = C.c_int
+            _ref.ref_permutation.argtypes = [C.c_void_p] * 3 + [C.c_int] + [C.c_void_p] * 4 + [C.c_int] * 5
     return _ref
 
 
@@ -151,3 +158,39 @@ def ref_contract(w, A, B, Cb, D=None):
     if rc != 0:
         raise RuntimeError(f"reference contraction returned status {rc}")
     return D
+
+
+def _perm_alpha(w):
+    return np.array([w["alpha"]], dtype=np.float16 if w["scalar"] == "f16" else np.float32)
+
+
+def permute(w, A):
+    """Runs the permutation oracle on a packed host tensor; returns packed B (NaN-prefilled)."""
+    from hiptensor_amd import workloads as wl
+
+    B = wl.nan_buffer(w["dtype"], max(int(np.prod(w["lensB"])), 1))
+    alpha = _perm_alpha(w)
+    lA, mA, lB, mB = _i64(w["lensA"]), _i32(w["modesA"]), _i64(w["lensB"]), _i32(w["modesB"])
+    rc = lib().oracle_permutation(HIP_TYPE[w["dtype"]], HIP_TYPE[w["scalar"]], _p(alpha), _p(A), _p(B),
+                                  len(lA), _p(lA), _p(mA), _p(lB), _p(mB), w["opA"], w["opB"])
+    if rc != 0:
+        raise RuntimeError(f"oracle_permutation failed with {rc}")
+    return B
+
+
+def ref_permute(w, A):
+    """Runs the compiled reference's CPU permutation; None if oracle/_ref is absent."""
+    from hiptensor_amd import workloads as wl
+
+    r = ref_lib()
+    if r is None or not hasattr(r, "ref_permutation"):
+        return None
+    B = wl.nan_buffer(w["dtype"], max(int(np.prod(w["lensB"])), 1))
+    alpha = _perm_alpha(w)
+    lA, mA, lB, mB = _i64(w["lensA"]), _i32(w["modesA"]), _i64(w["lensB"]), _i32(w["modesB"])
+    t = HIP_TYPE[w["dtype"]]
+    rc = r.ref_permutation(_p(alpha), _p(A), _p(B), len(lA), _p(lA), _p(mA), _p(lB), _p(mB),
+                           t, t, w["opA"], w["opB"], HIP_TYPE[w["scalar"]])
+    if rc != 0:
+        raise RuntimeError(f"reference permutation returned status {rc}")
+    return B

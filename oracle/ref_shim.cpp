@@ -73,3 +73,35 @@ extern "C" int ref_contraction(int            computeType,
                                               (hipDataType)typeD,
                                               nullptr);
 }
+
+#include "permutation_cpu_reference.hpp"
+
+// The reference's hiptensorPermutationReference
+// (library/src/permutation/permutation_cpu_reference.hpp:33-43).  The handle is not read
+// (permutation_cpu_reference.cpp:31-83); the descriptors are built here the way
+// hiptensorInitTensorDescriptor fills them for NULL strides (library/src/hiptensor.cpp:199-206).
+extern "C" int ref_permutation(const void*    alpha,
+                               const void*    A,
+                               void*          B,
+                               int            rank,
+                               const int64_t* lenA,
+                               const int32_t* modeA,
+                               const int64_t* lenB,
+                               const int32_t* modeB,
+                               int            typeA,
+                               int            typeB,
+                               int            opA,
+                               int            opB,
+                               int            typeScalar)
+{
+    auto desc = [rank](const int64_t* len, int type, int op) {
+        std::vector<size_t> l(len, len + rank), s(rank, 1);
+        for(int i = rank - 2; i >= 0; --i)
+            s[i] = s[i + 1] * l[i + 1];
+        return hiptensorTensorDescriptor_t{(hipDataType)type, l, s, (hiptensorOperator_t)op};
+    };
+    auto dA = desc(lenA, typeA, opA);
+    auto dB = desc(lenB, typeB, opB);
+    return (int)hiptensorPermutationReference(
+        nullptr, alpha, A, &dA, modeA, B, &dB, modeB, (hipDataType)typeScalar, nullptr);
+}

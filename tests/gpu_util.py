@@ -36,3 +36,28 @@ def run_gpu(handle, w, inp=None, algo=api.HIPTENSOR_ALGO_DEFAULT, pref=api.HIPTE
     api.check(st, "hiptensorContraction " + w["name"])
     out = D.cpu().numpy().view(wl.NP_STORE[w["dtype"]])
     return (out, info) if return_info else out
+
+
+def run_gpu_permutation(handle, w, A=None, a_shift=0, b_shift=0, return_info=False):
+    """Runs one permutation workload; returns packed B as a host array of the storage type.
+    a_shift / b_shift move the two device tensors off their allocation's alignment by that
+    many elements.  B is pre-filled with NaN, so an element left unwritten shows."""
+    import torch
+
+    if A is None:
+        A = wl.permutation_input(w)
+    t = wl.NP_STORE[w["dtype"]]
+    n = max(int(np.prod(w["lensB"])), 1)
+    item = np.dtype(t).itemsize
+    hostA = np.concatenate([np.zeros(a_shift, dtype=t), np.ascontiguousarray(A, dtype=t)])
+    dA = to_device(hostA)
+    dB = to_device(wl.nan_buffer(w["dtype"], n + b_shift))
+    p = wl.Permutation(handle, w)
+    pa, pb = dA.data_ptr() + a_shift * item, dB.data_ptr() + b_shift * item
+    info = p.info(pa, pb)
+    st = p.run(pa, pb, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    p.close()
+    api.check(st, "hiptensorPermutation " + w["name"])
+    out = dB.cpu().numpy().view(t)[b_shift:]
+    return (out, info) if return_info else out

@@ -1,0 +1,62 @@
+"""Permutation shapes shared by the CPU and GPU test suites.
+
+VALIDATION follows the reference's own matrices (test/02_permutation/configs/validation/
+rank{2..6}_test_params.yaml, data only): per rank the listed lengths, every order of the modes
+("Permuted Dims" lists all of them), alphas 0 / 1 / 2.3, the four operator pairs and the three
+(data type, scalar type) rows.  LARGE are shapes big enough to reach the tiled kernels.
+"""
+import itertools
+
+from hiptensor_amd import api
+from hiptensor_amd import workloads as wl
+
+TYPE_ROWS = [("f32", "f32"), ("f16", "f16"), ("f16", "f32")]
+ALPHAS = [0.0, 1.0, 2.3]
+OPS = [(api.HIPTENSOR_OP_IDENTITY, api.HIPTENSOR_OP_IDENTITY), (api.HIPTENSOR_OP_IDENTITY, api.HIPTENSOR_OP_SQRT),
+       (api.HIPTENSOR_OP_SQRT, api.HIPTENSOR_OP_IDENTITY), (api.HIPTENSOR_OP_SQRT, api.HIPTENSOR_OP_SQRT)]
+LENGTHS = {
+    2: [[1, 1], [5, 2], [3, 4], [15, 12], [23, 11]],
+    3: [[1, 1, 1], [5, 2, 3], [5, 2, 4], [15, 12, 23], [12, 23, 11]],
+    4: [[1, 1, 1, 1], [5, 2, 3, 4], [5, 2, 1, 1], [15, 12, 23, 11]],
+    5: [[1, 1, 1, 1, 1], [5, 2, 3, 4, 5], [5, 2, 1, 1, 2], [15, 12, 23, 11, 2]],
+    6: [[1, 1, 1, 1, 1, 1], [5, 2, 3, 4, 1, 2], [5, 2, 1, 1, 1, 2], [15, 12, 23, 11, 1, 2]],
+}
+
+
+def validation(rank, thin=1):
+    """Workloads of one rank.  thin > 1 keeps every thin-th (alpha, operators, type row)
+    combination per (lengths, order), cycling so that all combinations still occur."""
+    combos = list(itertools.product(ALPHAS, OPS, TYPE_ROWS))
+    out, n = [], 0
+    for lens in LENGTHS[rank]:
+        for perm in itertools.permutations(range(rank)):
+            for k, (alpha, (oa, ob), (dt, sc)) in enumerate(combos):
+                if (k + n) % thin == 0:
+                    out.append(wl.permutation(dt, lens, perm, alpha, sc, oa, ob))
+            n += 1
+    return out
+
+
+# (lengths, order): shapes that select the copy, tiled, rows and gather kernels with full and
+# narrowed vectors, edges that do not fill a tile, and the sample program's 33 x 32 x 34 x 35
+LARGE = [
+    ([64, 64, 64], [0, 1, 2]),            # nothing moves: scaled copy
+    ([33, 32, 34, 35], [2, 3, 1, 0]),     # samples/02_permutation/permutation.cpp
+    ([256, 192], [1, 0]),                 # plain transpose, whole vectors
+    ([250, 130], [1, 0]),                 # pairs only, ragged tiles
+    ([255, 129], [1, 0]),                 # scalar accesses
+    ([128, 24, 96], [2, 1, 0]),
+    ([128, 24, 96], [1, 0, 2]),           # batched transpose with a short second mode
+    ([128, 24, 96], [0, 2, 1]),           # shared fastest mode: rows
+    ([40, 50, 60], [0, 2, 1]),
+    ([1024, 20, 4], [1, 0, 2]),           # long i, short j
+    ([20, 1024, 4], [1, 0, 2]),           # short i, long j
+    ([6, 70, 80], [1, 0, 2]),             # short fastest mode: gather
+    ([8, 16, 8, 16, 8, 16], [5, 3, 1, 4, 2, 0]),
+    ([32, 8, 16, 4, 8, 4], [1, 0, 3, 2, 5, 4]),
+    ([512, 512], [1, 0]),
+]
+
+
+def large(dtype, scalar=None, alpha=1.7, ops=OPS[0]):
+    return [wl.permutation(dtype, lens, perm, alpha, scalar or dtype, ops[0], ops[1]) for lens, perm in LARGE]

@@ -1,0 +1,146 @@
+"""hiptensorPermutation on the GPU against the CPU oracle, bit for bit (a NaN matches a NaN of
+any payload: the device and the host form different quiet NaNs from 0 * inf).
+
+Covers the reference's validation matrix (test/02_permutation/configs/validation/*.yaml: every
+mode order of ranks 2..6, three alphas, four operator pairs, three type rows), larger shapes
+that reach every kernel, every tile shape and vector width through the selection override,
+pointers off their natural alignment, and a full-size round trip.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import gpu_util
+import perm_cases
+from hiptensor_amd import api
+from hiptensor_amd import workloads as wl
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def _same(got, want):
+    if got.shape != want.shape:
+        return False
+    bits = got.view(np.uint8).reshape(got.size, -1) == want.view(np.uint8).reshape(want.size, -1)
+    return bool(np.all(bits.all(axis=1) | (np.isnan(got) & np.isnan(want))))
+
+
+class _Override:
+    """Sets the selection override for the duration of a block."""
+
+    def __init__(self, value):
+        self.value = value
+
+    def __enter__(self):
+        self.old = os.environ.get("HIPTENSOR_AMD_PERMUTE")
+        if self.value:
+            os.environ["HIPTENSOR_AMD_PERMUTE"] = self.value
+        else:
+            os.environ.pop("HIPTENSOR_AMD_PERMUTE", None)
+
+    def __exit__(self, *a):
+        if self.old is None:
+            os.environ.pop("HIPTENSOR_AMD_PERMUTE", None)
+        else:
+            os.environ["HIPTENSOR_AMD_PERMUTE"] = self.old
+
+
+def _check(handle, oracle_mod, w, names=None, **kw):
+    A = wl.permutation_input(w)
+    got, info = gpu_util.run_gpu_permutation(handle, w, A, return_info=True, **kw)
+    want = oracle_mod.permute(w, A)
+    assert _same(got, want), (w["name"], w["scalar"], w["alpha"], w["opA"], w["opB"], info["kernel_name"])
+    if names is not None:
+        names.add(info["kernel_name"])
+
+
+def test_known_answer_vector(gpu_handle):
+    with open(os.path.join(HERE, "golden", "permutation_known_answer.json")) as f:
+        k = json.load(f)
+    lens = [k["extent"][str(m)] for m in k["modesA"]]
+    perm = [k["modesA"].index(m) for m in k["modesB"]]
+    w = wl.permutation("f32", lens, perm, k["alpha"])
+    got = gpu_util.run_gpu_permutation(gpu_handle, w, np.arange(120, dtype=np.float32))
+    want = np.array(k["expected"], dtype=np.float32)
+    assert np.max(np.abs(got - want) / (np.abs(want) + 1.0)) < 10 * np.finfo(np.float32).eps
+
+
+@pytest.mark.parametrize("rank", [2, 3, 4, 5, 6])
+@pytest.mark.parametrize("override", ["", "gather", "tiled,-1,8"])
+def test_validation_matrix(gpu_handle, oracle_mod, rank, override):
+    thin = {2: 1, 3: 1, 4: 3, 5: 13, 6: 79}[rank] * (1 if not override else 3)
+    with _Override(override):
+        for w in perm_cases.validation(rank, thin=thin):
+            _check(gpu_handle, oracle_mod, w)
+
+
+@pytest.mark.parametrize("dtype,scalar", perm_cases.TYPE_ROWS)
+def test_large_shapes_default_selection(gpu_handle, oracle_mod, dtype, scalar):
+    names = set()
+    for ops in perm_cases.OPS:
+        for w in perm_cases.large(dtype, scalar, 1.7, ops):
+            _check(gpu_handle, oracle_mod, w, names)
+    kinds = {n.split("_")[1] for n in names}
+    assert kinds == {"copy", "tiled", "rows", "gather"}, names
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("maxvec", [1, 2, 8])
+def test_every_tile_and_vector_width(gpu_handle, oracle_mod, dtype, tile, maxvec):
+    names = set()
+    with _Override(f"tiled,{tile},{maxvec}"):
+        for w in perm_cases.large(dtype, alpha=-0.75, ops=perm_cases.OPS[2]):
+            _check(gpu_handle, oracle_mod, w, names)
+    assert any(n.startswith("permute_tiled") for n in names) and any(n.startswith("permute_rows") for n in names)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_pointers_off_their_alignment(gpu_handle, oracle_mod, dtype):
+    for a_shift, b_shift in ((1, 0), (0, 1), (2, 2), (1, 3), (4, 2)):
+        for lens, perm in (([256, 192], [1, 0]), ([128, 24, 96], [0, 2, 1]), ([64, 64, 64], [0, 1, 2])):
+            _check(gpu_handle, oracle_mod, wl.permutation(dtype, lens, perm, 1.25), a_shift=a_shift, b_shift=b_shift)
+
+
+def test_zero_extent_is_a_no_op(gpu_handle):
+    import torch
+
+    w = wl.permutation("f32", [4, 0, 3], [2, 0, 1])
+    p = wl.Permutation(gpu_handle, w)
+    buf = torch.zeros(16, device="cuda")
+    assert p.run(buf.data_ptr(), buf.data_ptr() + 32) == api.HIPTENSOR_STATUS_SUCCESS
+    p.close()
+
+
+def test_full_size_round_trip(gpu_handle):
+    """2^28 f32 elements (1 GiB each way): a permutation followed by its inverse returns A, and
+    B is a rearrangement of A (same multiset, checked through order-free sums of the bit
+    patterns)."""
+    import torch
+
+    lens, perm = [512, 64, 128, 64], [2, 0, 3, 1]
+    inv = [perm.index(i) for i in range(4)]
+    n = int(np.prod(lens))
+    A = torch.randint(-(2 ** 31), 2 ** 31 - 1, (n,), dtype=torch.int32, device="cuda")
+    A &= ~(0x7F800000)  # exponent field cleared: zeros and denormals only, which alpha = 1 must return bit for bit
+    B = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    A2 = torch.full((n,), -1, dtype=torch.int32, device="cuda")
+    fwd = wl.Permutation(gpu_handle, wl.permutation("f32", lens, perm))
+    back = wl.Permutation(gpu_handle, wl.permutation("f32", [lens[p] for p in perm], inv))
+    api.check(fwd.run(A.data_ptr(), B.data_ptr(), torch.cuda.current_stream().cuda_stream), "forward")
+    api.check(back.run(B.data_ptr(), A2.data_ptr(), torch.cuda.current_stream().cuda_stream), "back")
+    torch.cuda.synchronize()
+    assert fwd.info(A.data_ptr(), B.data_ptr())["kernel"] == api.PERM_TILED
+    assert torch.equal(A, A2)
+    assert int(A.to(torch.int64).sum()) == int(B.to(torch.int64).sum())
+    assert int((A.to(torch.int64) ** 2 % 1000003).sum()) == int((B.to(torch.int64) ** 2 % 1000003).sum())
+    # spot check of the index map against the definition
+    a = A.view(*reversed(lens))  # torch is row-major: reversed extents give first-mode-fastest
+    b = B.view(*reversed([lens[p] for p in perm]))
+    want = a.permute(*[3 - perm[3 - d] for d in range(4)])
+    assert torch.equal(b[::7, ::5, ::3, ::11], want[::7, ::5, ::3, ::11])
+    fwd.close()
+    back.close()
