@@ -2,6 +2,7 @@
 """Benchmark of the contraction path on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all] [--no-cpu]
+  python bench.py --permutation [--workload NAME] [--all]      (the permutation beside it)
 
 A step is one hiptensorContraction call (through the flat C ABI) on inputs that are already
 resident in HBM; plan creation is outside the timed region, and so is a short untimed load
@@ -78,6 +79,109 @@ def measure(handle, w, steps, warmup, settle_s=0.25):
     return out
 
 
+def measure_permutation(handle, w, steps, warmup, settle_s=0.25):
+    """One step = one hiptensorPermutation call, tensors resident in HBM."""
+    import torch
+
+    from hiptensor_amd import workloads as wl
+
+    n = 1
+    for l in w["lensA"]:
+        n *= l
+    nbytes = n * wl.ELEM_BYTES[w["dtype"]]
+    A = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    from hiptensor_amd._lib import lib as _native
+    stream = torch.cuda.current_stream()
+    # finite pseudo-random elements (class ids of the fill: 0 f16, 2 f32)
+    assert _native.hiptk_fill_pattern(A.data_ptr(), nbytes, 0 if w["dtype"] == "f16" else 2, stream.cuda_stream) == 0
+    B = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    p = wl.Permutation(handle, w)
+    info = p.info(A.data_ptr(), B.data_ptr())
+    args = (A.data_ptr(), B.data_ptr(), stream.cuda_stream)
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < settle_s:
+        for _ in range(5):
+            assert p.run(*args) == 0
+        torch.cuda.synchronize()
+    for _ in range(warmup):
+        assert p.run(*args) == 0
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(steps):
+        st = p.run(*args)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    assert st == 0
+    p.close()
+    return {"ms_per_step": (t1 - t0) * 1e3 / steps, "kernel_ms": e0.elapsed_time(e1) / steps, "info": info}
+
+
+def cpu_baseline_permutation(w, budget_elems=1.2e8):
+    """Times the CPU permutation on the same mode order with the slowest mode of A cut down to
+    about budget_elems elements.  Uses the compiled reference when oracle/_ref is present."""
+    import numpy as np
+
+    import oracle
+    from hiptensor_amd import workloads as wl
+
+    lens = list(w["lensA"])
+    inner = int(np.prod(lens[:-1]))
+    take = max(1, min(lens[-1], int(budget_elems // inner)))
+    lens[-1] = take
+    sub = wl.permutation(w["dtype"], lens, w["perm"], w["alpha"], w["scalar"], w["opA"], w["opB"])
+    A = wl.permutation_input(sub)
+    use_ref = oracle.ref_lib() is not None and hasattr(oracle.ref_lib(), "ref_permutation")
+    t0 = time.perf_counter()
+    (oracle.ref_permute if use_ref else oracle.permute)(sub, A)
+    dt = time.perf_counter() - t0
+    return {"value": wl.permutation_bytes(sub) / dt / 1e9, "unit": "GB/s", "cores": 1,
+            "kind": "reference" if use_ref else "port",
+            "sample": f"slowest mode of A cut from {w['lensA'][-1]} to {take} ({int(np.prod(lens))} elements)",
+            "ms_sample": dt * 1e3}
+
+
+def permutation_line(a, handle, prop):
+    """The JSON line of --permutation: GB/s of one permutation workload against HBM."""
+    from hiptensor_amd import workloads as wl
+
+    cfgs = wl.permutation_configs()
+    name = a.workload if a.workload in cfgs else "perm_f32_rank4"
+    w = cfgs[name]
+    r = measure_permutation(handle, w, a.steps, a.warmup, a.settle)
+    nbytes = wl.permutation_bytes(w)
+    gbs = nbytes / (r["kernel_ms"] * 1e-3) / 1e9
+    out = {
+        "metric": "permutation GB/s (bytes read + bytes written, and fraction of HBM peak) on 1 MI355X",
+        "value": nbytes / (r["ms_per_step"] * 1e-3) / 1e9, "unit": "GB/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "settle_s": a.settle, "ms_per_step": r["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": w["name"], "lengths": w["lensA"], "permuted_dims": w["perm"], "alpha": w["alpha"],
+                   "kernel": r["info"]["kernel_name"]},
+        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((w["name"], r["info"]["kernel_name"])),
+                     "kernel_ms": r["kernel_ms"], "algorithmic_bytes": nbytes},
+        "device": {"name": prop.name, "cus": prop.multi_processor_count},
+    }
+    if a.all:
+        others = {}
+        for oname, ow in cfgs.items():
+            if oname == name:
+                continue
+            rr = measure_permutation(handle, ow, max(5, a.steps // 4), max(2, a.warmup // 4), a.settle)
+            ob = wl.permutation_bytes(ow)
+            others[oname] = {"kernel_ms": rr["kernel_ms"], "GBs": ob / (rr["kernel_ms"] * 1e-3) / 1e9,
+                             "frac_hbm": ob / (rr["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                             "kernel": rr["info"]["kernel_name"], "dtype": ow["dtype"], "workload": ow["name"]}
+        out["others"] = others
+    if not a.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_permutation(w)
+    return out
+
+
 def cpu_baseline(w, budget_macs=8.6e9):
     """Times the CPU contraction on a slab of the workload: the outputs whose slowest M mode
     lies in a leading sub-range, full N and K.  Uses the compiled reference when oracle/_ref
@@ -131,6 +235,9 @@ def main():
     ap.add_argument("--workload", default="cfg2_f16_scale")
     ap.add_argument("--all", action="store_true", help="also time every other configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--permutation", action="store_true",
+                    help="time hiptensorPermutation instead (workload: a name of workloads.permutation_configs(), "
+                         "default perm_f32_rank4); the JSON line then carries GB/s against the HBM roofline")
     ap.add_argument("--pcie", action="store_true",
                     help="also time the step with operands copied from, and the result to, pinned host memory")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -153,6 +260,11 @@ def main():
     clock_ghz = getattr(prop, "clock_rate", 2400000) / 1e6
     cus = prop.multi_processor_count
     handle = api.check(api.hiptensorCreate(), "hiptensorCreate")
+    if a.permutation:
+        out = permutation_line(a, handle, prop)
+        api.hiptensorDestroy(handle)
+        print(json.dumps(out))
+        return
     cfgs = wl.baseline_configs()
     w = cfgs[a.workload]
     r = measure(handle, w, a.steps, a.warmup, a.settle)

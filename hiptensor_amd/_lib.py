@@ -24,7 +24,7 @@ def _load():
     return C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
 
 
-lib = _load()
+_cdll = _load()
 
 vp = C.c_void_p
 i64p = C.POINTER(C.c_int64)
@@ -88,8 +88,25 @@ _SIGS = {
     "hiptensorAmdPlanTable": (C.c_int64, [vp, C.c_int, i32p, C.c_int64]),
     "hiptk_mfma_ceiling": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_double)]),
     "hiptk_tile_count": (C.c_int, [C.c_int]),
+    "hiptk_tile_info": (C.c_int, [C.c_int, C.c_int, vp]),
+    "hiptk_fill_pattern": (C.c_int, [vp, C.c_uint64, C.c_int, vp]),
 }
-for _name, (_res, _args) in _SIGS.items():
-    _fn = getattr(lib, _name)
-    _fn.restype = _res
-    _fn.argtypes = _args
+
+
+class _Declared:
+    """The library's functions, each with its argument types set.  A function that has no
+    entry in _SIGS cannot be reached: ctypes would otherwise pass every Python int as a C int
+    and silently cut a device address down to 32 bits."""
+
+    def __init__(self, cdll):
+        for name, (res, args) in _SIGS.items():
+            fn = getattr(cdll, name)
+            fn.restype = res
+            fn.argtypes = args
+            object.__setattr__(self, name, fn)
+
+    def __getattr__(self, name):
+        raise AttributeError(f"{name} has no declared signature in hiptensor_amd/_lib.py")
+
+
+lib = _Declared(_cdll)

@@ -361,3 +361,24 @@ class Permutation:
     def close(self):
         api.destroy("tensor", self.dA)
         api.destroy("tensor", self.dB)
+
+
+def permutation_configs():
+    """Permutation workloads the benchmark times: tensors of about 1 GiB, far larger than the
+    256 MiB last-level cache, so that the figures are HBM figures."""
+    return {
+        "perm_f32_rank4": permutation("f32", [512, 64, 128, 64], [2, 0, 3, 1], 1.5, name="perm_f32_512x64x128x64_2031"),
+        "perm_f16_rank4": permutation("f16", [1024, 64, 128, 64], [2, 0, 3, 1], 1.5, name="perm_f16_1024x64x128x64_2031"),
+        "perm_f32_transpose": permutation("f32", [16384, 16384], [1, 0], 1.5, name="perm_f32_16384x16384_10"),
+        "perm_f16_transpose": permutation("f16", [32768, 16384], [1, 0], 1.5, name="perm_f16_32768x16384_10"),
+        "perm_f32_rows": permutation("f32", [256, 64, 128, 128], [0, 2, 1, 3], 1.5, name="perm_f32_256x64x128x128_0213"),
+        "perm_f32_copy": permutation("f32", [512, 64, 128, 64], [0, 1, 2, 3], 1.5, name="perm_f32_512x64x128x64_0123"),
+        "perm_f16_nchw_to_nhwc": permutation("f16", [224, 224, 64, 256], [2, 0, 1, 3], 1.0, name="perm_f16_224x224x64x256_2013"),
+        "perm_f32_channels3": permutation("f32", [512, 512, 3, 256], [2, 0, 1, 3], 1.0, name="perm_f32_512x512x3x256_2013"),
+        "perm_f32_sample": permutation("f32", [33, 32, 34, 35], [2, 3, 1, 0], 1.0, name="perm_f32_33x32x34x35_2310"),
+    }
+
+
+def permutation_bytes(w):
+    """Every element read once and written once."""
+    return 2 * ELEM_BYTES[w["dtype"]] * int(np.prod(w["lensA"]))

@@ -29,7 +29,7 @@ def test_c_abi_symbols_exported():
         missing = [n for n in names if n not in syms]
         assert not missing, (header, missing)
         for n in names:
-            assert getattr(_lib.lib, n) is not None
+            assert getattr(_lib._cdll, n) is not None  # resolvable through the loader too
 
 
 def test_cpp_api_symbols_exported():
@@ -38,3 +38,18 @@ def test_cpp_api_symbols_exported():
     assert "hiptensorContraction" in names and "hiptensorInitContractionPlan" in names
     for n in names:
         assert re.search(rf"\b{n}\(", out), n
+
+
+def test_bindings_reach_declared_functions_only():
+    """A ctypes function without argument types passes Python ints as C ints, which cuts a
+    device address to 32 bits; the binding therefore refuses any function it has no signature for,
+    and every address parameter of a declared one is pointer-sized."""
+    import ctypes
+
+    import pytest
+
+    with pytest.raises(AttributeError):
+        _lib.lib.hiptk_permute  # kernel-layer entry that Python has no business calling
+    for name, (_, args) in _lib._SIGS.items():
+        assert getattr(_lib.lib, name).argtypes == args
+    assert _lib._SIGS["hiptk_fill_pattern"][1][0] is ctypes.c_void_p

@@ -100,8 +100,5 @@ def _tile_exists(cls, tile):
                     ("bk", ctypes.c_int32), ("threads", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
                     ("name", ctypes.c_char * 64)]
 
-    fn = lib.hiptk_tile_info
-    fn.restype = ctypes.c_int
-    fn.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(TileInfo)]
     ti = TileInfo()
-    return fn(cls, tile, ctypes.byref(ti)) == 0
+    return lib.hiptk_tile_info(cls, tile, ctypes.byref(ti)) == 0
