@@ -36,9 +36,11 @@ namespace
         return sign ? -v : v;
     }
 
-    // HIPTENSOR_AMD_PERMUTE="kernel[,tile[,maxvec]]": kernel is auto | gather | tiled | rows
-    // (tiled and rows name the same preference: whichever of the two the layout admits),
-    // tile is 0..2 or -1, maxvec caps the vector width.  For tests and experiments.
+    // HIPTENSOR_AMD_PERMUTE="kernel[,tile[,maxvec[,group]]]": kernel is auto | gather | tiled |
+    // rows | strip (tiled and rows name the same preference: whichever of the two the layout
+    // admits; strip is taken wherever a short tile mode admits it),
+    // tile is 0..2 or -1, maxvec caps the vector width, group sets the band width of the
+    // workgroup order.  For tests and experiments.
     hipta::PermuteTuning tuningFromEnv()
     {
         hipta::PermuteTuning t;
@@ -55,6 +57,8 @@ namespace
                 t.kernel = HIPTK_PERM_GATHER;
             else if(!std::strcmp(tok, "tiled") || !std::strcmp(tok, "rows"))
                 t.kernel = HIPTK_PERM_TILED;
+            else if(!std::strcmp(tok, "strip"))
+                t.kernel = HIPTK_PERM_STRIP;
             tok = strtok_r(nullptr, ",", &save);
         }
         if(tok)
@@ -63,7 +67,12 @@ namespace
             tok    = strtok_r(nullptr, ",", &save);
         }
         if(tok)
+        {
             t.max_vec = std::atoi(tok);
+            tok       = strtok_r(nullptr, ",", &save);
+        }
+        if(tok)
+            t.group = std::atoi(tok);
         return t;
     }
 }

@@ -151,6 +151,7 @@ namespace hipta
             out.b_stride[d] = (int32_t)bs[d];
         }
         out.vec_r = out.vec_w = 1;
+        out.group             = tune.group >= 1 ? tune.group : 1;
         const int cap         = std::max(1, tune.max_vec);
 
         if(r == 1)
@@ -167,15 +168,22 @@ namespace hipta
             if(bs[d] == 1)
                 jB = d;
 
-        // layout-admissible kernels: TILED needs differing fastest modes, ROWS a shared one
+        // layout-admissible kernels: TILED needs differing fastest modes, ROWS a shared one,
+        // STRIP a tile mode of at most 16 elements whose partner follows it directly in memory
         const bool shared = jB == 0;
+        const bool stripJ = !shared && ext[jB] <= 16 && bs[0] == ext[jB]; // short j, B holds i right after it
+        const bool stripI = !shared && ext[0] <= 16 && jB == 1 && !stripJ; // short i, A holds j right after it
         int        kernel;
         if(tune.kernel == HIPTK_PERM_GATHER)
             kernel = HIPTK_PERM_GATHER;
+        else if(tune.kernel == HIPTK_PERM_STRIP && (stripJ || stripI))
+            kernel = HIPTK_PERM_STRIP;
         else if(tune.kernel == HIPTK_PERM_TILED || tune.kernel == HIPTK_PERM_ROWS)
             kernel = shared ? HIPTK_PERM_ROWS : HIPTK_PERM_TILED;
         else if(count <= 16384)
             kernel = HIPTK_PERM_GATHER; // a launch's worth of latency either way
+        else if((stripJ && ext[0] >= 64) || (stripI && ext[jB] >= 64))
+            kernel = HIPTK_PERM_STRIP;
         else if(shared)
             kernel = ext[0] >= 16 ? HIPTK_PERM_ROWS : HIPTK_PERM_GATHER;
         else
@@ -185,6 +193,33 @@ namespace hipta
             return PermuteStatus::OK;
 
         out.mode_i = 0;
+        if(kernel == HIPTK_PERM_STRIP)
+        {
+            out.mode_j = jB;
+            out.tile   = stripJ ? 0 : 1;
+            const int64_t        run = ext[0] * ext[jB];
+            std::vector<int64_t> linOthers, rowOthers;
+            for(int d = 1; d < r; ++d)
+            {
+                if(d != jB)
+                    linOthers.push_back(stripJ ? bs[d] : as[d]);
+                if(stripJ || d != jB)
+                    rowOthers.push_back(stripJ ? as[d] : bs[d]);
+            }
+            if(!stripJ)
+                rowOthers.push_back(bs[0]);
+            if(stripJ)
+            {
+                out.vec_r = pickVec(in.elem_bytes, cap, ext[0], rowOthers, in.A, false);
+                out.vec_w = pickVec(in.elem_bytes, cap, run, linOthers, in.B, false);
+            }
+            else
+            {
+                out.vec_r = pickVec(in.elem_bytes, cap, run, linOthers, in.A, false);
+                out.vec_w = pickVec(in.elem_bytes, cap, ext[jB], rowOthers, in.B, false);
+            }
+            return PermuteStatus::OK;
+        }
         std::vector<int64_t> aOthers(as.begin() + 1, as.end());
         const int            vr = pickVec(in.elem_bytes, cap, ext[0], aOthers, in.A, false);
         if(kernel == HIPTK_PERM_TILED)

@@ -37,6 +37,7 @@ namespace hipta
         int kernel  = -1; // HIPTK_PERM_* to use wherever the layout admits it, -1: automatic
         int tile    = -1; // 0..2, -1: automatic
         int max_vec = 8; // cap on elements per load / store
+        int group   = -1; // tiles per band of the workgroup order, -1: automatic
     };
 
     // Fills `out` (alpha and the operators are left for the caller); out.rank is the number of

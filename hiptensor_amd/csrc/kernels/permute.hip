@@ -10,6 +10,10 @@
 //             workgroup on the scalar unit.
 //   * ROWS    A and B share the fastest mode: runs of it are contiguous on both sides and go
 //             from registers straight back to memory, no LDS.
+//   * STRIP   like TILED, for a tile mode too short to give long runs (the 3 of an RGB image,
+//             say) when the other tile mode follows it directly in memory on that side: a
+//             workgroup takes a strip of the long mode times the whole short mode, which is one
+//             contiguous run on the short mode's side, and moves it linearly there.
 //   * GATHER  one thread per element of B; covers tiny tensors and awkward extents.
 // Element operation per Composable Kernel's UnaryCombinedOp<Aop, Scale, Bop>
 // (ck/tensor_operation/gpu/element/combined_element_wise_operation.hpp:14-32): every step is
@@ -39,6 +43,7 @@ namespace hiptk
             uint32_t    a_j; // A stride of mode j (mode i has stride 1 in A)
             uint32_t    b_i, b_j; // B strides (TILED: b_j == 1, ROWS: b_i == 1)
             uint32_t    nt_i, nt_j; // tiles along i and j
+            uint32_t    group; // tile order: bands of `group` tiles along j, walked j-first
             int32_t     nb; // modes that only pick the tile's base
             uint32_t    bext[PERM_BATCH], ba[PERM_BATCH], bb[PERM_BATCH];
             float       alpha;
@@ -89,12 +94,20 @@ namespace hiptk
             T* __restrict__ B       = static_cast<T*>(a.B);
             const int tid           = threadIdx.x;
 
-            uint32_t       blk = blockIdx.x;
-            const uint32_t ti  = blk % a.nt_i;
-            blk /= a.nt_i;
-            const uint32_t tj = blk % a.nt_j;
-            blk /= a.nt_j;
-            uint32_t aoff = 0, boff = 0;
+            // Workgroups that run at the same time should spread over both tile modes: tiles that
+            // are neighbours along i touch neighbouring addresses of A, neighbours along j
+            // neighbouring addresses of B.  The tile plane is cut into bands of `group` tiles
+            // along j; inside a band the walk is j-first.
+            const uint32_t plane = a.nt_i * a.nt_j;
+            uint32_t       blk   = blockIdx.x / plane;
+            const uint32_t lin   = blockIdx.x - blk * plane;
+            const uint32_t band  = lin / (a.group * a.nt_i);
+            const uint32_t rem   = lin - band * (a.group * a.nt_i);
+            const uint32_t left  = a.nt_j - band * a.group;
+            const uint32_t rows  = left < a.group ? left : a.group;
+            const uint32_t ti    = rem / rows;
+            const uint32_t tj    = band * a.group + (rem - ti * rows);
+            uint32_t       aoff = 0, boff = 0;
             for(int d = 0; d < a.nb; ++d)
             {
                 const uint32_t c = blk % a.bext[d];
@@ -155,6 +168,143 @@ namespace hiptk
                         o.v[e] = tile[(jv * VW + e) * PITCH + i];
                     if(ok)
                         *reinterpret_cast<Vec<T, VW>*>(B + boff + jv * VW + i * a.b_i) = o;
+                }
+            }
+        }
+
+        struct SArgs
+        {
+            const void* A;
+            void*       B;
+            uint32_t    e_s, e_l; // extents of the short and of the long tile mode
+            uint32_t    row_stride; // stride of the short mode on the side that is walked in rows
+            uint32_t    magic; // floor(2^32 / e_s) + 1: v / e_s == umulhi(v, magic) for v < 2^28
+            uint32_t    nt; // strips along the long mode
+            int32_t     nb;
+            uint32_t    bext[PERM_BATCH], ba[PERM_BATCH], bb[PERM_BATCH];
+            float       alpha;
+            int32_t     op_a, op_b;
+        };
+
+        // LINEAR_WRITE: the long mode is A's fastest, the short one B's fastest, and B holds the
+        // long mode right after the short one, so a strip is one run of cnt * e_s elements of B.
+        // It is read in e_s rows of A and written linearly.  !LINEAR_WRITE is the mirror image:
+        // the short mode is A's fastest with the long one right after it; the strip is read
+        // linearly from A and written in e_s rows of B.
+        template <typename T, int TL, int VL, int VS, bool LINEAR_WRITE>
+        __global__ __launch_bounds__(PERM_THREADS) void permute_strip_kernel(SArgs a)
+        {
+            constexpr int NT    = PERM_THREADS;
+            constexpr int U     = 4; // loads in flight per thread
+            constexpr int PITCH = TL + 1;
+            constexpr int VPR   = TL / VS; // row vectors per strip row
+            static_assert(TL % VS == 0 && TL % VL == 0, "strip shape");
+            extern __shared__ unsigned char strip_smem[];
+            T* tile = reinterpret_cast<T*>(strip_smem); // [e_s][PITCH]
+
+            const T* __restrict__ A = static_cast<const T*>(a.A);
+            T* __restrict__ B       = static_cast<T*>(a.B);
+            const uint32_t tid      = threadIdx.x;
+
+            uint32_t       blk = blockIdx.x;
+            const uint32_t t   = blk % a.nt;
+            blk /= a.nt;
+            uint32_t aoff = 0, boff = 0;
+            for(int d = 0; d < a.nb; ++d)
+            {
+                const uint32_t c = blk % a.bext[d];
+                blk /= a.bext[d];
+                aoff += c * a.ba[d];
+                boff += c * a.bb[d];
+            }
+            const uint32_t l0  = t * TL;
+            const uint32_t cnt = (a.e_l - l0) < (uint32_t)TL ? (a.e_l - l0) : (uint32_t)TL;
+            const T        alpha = static_cast<T>(a.alpha);
+            const uint32_t nrv   = a.e_s * VPR; // row vectors of the strip (tail rows included)
+            const uint32_t nlv   = cnt * a.e_s / VL; // linear vectors of the strip
+
+            if constexpr(LINEAR_WRITE)
+            {
+                aoff += l0;
+                boff += l0 * a.e_s;
+                for(uint32_t u0 = 0; u0 < nrv; u0 += NT * U)
+                {
+                    Vec<T, VS> r[U];
+#pragma unroll
+                    for(int k = 0; k < U; ++k)
+                    {
+                        const uint32_t u = u0 + tid + k * NT, s = u / VPR, xv = u % VPR;
+                        r[k]             = Vec<T, VS>{};
+                        if(u < nrv && xv * VS < cnt)
+                            r[k] = *reinterpret_cast<const Vec<T, VS>*>(A + aoff + xv * VS + s * a.row_stride);
+                    }
+#pragma unroll
+                    for(int k = 0; k < U; ++k)
+                    {
+                        const uint32_t u = u0 + tid + k * NT, s = u / VPR, xv = u % VPR;
+                        if(u < nrv)
+                        {
+#pragma unroll
+                            for(int e = 0; e < VS; ++e)
+                                tile[s * PITCH + xv * VS + e] = element_op(r[k].v[e], alpha, a.op_a, a.op_b);
+                        }
+                    }
+                }
+                __syncthreads();
+                for(uint32_t u = tid; u < nlv; u += NT)
+                {
+                    Vec<T, VL> o;
+#pragma unroll
+                    for(int e = 0; e < VL; ++e)
+                    {
+                        const uint32_t v = u * VL + e, x = __umulhi(v, a.magic), sidx = v - x * a.e_s;
+                        o.v[e]           = tile[sidx * PITCH + x];
+                    }
+                    *reinterpret_cast<Vec<T, VL>*>(B + boff + u * VL) = o;
+                }
+            }
+            else
+            {
+                aoff += l0 * a.e_s;
+                boff += l0;
+                for(uint32_t u0 = 0; u0 < nlv; u0 += NT * U)
+                {
+                    Vec<T, VL> r[U];
+#pragma unroll
+                    for(int k = 0; k < U; ++k)
+                    {
+                        const uint32_t u = u0 + tid + k * NT;
+                        r[k]             = Vec<T, VL>{};
+                        if(u < nlv)
+                            r[k] = *reinterpret_cast<const Vec<T, VL>*>(A + aoff + u * VL);
+                    }
+#pragma unroll
+                    for(int k = 0; k < U; ++k)
+                    {
+                        const uint32_t u = u0 + tid + k * NT;
+                        if(u < nlv)
+                        {
+#pragma unroll
+                            for(int e = 0; e < VL; ++e)
+                            {
+                                const uint32_t v = u * VL + e, x = __umulhi(v, a.magic), sidx = v - x * a.e_s;
+                                tile[sidx * PITCH + x] = element_op(r[k].v[e], alpha, a.op_a, a.op_b);
+                            }
+                        }
+                    }
+                }
+                __syncthreads();
+                for(uint32_t u = tid; u < nrv; u += NT)
+                {
+                    const uint32_t s = u / VPR, xv = u % VPR;
+                    if(xv * VS < cnt)
+                    {
+                        Vec<T, VS> o;
+#pragma unroll
+                        for(int e = 0; e < VS; ++e)
+                            o.v[e] = tile[s * PITCH + xv * VS + e];
+                        *reinterpret_cast<Vec<T, VS>*>(B + boff + xv * VS + s * a.row_stride) = o;
+                    }
                 }
             }
         }
@@ -278,6 +428,41 @@ namespace hiptk
             return -1;
         }
 
+        constexpr int STRIP_MAX_SHORT = 16; // longest "short" mode the strip kernels take
+
+        template <typename T>
+        constexpr int strip_len()
+        {
+            return sizeof(T) == 4 ? 512 : 1024;
+        }
+
+        template <typename T, int VMAX>
+        int launch_strip(bool linear_write, int vl, int vs, const SArgs& a, uint32_t grid, hipStream_t s)
+        {
+            constexpr int TL  = strip_len<T>();
+            const size_t  lds = (size_t)a.e_s * (TL + 1) * sizeof(T);
+#define HIPTK_STRIP_CASE(L, S)                                                                                      \
+    if(vl == L && vs == S)                                                                                          \
+    {                                                                                                               \
+        if(linear_write)                                                                                            \
+            hipLaunchKernelGGL((permute_strip_kernel<T, TL, L, S, true>), dim3(grid), dim3(PERM_THREADS), lds, s, a);  \
+        else                                                                                                        \
+            hipLaunchKernelGGL((permute_strip_kernel<T, TL, L, S, false>), dim3(grid), dim3(PERM_THREADS), lds, s, a); \
+        return (int)hipGetLastError();                                                                              \
+    }
+            HIPTK_STRIP_CASE(1, 1)
+            HIPTK_STRIP_CASE(1, 2)
+            HIPTK_STRIP_CASE(1, VMAX)
+            HIPTK_STRIP_CASE(2, 1)
+            HIPTK_STRIP_CASE(2, 2)
+            HIPTK_STRIP_CASE(2, VMAX)
+            HIPTK_STRIP_CASE(VMAX, 1)
+            HIPTK_STRIP_CASE(VMAX, 2)
+            HIPTK_STRIP_CASE(VMAX, VMAX)
+#undef HIPTK_STRIP_CASE
+            return -1;
+        }
+
         bool vec_allowed(int elem_bytes, int v)
         {
             return v == 1 || v == 2 || (elem_bytes == 4 ? v == 4 : v == 8);
@@ -375,6 +560,17 @@ extern "C" const char* hiptk_permute_kernel_name(const hiptk_permute_t* p)
         break;
     }
     case HIPTK_PERM_GATHER: snprintf(name, sizeof(name), "permute_gather_%s", type_tag(p->elem_bytes)); break;
+    case HIPTK_PERM_STRIP:
+        if((p->tile == 0 || p->tile == 1) && vec_allowed(p->elem_bytes, p->vec_r) && vec_allowed(p->elem_bytes, p->vec_w))
+            snprintf(name,
+                     sizeof(name),
+                     "permute_strip_%s_%s_%d_r%d_w%d",
+                     type_tag(p->elem_bytes),
+                     p->tile == 0 ? "linear_write" : "linear_read",
+                     p->elem_bytes == 4 ? strip_len<float>() : strip_len<_Float16>(),
+                     p->vec_r,
+                     p->vec_w);
+        break;
     default: break;
     }
     return name;
@@ -472,6 +668,7 @@ extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, v
         a.b_j   = (uint32_t)p->b_stride[mj];
         a.nt_i  = (a.e_i + t.ti - 1) / t.ti;
         a.nt_j  = (a.e_j + t.tj - 1) / t.tj;
+        a.group = (uint32_t)std::max(1, std::min(p->group, (int32_t)a.nt_j));
         a.alpha = p->alpha;
         a.op_a  = p->op_a;
         a.op_b  = p->op_b;
@@ -490,6 +687,73 @@ extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, v
             return HIPTK_ERR_ARG;
         rc = p->elem_bytes == 4 ? launch_tile_shape<float, 4>(p->tile, transpose, vr, vw, a, (uint32_t)grid, s)
                                 : launch_tile_shape<_Float16, 8>(p->tile, transpose, vr, vw, a, (uint32_t)grid, s);
+    }
+    else if(p->kernel == HIPTK_PERM_STRIP)
+    {
+        // tile == 0: long mode 0 (A's fastest), short mode mode_j (B's fastest), B holds mode 0
+        //            right after it; the strip is linear in B.
+        // tile == 1: short mode 0 (A's fastest) with long mode mode_j right after it in A and
+        //            fastest in B; the strip is linear in A.
+        const int  mj           = p->mode_j;
+        const bool linear_write = p->tile == 0;
+        if(p->rank < 2 || p->mode_i != 0 || mj < 1 || mj >= p->rank || (p->tile != 0 && p->tile != 1))
+            return HIPTK_ERR_ARG;
+        if(!vec_allowed(p->elem_bytes, p->vec_r) || !vec_allowed(p->elem_bytes, p->vec_w))
+            return HIPTK_ERR_NO_KERNEL;
+        const int ms = linear_write ? mj : 0, ml = linear_write ? 0 : mj; // short, long
+        if(p->extent[ms] > STRIP_MAX_SHORT || p->b_stride[mj] != 1)
+            return HIPTK_ERR_ARG;
+        if(linear_write ? p->b_stride[0] != p->extent[mj] : p->a_stride[mj] != p->extent[0])
+            return HIPTK_ERR_ARG;
+        // vector preconditions: the linear side needs whole vectors in every strip and aligned
+        // strip starts, the row side whole vectors in every row
+        const int     vr = p->vec_r, vw = p->vec_w;
+        const int     vl = linear_write ? vw : vr, vs = linear_write ? vr : vw;
+        const int64_t run = (int64_t)p->extent[0] * p->extent[mj];
+        const int32_t* lin_stride = linear_write ? p->b_stride : p->a_stride;
+        const int32_t* row_stride = linear_write ? p->a_stride : p->b_stride;
+        if(run % vl != 0 || p->extent[ml] % vs != 0)
+            return HIPTK_ERR_ARG;
+        for(int d = 1; d < p->rank; ++d)
+        {
+            if(d != mj && lin_stride[d] % vl != 0)
+                return HIPTK_ERR_ARG;
+            if((d != mj || linear_write) && row_stride[d] % vs != 0)
+                return HIPTK_ERR_ARG;
+        }
+        if(!linear_write && p->b_stride[0] % vs != 0)
+            return HIPTK_ERR_ARG;
+        if(!aligned(A, vr * p->elem_bytes) || !aligned(B, vw * p->elem_bytes))
+            return HIPTK_ERR_ARG;
+
+        const int TL = p->elem_bytes == 4 ? strip_len<float>() : strip_len<_Float16>();
+        SArgs     a;
+        memset(&a, 0, sizeof(a));
+        a.A          = A;
+        a.B          = B;
+        a.e_s        = (uint32_t)p->extent[ms];
+        a.e_l        = (uint32_t)p->extent[ml];
+        a.row_stride = (uint32_t)(linear_write ? p->a_stride[mj] : p->b_stride[0]);
+        a.magic      = (uint32_t)((uint64_t(1) << 32) / a.e_s) + 1u;
+        a.nt         = (a.e_l + TL - 1) / TL;
+        a.alpha      = p->alpha;
+        a.op_a       = p->op_a;
+        a.op_b       = p->op_b;
+        int64_t grid = a.nt;
+        for(int d = 1; d < p->rank; ++d)
+        {
+            if(d == mj)
+                continue;
+            a.bext[a.nb] = (uint32_t)p->extent[d];
+            a.ba[a.nb]   = (uint32_t)p->a_stride[d];
+            a.bb[a.nb]   = (uint32_t)p->b_stride[d];
+            ++a.nb;
+            grid *= p->extent[d];
+        }
+        if(grid >= (int64_t(1) << 31))
+            return HIPTK_ERR_ARG;
+        rc = p->elem_bytes == 4 ? launch_strip<float, 4>(linear_write, vl, vs, a, (uint32_t)grid, s)
+                                : launch_strip<_Float16, 8>(linear_write, vl, vs, a, (uint32_t)grid, s);
     }
     else
         return HIPTK_ERR_NO_KERNEL;

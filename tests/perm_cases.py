@@ -51,10 +51,16 @@ LARGE = [
     ([40, 50, 60], [0, 2, 1]),
     ([1024, 20, 4], [1, 0, 2]),           # long i, short j
     ([20, 1024, 4], [1, 0, 2]),           # short i, long j
-    ([6, 70, 80], [1, 0, 2]),             # short fastest mode: gather
+    ([6, 70, 80], [2, 1, 0]),             # short fastest mode: gather
     ([8, 16, 8, 16, 8, 16], [5, 3, 1, 4, 2, 0]),
     ([32, 8, 16, 4, 8, 4], [1, 0, 3, 2, 5, 4]),
     ([512, 512], [1, 0]),
+    ([3000, 3, 5], [1, 0, 2]),            # short B-fastest mode: strip, linear in B
+    ([3, 3000, 5], [1, 0, 2]),            # short A-fastest mode: strip, linear in A
+    ([1001, 7, 3], [1, 0, 2]),            # odd extents: scalar strip
+    ([16, 1030, 2], [1, 0, 2]),
+    ([2050, 16, 3], [1, 0, 2]),
+    ([2, 4096, 3, 2], [1, 0, 3, 2]),
 ]
 
 
