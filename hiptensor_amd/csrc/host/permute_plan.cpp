@@ -12,8 +12,8 @@ namespace hipta
             int ti, tj;
         };
         // the kernel layer's tile shapes (elements): square, long along i, long along j
-        constexpr Tile TILES4[3] = {{64, 64}, {256, 16}, {16, 256}};
-        constexpr Tile TILES2[3] = {{128, 128}, {512, 32}, {32, 512}};
+        constexpr Tile TILES4[4] = {{64, 64}, {256, 16}, {16, 256}, {128, 128}};
+        constexpr Tile TILES2[4] = {{128, 128}, {512, 32}, {32, 512}, {256, 128}};
 
         bool alignedTo(const void* p, int64_t bytes)
         {
@@ -169,10 +169,10 @@ namespace hipta
                 jB = d;
 
         // layout-admissible kernels: TILED needs differing fastest modes, ROWS a shared one,
-        // STRIP a tile mode of at most 16 elements whose partner follows it directly in memory
+        // STRIP a tile mode of at most 64 elements whose partner follows it directly in memory
         const bool shared = jB == 0;
-        const bool stripJ = !shared && ext[jB] <= 16 && bs[0] == ext[jB]; // short j, B holds i right after it
-        const bool stripI = !shared && ext[0] <= 16 && jB == 1 && !stripJ; // short i, A holds j right after it
+        const bool stripJ = !shared && ext[jB] <= 64 && ext[jB] <= ext[0] && bs[0] == ext[jB]; // short j, B holds i right after it
+        const bool stripI = !shared && ext[0] <= 64 && jB == 1 && !stripJ; // short i, A holds j right after it
         int        kernel;
         if(tune.kernel == HIPTK_PERM_GATHER)
             kernel = HIPTK_PERM_GATHER;
@@ -182,7 +182,7 @@ namespace hipta
             kernel = shared ? HIPTK_PERM_ROWS : HIPTK_PERM_TILED;
         else if(count <= 16384)
             kernel = HIPTK_PERM_GATHER; // a launch's worth of latency either way
-        else if((stripJ && ext[0] >= 64) || (stripI && ext[jB] >= 64))
+        else if((stripJ && ext[0] >= 256) || (stripI && ext[jB] >= 256))
             kernel = HIPTK_PERM_STRIP;
         else if(shared)
             kernel = ext[0] >= 16 ? HIPTK_PERM_ROWS : HIPTK_PERM_GATHER;
@@ -232,7 +232,18 @@ namespace hipta
             out.vec_r         = vr;
             out.vec_w         = pickVec(in.elem_bytes, cap, ext[jB], bOthers, in.B, false);
             const int order[] = {0, 1, 2};
-            out.tile          = tune.tile >= 0 && tune.tile <= 2 ? tune.tile : pickTile(in.elem_bytes, ext[0], ext[jB], order);
+            out.tile          = tune.tile >= 0 && tune.tile <= 3 ? tune.tile : pickTile(in.elem_bytes, ext[0], ext[jB], order);
+            // The 64 KiB tile doubles the contiguous run (on both sides for f32: 512 bytes; on A's
+            // side for f16), which HBM rewards as long as the tile grid does not lose much more
+            // of it at the edges.
+            if(tune.tile < 0)
+            {
+                const Tile*  ts   = in.elem_bytes == 4 ? TILES4 : TILES2;
+                const double cur  = coverage(ext[0], ts[out.tile].ti) * coverage(ext[jB], ts[out.tile].tj);
+                const double big  = coverage(ext[0], ts[3].ti) * coverage(ext[jB], ts[3].tj);
+                if(big >= 0.9 * cur)
+                    out.tile = 3;
+            }
         }
         else
         {

@@ -80,15 +80,21 @@ namespace hiptk
             return y;
         }
 
-        template <typename T, int TI, int TJ, int VR, int VW, bool TRANSPOSE>
-        __global__ __launch_bounds__(PERM_THREADS) void permute_tile_kernel(PArgs a)
+        // The tile in LDS is [TJ][TI].  Column reads must spread over the 64 banks: the small
+        // tiles pad each row by one element; the 64 KiB tiles have no room for padding and XOR
+        // the column index with the row number instead (in units of one 32-bit word).
+        template <typename T, int TI, int TJ, int VR, int VW, bool TRANSPOSE, int NT = PERM_THREADS, bool SWZ = false>
+        __global__ __launch_bounds__(NT) void permute_tile_kernel(PArgs a)
         {
-            constexpr int NT    = PERM_THREADS;
-            constexpr int PITCH = TI + 1; // odd pitch: column reads spread over the banks
+            constexpr int PITCH = SWZ ? TI : TI + 4 / (int)sizeof(T); // an odd number of 32-bit words
             constexpr int VPR   = TI / VR; // vectors per tile row
             constexpr int NRV   = VPR * TJ / NT; // vectors per thread, read side
             static_assert(TI % VR == 0 && (VPR * TJ) % NT == 0 && NRV >= 1, "read shape");
+            static_assert(!SWZ || TI * sizeof(T) >= 256, "a swizzled row spans all 64 banks");
             __shared__ T tile[TRANSPOSE ? TJ * PITCH : 1];
+            auto         at = [](uint32_t j, uint32_t i) -> uint32_t {
+                return SWZ ? j * TI + (i ^ ((j & 63u) * (4u / sizeof(T)))) : j * PITCH + i;
+            };
 
             const T* __restrict__ A = static_cast<const T*>(a.A);
             T* __restrict__ B       = static_cast<T*>(a.B);
@@ -125,11 +131,12 @@ namespace hiptk
 #pragma unroll
             for(int k = 0; k < NRV; ++k)
             {
+                // Lanes outside the extents load the tile's first element instead of branching
+                // around the load: a branch per load would make the compiler wait for each load
+                // before issuing the next, and the loads must all be in flight together.
                 const uint32_t v = tid + k * NT, iv = v % VPR, j = v / VPR;
                 const bool     ok = (i0 + iv * VR < a.e_i) && (j0 + j < a.e_j);
-                r[k]              = Vec<T, VR>{};
-                if(ok)
-                    r[k] = *reinterpret_cast<const Vec<T, VR>*>(A + aoff + iv * VR + j * a.a_j);
+                r[k] = *reinterpret_cast<const Vec<T, VR>*>(A + aoff + (ok ? iv * VR + j * a.a_j : 0u));
             }
 #pragma unroll
             for(int k = 0; k < NRV; ++k)
@@ -142,7 +149,7 @@ namespace hiptk
                 {
 #pragma unroll
                     for(int e = 0; e < VR; ++e)
-                        tile[j * PITCH + iv * VR + e] = r[k].v[e];
+                        tile[at(j, iv * VR + e)] = r[k].v[e];
                 }
                 else
                 {
@@ -165,7 +172,7 @@ namespace hiptk
                     Vec<T, VW>     o;
 #pragma unroll
                     for(int e = 0; e < VW; ++e)
-                        o.v[e] = tile[(jv * VW + e) * PITCH + i];
+                        o.v[e] = tile[at(jv * VW + e, i)];
                     if(ok)
                         *reinterpret_cast<Vec<T, VW>*>(B + boff + jv * VW + i * a.b_i) = o;
                 }
@@ -191,12 +198,30 @@ namespace hiptk
         // It is read in e_s rows of A and written linearly.  !LINEAR_WRITE is the mirror image:
         // the short mode is A's fastest with the long one right after it; the strip is read
         // linearly from A and written in e_s rows of B.
+        // Position of a linear index v of a strip: v = x * e_s + s.  One division per thread finds
+        // the first position; afterwards the walk only adds (32-bit integer multiplies and
+        // divides run at a quarter of the add rate, and this kernel has one per element to spare).
+        struct StripPos
+        {
+            uint32_t s, x;
+            __device__ void advance(uint32_t ds, uint32_t dx, uint32_t e_s)
+            {
+                s += ds;
+                x += dx;
+                if(s >= e_s)
+                {
+                    s -= e_s;
+                    ++x;
+                }
+            }
+        };
+
         template <typename T, int TL, int VL, int VS, bool LINEAR_WRITE>
         __global__ __launch_bounds__(PERM_THREADS) void permute_strip_kernel(SArgs a)
         {
             constexpr int NT    = PERM_THREADS;
-            constexpr int U     = 4; // loads in flight per thread
-            constexpr int PITCH = TL + 1;
+            constexpr int U     = 8; // loads in flight per thread: a whole 32 KiB strip of full vectors
+            constexpr int PITCH = TL + 4 / (int)sizeof(T); // an odd number of 32-bit words: rows start in different banks
             constexpr int VPR   = TL / VS; // row vectors per strip row
             static_assert(TL % VS == 0 && TL % VL == 0, "strip shape");
             extern __shared__ unsigned char strip_smem[];
@@ -223,6 +248,13 @@ namespace hiptk
             const uint32_t nrv   = a.e_s * VPR; // row vectors of the strip (tail rows included)
             const uint32_t nlv   = cnt * a.e_s / VL; // linear vectors of the strip
 
+            // the walk over linear vectors u = tid, tid + NT, ...: first element v = u * VL
+            StripPos pos;
+            pos.x = __umulhi(tid * VL, a.magic);
+            pos.s = tid * VL - pos.x * a.e_s;
+            const uint32_t step_x = __umulhi((uint32_t)(NT * VL), a.magic); // scalar
+            const uint32_t step_s = NT * VL - step_x * a.e_s;
+
             if constexpr(LINEAR_WRITE)
             {
                 aoff += l0;
@@ -233,10 +265,10 @@ namespace hiptk
 #pragma unroll
                     for(int k = 0; k < U; ++k)
                     {
+                        // out-of-range lanes load the strip's first element (no branch: see the tile kernel)
                         const uint32_t u = u0 + tid + k * NT, s = u / VPR, xv = u % VPR;
-                        r[k]             = Vec<T, VS>{};
-                        if(u < nrv && xv * VS < cnt)
-                            r[k] = *reinterpret_cast<const Vec<T, VS>*>(A + aoff + xv * VS + s * a.row_stride);
+                        const bool     ok = u < nrv && xv * VS < cnt;
+                        r[k] = *reinterpret_cast<const Vec<T, VS>*>(A + aoff + (ok ? xv * VS + s * a.row_stride : 0u));
                     }
 #pragma unroll
                     for(int k = 0; k < U; ++k)
@@ -254,13 +286,15 @@ namespace hiptk
                 for(uint32_t u = tid; u < nlv; u += NT)
                 {
                     Vec<T, VL> o;
+                    StripPos   q = pos;
 #pragma unroll
                     for(int e = 0; e < VL; ++e)
                     {
-                        const uint32_t v = u * VL + e, x = __umulhi(v, a.magic), sidx = v - x * a.e_s;
-                        o.v[e]           = tile[sidx * PITCH + x];
+                        o.v[e] = tile[q.s * PITCH + q.x];
+                        q.advance(1, 0, a.e_s);
                     }
                     *reinterpret_cast<Vec<T, VL>*>(B + boff + u * VL) = o;
+                    pos.advance(step_s, step_x, a.e_s);
                 }
             }
             else
@@ -274,9 +308,7 @@ namespace hiptk
                     for(int k = 0; k < U; ++k)
                     {
                         const uint32_t u = u0 + tid + k * NT;
-                        r[k]             = Vec<T, VL>{};
-                        if(u < nlv)
-                            r[k] = *reinterpret_cast<const Vec<T, VL>*>(A + aoff + u * VL);
+                        r[k] = *reinterpret_cast<const Vec<T, VL>*>(A + aoff + (u < nlv ? u * VL : 0u));
                     }
 #pragma unroll
                     for(int k = 0; k < U; ++k)
@@ -284,13 +316,15 @@ namespace hiptk
                         const uint32_t u = u0 + tid + k * NT;
                         if(u < nlv)
                         {
+                            StripPos q = pos;
 #pragma unroll
                             for(int e = 0; e < VL; ++e)
                             {
-                                const uint32_t v = u * VL + e, x = __umulhi(v, a.magic), sidx = v - x * a.e_s;
-                                tile[sidx * PITCH + x] = element_op(r[k].v[e], alpha, a.op_a, a.op_b);
+                                tile[q.s * PITCH + q.x] = element_op(r[k].v[e], alpha, a.op_a, a.op_b);
+                                q.advance(1, 0, a.e_s);
                             }
                         }
+                        pos.advance(step_s, step_x, a.e_s);
                     }
                 }
                 __syncthreads();
@@ -323,9 +357,7 @@ namespace hiptk
             for(int u = 0; u < U; ++u)
             {
                 const uint32_t idx = base + u * PERM_THREADS;
-                r[u]               = Vec<T, V>{};
-                if(idx < nvec)
-                    r[u] = A[idx];
+                r[u]               = A[idx < nvec ? idx : 0u];
             }
 #pragma unroll
             for(int u = 0; u < U; ++u)
@@ -362,24 +394,34 @@ namespace hiptk
         {
             int ti, tj;
         };
-        // element tiles per element size: square, long along i, long along j
-        constexpr TileShape TILES4[3] = {{64, 64}, {256, 16}, {16, 256}};
-        constexpr TileShape TILES2[3] = {{128, 128}, {512, 32}, {32, 512}};
+        // element tiles per element size: square, long along i, long along j, and a 64 KiB tile
+        // (512 threads, TILED only) whose rows and columns are twice as long as the square's
+        constexpr int       NUM_TILES         = 4;
+        constexpr TileShape TILES4[NUM_TILES] = {{64, 64}, {256, 16}, {16, 256}, {128, 128}};
+        constexpr TileShape TILES2[NUM_TILES] = {{128, 128}, {512, 32}, {32, 512}, {256, 128}};
 
-        template <typename T, int TI, int TJ, int VR, int VW, bool TR>
+        template <typename T, int TI, int TJ, int VR, int VW, bool TR, bool BIG>
         int launch_tile(const PArgs& a, uint32_t grid, hipStream_t s)
         {
-            hipLaunchKernelGGL((permute_tile_kernel<T, TI, TJ, VR, VW, TR>), dim3(grid), dim3(PERM_THREADS), 0, s, a);
+            if constexpr(BIG)
+            {
+                if constexpr(TR)
+                    hipLaunchKernelGGL((permute_tile_kernel<T, TI, TJ, VR, VW, true, 512, true>), dim3(grid), dim3(512), 0, s, a);
+                else
+                    return -1;
+            }
+            else
+                hipLaunchKernelGGL((permute_tile_kernel<T, TI, TJ, VR, VW, TR>), dim3(grid), dim3(PERM_THREADS), 0, s, a);
             return (int)hipGetLastError();
         }
 
-        template <typename T, int TI, int TJ, int VMAX>
+        template <typename T, int TI, int TJ, int VMAX, bool BIG = false>
         int launch_tile_vec(bool transpose, int vr, int vw, const PArgs& a, uint32_t grid, hipStream_t s)
         {
-#define HIPTK_PERM_CASE(R, W)                                           \
-    if(vr == R && vw == W)                                              \
-        return transpose ? launch_tile<T, TI, TJ, R, W, true>(a, grid, s) \
-                         : (R == W ? launch_tile<T, TI, TJ, R, R, false>(a, grid, s) : -1);
+#define HIPTK_PERM_CASE(R, W)                                                   \
+    if(vr == R && vw == W)                                                      \
+        return transpose ? launch_tile<T, TI, TJ, R, W, true, BIG>(a, grid, s)   \
+                         : (R == W ? launch_tile<T, TI, TJ, R, R, false, BIG>(a, grid, s) : -1);
             HIPTK_PERM_CASE(1, 1)
             HIPTK_PERM_CASE(1, 2)
             HIPTK_PERM_CASE(1, VMAX)
@@ -402,6 +444,7 @@ namespace hiptk
             case 0: return launch_tile_vec<T, TS[0].ti, TS[0].tj, VMAX>(transpose, vr, vw, a, grid, s);
             case 1: return launch_tile_vec<T, TS[1].ti, TS[1].tj, VMAX>(transpose, vr, vw, a, grid, s);
             case 2: return launch_tile_vec<T, TS[2].ti, TS[2].tj, VMAX>(transpose, vr, vw, a, grid, s);
+            case 3: return launch_tile_vec<T, TS[3].ti, TS[3].tj, VMAX, true>(transpose, vr, vw, a, grid, s);
             default: return -1;
             }
         }
@@ -428,19 +471,20 @@ namespace hiptk
             return -1;
         }
 
-        constexpr int STRIP_MAX_SHORT = 16; // longest "short" mode the strip kernels take
+        // Strips hold e_s rows of TL elements in LDS (about 32 KiB at most): 2 KiB rows while the
+        // short mode has at most 8 elements, 512-byte rows up to 64.
+        constexpr int STRIP_MAX_SHORT = 64;
+        constexpr int STRIP_WIDE_MAX  = 8;
 
-        template <typename T>
-        constexpr int strip_len()
+        constexpr int strip_len(int elem_bytes, int e_s)
         {
-            return sizeof(T) == 4 ? 512 : 1024;
+            return (e_s <= STRIP_WIDE_MAX ? 2048 : 512) / elem_bytes;
         }
 
-        template <typename T, int VMAX>
-        int launch_strip(bool linear_write, int vl, int vs, const SArgs& a, uint32_t grid, hipStream_t s)
+        template <typename T, int VMAX, int TL>
+        int launch_strip_len(bool linear_write, int vl, int vs, const SArgs& a, uint32_t grid, hipStream_t s)
         {
-            constexpr int TL  = strip_len<T>();
-            const size_t  lds = (size_t)a.e_s * (TL + 1) * sizeof(T);
+            const size_t lds = (size_t)a.e_s * (TL * sizeof(T) + 4);
 #define HIPTK_STRIP_CASE(L, S)                                                                                      \
     if(vl == L && vs == S)                                                                                          \
     {                                                                                                               \
@@ -461,6 +505,14 @@ namespace hiptk
             HIPTK_STRIP_CASE(VMAX, VMAX)
 #undef HIPTK_STRIP_CASE
             return -1;
+        }
+
+        template <typename T, int VMAX>
+        int launch_strip(bool linear_write, int vl, int vs, const SArgs& a, uint32_t grid, hipStream_t s)
+        {
+            if(a.e_s <= (uint32_t)STRIP_WIDE_MAX)
+                return launch_strip_len<T, VMAX, strip_len(sizeof(T), 1)>(linear_write, vl, vs, a, grid, s);
+            return launch_strip_len<T, VMAX, strip_len(sizeof(T), STRIP_MAX_SHORT)>(linear_write, vl, vs, a, grid, s);
         }
 
         bool vec_allowed(int elem_bytes, int v)
@@ -543,9 +595,9 @@ extern "C" const char* hiptk_permute_kernel_name(const hiptk_permute_t* p)
     case HIPTK_PERM_TILED:
     case HIPTK_PERM_ROWS:
     {
-        if(p->tile < 0 || p->tile > 2 || !vec_allowed(p->elem_bytes, p->vec_r) || !vec_allowed(p->elem_bytes, p->vec_w))
+        if(p->tile < 0 || p->tile >= NUM_TILES || !vec_allowed(p->elem_bytes, p->vec_r) || !vec_allowed(p->elem_bytes, p->vec_w))
             break;
-        if(p->kernel == HIPTK_PERM_ROWS && p->vec_r != p->vec_w)
+        if(p->kernel == HIPTK_PERM_ROWS && (p->vec_r != p->vec_w || p->tile == 3))
             break;
         const TileShape t = (p->elem_bytes == 4 ? TILES4 : TILES2)[p->tile];
         snprintf(name,
@@ -561,13 +613,14 @@ extern "C" const char* hiptk_permute_kernel_name(const hiptk_permute_t* p)
     }
     case HIPTK_PERM_GATHER: snprintf(name, sizeof(name), "permute_gather_%s", type_tag(p->elem_bytes)); break;
     case HIPTK_PERM_STRIP:
-        if((p->tile == 0 || p->tile == 1) && vec_allowed(p->elem_bytes, p->vec_r) && vec_allowed(p->elem_bytes, p->vec_w))
+        if((p->tile == 0 || p->tile == 1) && p->mode_j >= 1 && p->mode_j < p->rank && vec_allowed(p->elem_bytes, p->vec_r)
+           && vec_allowed(p->elem_bytes, p->vec_w))
             snprintf(name,
                      sizeof(name),
                      "permute_strip_%s_%s_%d_r%d_w%d",
                      type_tag(p->elem_bytes),
                      p->tile == 0 ? "linear_write" : "linear_read",
-                     p->elem_bytes == 4 ? strip_len<float>() : strip_len<_Float16>(),
+                     strip_len(p->elem_bytes, p->extent[p->tile == 0 ? p->mode_j : 0]),
                      p->vec_r,
                      p->vec_w);
         break;
@@ -632,7 +685,7 @@ extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, v
     {
         const bool transpose = p->kernel == HIPTK_PERM_TILED;
         const int  mi = p->mode_i, mj = p->mode_j;
-        if(p->rank < 2 || mi != 0 || mj < 1 || mj >= p->rank || p->tile < 0 || p->tile > 2)
+        if(p->rank < 2 || mi != 0 || mj < 1 || mj >= p->rank || p->tile < 0 || p->tile >= NUM_TILES)
             return HIPTK_ERR_ARG;
         if(!vec_allowed(p->elem_bytes, p->vec_r) || !vec_allowed(p->elem_bytes, p->vec_w))
             return HIPTK_ERR_NO_KERNEL;
@@ -726,7 +779,7 @@ extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, v
         if(!aligned(A, vr * p->elem_bytes) || !aligned(B, vw * p->elem_bytes))
             return HIPTK_ERR_ARG;
 
-        const int TL = p->elem_bytes == 4 ? strip_len<float>() : strip_len<_Float16>();
+        const int TL = strip_len(p->elem_bytes, p->extent[ms]);
         SArgs     a;
         memset(&a, 0, sizeof(a));
         a.A          = A;

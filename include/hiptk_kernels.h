@@ -150,7 +150,7 @@ enum
     HIPTK_PERM_ROWS   = 2, /* both tensors share the fastest mode (mode_i == 0): runs of that mode
                               are copied, tiles span it and one further mode (mode_j)             */
     HIPTK_PERM_GATHER = 3, /* one thread per element of B, any layout                             */
-    HIPTK_PERM_STRIP  = 4  /* TILED with one tile mode of at most 16 elements whose partner follows it
+    HIPTK_PERM_STRIP  = 4  /* TILED with one tile mode of at most 64 elements whose partner follows it
                               directly in memory on that side: a strip of the long mode times the
                               whole short mode is one contiguous run there.  tile == 0: mode_j is the
                               short one and the run lies in B; tile == 1: mode 0 is the short one and
@@ -170,7 +170,9 @@ typedef struct hiptk_permute
     float   alpha;      /* multiplies in float for f32, rounded to half first for f16             */
     int32_t kernel;     /* HIPTK_PERM_*                                                           */
     int32_t mode_i, mode_j; /* TILED / ROWS: positions (in this struct's order) of the two tile modes */
-    int32_t tile;       /* TILED / ROWS: 0 square, 1 long along mode_i, 2 long along mode_j       */
+    int32_t tile;       /* TILED / ROWS: 0 square, 1 long along mode_i, 2 long along mode_j;
+                           TILED only: 3 a 64 KiB tile with rows and columns twice the square's;
+                           STRIP: 0 / 1, see HIPTK_PERM_STRIP                                     */
     int32_t vec_r;      /* elements per global load (1, 2, 4; 8 for f16)                          */
     int32_t vec_w;      /* elements per global store                                              */
     int32_t group;      /* TILED / ROWS: workgroups walk the tile plane in bands of this many tiles

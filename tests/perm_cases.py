@@ -61,6 +61,10 @@ LARGE = [
     ([16, 1030, 2], [1, 0, 2]),
     ([2050, 16, 3], [1, 0, 2]),
     ([2, 4096, 3, 2], [1, 0, 3, 2]),
+    ([300, 40, 3], [1, 0, 2]),            # short mode above 16: strips with 512-byte rows
+    ([64, 300, 2], [1, 0, 2]),
+    ([33, 290, 2], [1, 0, 2]),
+    ([520, 64, 2], [1, 0, 2]),
 ]
 
 

@@ -88,7 +88,7 @@ def test_large_shapes_default_selection(gpu_handle, oracle_mod, dtype, scalar):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
 @pytest.mark.parametrize("maxvec", [1, 2, 8])
 def test_every_tile_and_vector_width(gpu_handle, oracle_mod, dtype, tile, maxvec):
     names = set()
