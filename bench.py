@@ -177,6 +177,15 @@ def permutation_line(a, handle, prop):
                              "frac_hbm": ob / (rr["kernel_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBS,
                              "kernel": rr["info"]["kernel_name"], "dtype": ow["dtype"], "workload": ow["name"]}
         out["others"] = others
+    if a.copy_calibration:
+        import torch
+
+        src = torch.ones(1 << 28, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["copy_calibration"] = {"bytes_read": 1 << 28, "bytes_written": 1 << 28, "launches": 3}
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline_permutation(w)
     return out

@@ -1,4 +1,4 @@
-"""Reader for the reference's contraction test matrices (YAML).
+"""Reader for the reference's contraction and permutation test matrices (YAML).
 
 The reference drives its gtest suites from files such as
 test/01_contraction/configs/validation/bilinear_test_params_rank3.yaml; their keys are
@@ -14,6 +14,12 @@ mapped in test/llvm/yaml_parser_config.cpp:235-270 ("Log Level", "Tensor Data Ty
 
 `to_workload` turns one expanded case into the workload dictionary the rest of this
 package uses (hiptensor_amd.workloads), so a whole file can be run through the public API.
+
+The permutation suites (test/02_permutation/configs/**/rank{2..6}_test_params.yaml) use their
+own keys, mapped in test/llvm/yaml_parser_config.cpp:322-363 ("Log Level", "Tensor Data Types"
+as [data type, scalar type] rows, "Alphas", "Lengths", "Permuted Dims", "Operators" as [A, B]
+rows); the gtest runs their cartesian product (test/02_permutation/permutation_test_helpers.hpp).
+`load_permutation` / `expand_permutation` / `to_permutation_workload` cover them.
 Nothing here touches a device.
 """
 import itertools
@@ -174,3 +180,74 @@ def to_workload(case, name=""):
     w["workspace_pref"] = WORKSPACE[case["workspace_pref"]]
     w["default_strides"] = not explicit
     return w
+
+
+# ---------------------------------------------------------------------------
+# Permutation matrices
+# ---------------------------------------------------------------------------
+PERM_REQUIRED = ("Log Level", "Tensor Data Types", "Alphas", "Lengths", "Permuted Dims", "Operators")
+UNARY = {"HIPTENSOR_OP_IDENTITY": api.HIPTENSOR_OP_IDENTITY, "HIPTENSOR_OP_SQRT": api.HIPTENSOR_OP_SQRT}
+
+
+def is_permutation_document(doc):
+    return isinstance(doc, dict) and "Permuted Dims" in doc
+
+
+def load_permutation(path):
+    with open(path) as f:
+        return normalise_permutation(yaml.safe_load(f), str(path))
+
+
+def loads_permutation(text, name="<string>"):
+    return normalise_permutation(yaml.safe_load(text), name)
+
+
+def normalise_permutation(doc, name):
+    """Validated like the reference's reader (yaml_parser_config.cpp:338-362: no empty Lengths,
+    Alphas, Permuted Dims or Operators) and the fixture's own expectations
+    (test/02_permutation/permutation_test.cpp:166-180: ranks 2..6, two operators, two types)."""
+    if not isinstance(doc, dict):
+        raise ConfigError(f"{name}: not a mapping")
+    for k in PERM_REQUIRED:
+        if k not in doc:
+            raise ConfigError(f"{name}: missing key '{k}'")
+    for k in ("Lengths", "Alphas", "Permuted Dims", "Operators"):
+        if not doc[k]:
+            raise ConfigError(f"{name}: Error: Empty {k}")
+    out = {
+        "name": name,
+        "data_types": [list(r) for r in doc["Tensor Data Types"]],
+        "alphas": [float(a) for a in doc["Alphas"]],
+        "lengths": [list(l) for l in doc["Lengths"]],
+        "permuted_dims": [list(p) for p in doc["Permuted Dims"]],
+        "operators": [list(o) for o in doc["Operators"]],
+    }
+    for row in out["data_types"]:
+        if len(row) != 2 or any(DTYPE.get(t) not in ("f16", "f32") for t in row):
+            raise ConfigError(f"{name}: bad Tensor Data Types row {row} (two of HIP_R_16F / HIP_R_32F)")
+    for row in out["operators"]:
+        if len(row) != 2 or any(o not in UNARY for o in row):
+            raise ConfigError(f"{name}: bad Operators row {row}")
+    for l in out["lengths"]:
+        if not 2 <= len(l) <= 6:
+            raise ConfigError(f"{name}: lengths {l}: the permutation suites cover ranks 2..6")
+    for p in out["permuted_dims"]:
+        if sorted(p) != list(range(len(p))):
+            raise ConfigError(f"{name}: {p} is not an order of 0..{len(p) - 1}")
+    return out
+
+
+def expand_permutation(cfg):
+    """Cartesian product in the reference's nesting order; (lengths, order) pairs of different
+    rank are skipped."""
+    keys = ("data_types", "lengths", "permuted_dims", "alpha", "operators")
+    lists = (cfg["data_types"], cfg["lengths"], cfg["permuted_dims"], cfg["alphas"], cfg["operators"])
+    return [dict(zip(keys, v)) for v in itertools.product(*lists) if len(v[1]) == len(v[2])]
+
+
+def to_permutation_workload(case, name=""):
+    """Workload for one expanded case: mode k of B is mode permuted_dims[k] of A
+    (test/02_permutation/permutation_test.cpp:268-276)."""
+    dt, scalar = (DTYPE[t] for t in case["data_types"])
+    oa, ob = (UNARY[o] for o in case["operators"])
+    return wl.permutation(dt, case["lengths"], case["permuted_dims"], case["alpha"], scalar, oa, ob, name=name)

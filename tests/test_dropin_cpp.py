@@ -9,21 +9,23 @@ from hiptensor_amd import _lib
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BIN = os.path.join(ROOT, "tests", "cpp", "bin", "dropin_contraction")
+BIN_PERM = os.path.join(ROOT, "tests", "cpp", "bin", "dropin_permutation")
 REF_SAMPLES = "/root/reference/samples"
 HIPCC = "/opt/rocm/bin/hipcc"
 
 
 def build_dropin():
     os.makedirs(os.path.dirname(BIN), exist_ok=True)
-    subprocess.run([HIPCC, "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"),
-                    os.path.join(ROOT, "tests", "cpp", "dropin_contraction.cpp"), "-o", BIN,
-                    "-L" + os.path.dirname(_lib.LIB_PATH), "-lhiptensor_amd",
-                    "-Wl,-rpath,$ORIGIN/../../../hiptensor_amd/lib"], check=True, capture_output=True)
+    for out in (BIN, BIN_PERM):
+        src = os.path.join(ROOT, "tests", "cpp", os.path.basename(out) + ".cpp")
+        subprocess.run([HIPCC, "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"), src, "-o", out,
+                        "-L" + os.path.dirname(_lib.LIB_PATH), "-lhiptensor_amd",
+                        "-Wl,-rpath,$ORIGIN/../../../hiptensor_amd/lib"], check=True, capture_output=True)
 
 
 def test_dropin_program_builds_and_links():
     build_dropin()
-    assert os.path.exists(BIN)
+    assert os.path.exists(BIN) and os.path.exists(BIN_PERM)
 
 
 @pytest.mark.skipif(not os.path.isdir(REF_SAMPLES), reason="reference tree not mounted")
@@ -44,9 +46,28 @@ def test_reference_samples_compile_unchanged(sample, tmp_path):
     assert out.exists()
 
 
+@pytest.mark.skipif(not os.path.isdir(REF_SAMPLES), reason="reference tree not mounted")
+def test_reference_permutation_sample_compiles_unchanged(tmp_path):
+    """samples/02_permutation/permutation.cpp against these headers and this library."""
+    src = os.path.join(REF_SAMPLES, "02_permutation", "permutation.cpp")
+    out = tmp_path / "permutation"
+    subprocess.run([HIPCC, "-std=c++17", "-O0", "-I" + os.path.join(ROOT, "include"), "-I" + REF_SAMPLES, src,
+                    "-o", str(out), "-L" + os.path.dirname(_lib.LIB_PATH), "-lhiptensor_amd"],
+                   check=True, capture_output=True)
+    assert out.exists()
+
+
 @pytest.mark.gpu
 def test_dropin_program_runs():
     assert os.path.exists(BIN), "tests/cpp/bin/dropin_contraction is not built (build() makes it)"
     r = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0 and "dropin_contraction: ok" in r.stdout
+
+
+@pytest.mark.gpu
+def test_dropin_permutation_program_runs():
+    assert os.path.exists(BIN_PERM), "tests/cpp/bin/dropin_permutation is not built (build() makes it)"
+    r = subprocess.run([BIN_PERM], capture_output=True, text=True, timeout=120)
+    print(r.stdout, r.stderr, flush=True)
+    assert r.returncode == 0 and "dropin_permutation: ok" in r.stdout

@@ -30,3 +30,17 @@ def test_validation_document(gpu_handle, oracle_mod, name):
         assert run == ntypes * len(cfg["lengths"]) * (distinct_pairs + 8), (run, pairs)
     else:
         assert run == len(expanded)
+
+
+@pytest.mark.parametrize("rank", [2, 3, 4, 5, 6])
+def test_permutation_validation_document(gpu_handle, oracle_mod, rank):
+    """The permutation matrix of one rank (test/02_permutation/configs/validation), read from
+    its YAML schema: every case for ranks 2 and 3, every 5th / 23rd / 131st above."""
+    from run_yaml_config import run_permutation_cases
+
+    cfg = tc.loads_permutation(yaml_matrix.permutation_document(rank), f"permutation_rank{rank}")
+    expanded = tc.expand_permutation(cfg)
+    thin = {2: 1, 3: 1, 4: 5, 5: 23, 6: 131}[rank]
+    run = run_permutation_cases(gpu_handle, oracle_mod, expanded, f"permutation_rank{rank}", thin)
+    print(f"[case] permutation rank {rank}: {len(expanded)} expanded, {run} run", flush=True)
+    assert run == (len(expanded) + thin - 1) // thin

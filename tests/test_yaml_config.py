@@ -137,3 +137,56 @@ def test_reads_the_reference_files(host_handle, oracle_mod):
             b = oracle_mod.ref_contract(w, inp["A"], inp["B"], inp["C"])
             assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), key
         assert len(done) == 7 * 3 * 4  # type rows x length rows x distinct (alpha, beta) pairs
+
+
+# ---- permutation matrices (test/02_permutation/configs) ----
+
+REF_PERM_CONFIGS = "/root/reference/test/02_permutation/configs"
+
+
+def test_permutation_schema_and_expansion():
+    import math
+
+    import perm_cases
+
+    for rank in (2, 3, 4):
+        cfg = tc.loads_permutation(yaml_matrix.permutation_document(rank))
+        assert cfg["lengths"] == perm_cases.LENGTHS[rank] and cfg["alphas"] == perm_cases.ALPHAS
+        assert len(cfg["permuted_dims"]) == math.factorial(rank) and len(cfg["operators"]) == 4
+        exp = tc.expand_permutation(cfg)
+        assert len(exp) == 3 * len(cfg["lengths"]) * math.factorial(rank) * 3 * 4
+        w = tc.to_permutation_workload(exp[-1])
+        assert (w["dtype"], w["scalar"]) == ("f16", "f32") and w["alpha"] == 2.3
+        assert w["opA"] == w["opB"] == api.HIPTENSOR_OP_SQRT
+        assert w["lensB"] == [w["lensA"][p] for p in exp[-1]["permuted_dims"]]
+    text = yaml_matrix.permutation_document(2)
+    with pytest.raises(tc.ConfigError, match="missing key"):
+        tc.loads_permutation(text.replace("Permuted Dims:", "Permuted Dimensions:"))
+    with pytest.raises(tc.ConfigError, match="Empty Alphas"):
+        tc.loads_permutation(text.replace("Alphas:\n  - 0.0\n  - 1.0\n  - 2.3\n", "Alphas: []\n"))
+    with pytest.raises(tc.ConfigError, match="bad Tensor Data Types"):
+        tc.loads_permutation(text.replace("[ HIP_R_16F, HIP_R_32F]", "[ HIP_R_64F, HIP_R_32F]"))
+    with pytest.raises(tc.ConfigError, match="not an order"):
+        tc.loads_permutation(text.replace("  - [1, 0]", "  - [1, 1]"))
+    assert tc.is_permutation_document(__import__("yaml").safe_load(text))
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_PERM_CONFIGS), reason="reference tree not mounted")
+def test_every_reference_permutation_file_parses_and_plans(host_handle):
+    files = sorted(glob.glob(os.path.join(REF_PERM_CONFIGS, "**", "*.yaml"), recursive=True))
+    assert len(files) == 15
+    for path in files:
+        cfg = tc.load_permutation(path)
+        exp = tc.expand_permutation(cfg)
+        assert exp, path
+        for case in exp[:: max(1, len(exp) // 50)]:
+            p = wl.Permutation(host_handle, tc.to_permutation_workload(case))
+            assert p.info()["kernel_name"], (path, case)
+            p.close()
+    # the validation files are the matrix tests/perm_cases.py restates
+    import perm_cases
+
+    for rank in (2, 3, 4, 5, 6):
+        cfg = tc.load_permutation(os.path.join(REF_PERM_CONFIGS, "validation", f"rank{rank}_test_params.yaml"))
+        assert cfg["lengths"] == perm_cases.LENGTHS[rank] and cfg["alphas"] == perm_cases.ALPHAS
+        assert sorted(map(tuple, cfg["permuted_dims"])) == sorted(__import__("itertools").permutations(range(rank)))

@@ -68,3 +68,21 @@ def validation_documents():
                           [c[0] for c in cases.MODE_CASES], [c[1] for c in cases.MODE_CASES],
                           algos=ALGOS[:1], prefs=PREFS[:1])))
     return docs
+
+
+def permutation_document(rank):
+    """One rank of the permutation validation matrix in the reference's schema."""
+    import itertools
+
+    import perm_cases
+
+    inv = {v: k for k, v in {"HIPTENSOR_OP_IDENTITY": 1, "HIPTENSOR_OP_SQRT": 2}.items()}
+    hip = {"f32": "HIP_R_32F", "f16": "HIP_R_16F"}
+    out = ["---", "Log Level:       [ HIPTENSOR_LOG_LEVEL_ERROR, HIPTENSOR_LOG_LEVEL_PERF_TRACE ]", "Tensor Data Types:"]
+    out += [f"  - [ {hip[d]}, {hip[s]}]" for d, s in perm_cases.TYPE_ROWS]
+    out += ["Alphas:"] + [f"  - {a}" for a in perm_cases.ALPHAS]
+    out += ["Lengths:"] + [f"  - {_flow(l)}" for l in perm_cases.LENGTHS[rank]]
+    out += ["Operators:"] + [f"  - [{inv[a]}, {inv[b]}]" for a, b in perm_cases.OPS]
+    out += ["Permuted Dims:"] + [f"  - {_flow(list(p))}" for p in itertools.permutations(range(rank))]
+    out += ["..."]
+    return "\n".join(out) + "\n"
