@@ -155,3 +155,40 @@ def test_full_size_round_trip(gpu_handle):
     assert torch.equal(b[::7, ::5, ::3, ::11], want[::7, ::5, ::3, ::11])
     fwd.close()
     back.close()
+
+
+def test_permutation_inside_a_hip_graph(gpu_handle, oracle_mod):
+    """hiptensorPermutation is one kernel launch on the caller's stream (no allocation, no memset,
+    no synchronisation): tiled, strip and gather plans are captured into a HIP graph and replayed
+    three times with new values of A written between the replays; every replay equals the oracle."""
+    import torch
+
+    for lens, perm in (([256, 192], [1, 0]), ([3000, 3, 5], [1, 0, 2]), ([6, 70, 80], [2, 1, 0])):
+        w = wl.permutation("f32", lens, perm, 1.25)
+        A0 = wl.permutation_input(w)
+        n = A0.size
+        A = gpu_util.to_device(A0)
+        B = gpu_util.to_device(wl.nan_buffer("f32", n))
+        p = wl.Permutation(gpu_handle, w)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):  # warm-up outside the capture
+            assert p.run(A.data_ptr(), B.data_ptr(), side.cuda_stream) == 0
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            st = p.run(A.data_ptr(), B.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert st == 0
+        rng = np.random.default_rng(11)
+        for rep in range(3):
+            newA = A0.copy()
+            rng.shuffle(newA)
+            A.copy_(gpu_util.to_device(newA))
+            B.copy_(gpu_util.to_device(wl.nan_buffer("f32", n)))
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            got = B.cpu().numpy().view(np.float32)
+            assert _same(got, oracle_mod.permute(w, newA)), f"{w['name']} replay {rep}"
+        p.close()
