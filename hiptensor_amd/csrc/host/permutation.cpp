@@ -37,8 +37,8 @@ namespace
     }
 
     // HIPTENSOR_AMD_PERMUTE="kernel[,tile[,maxvec[,group]]]": kernel is auto | gather | tiled |
-    // rows | strip (tiled and rows name the same preference: whichever of the two the layout
-    // admits; strip is taken wherever a short tile mode admits it),
+    // rows | strip | grouped (tiled and rows name the same preference: whichever of the two the
+    // layout admits; strip and grouped are taken wherever the layout admits them),
     // tile is 0..2 or -1, maxvec caps the vector width, group sets the band width of the
     // workgroup order.  For tests and experiments.
     hipta::PermuteTuning tuningFromEnv()
@@ -59,6 +59,8 @@ namespace
                 t.kernel = HIPTK_PERM_TILED;
             else if(!std::strcmp(tok, "strip"))
                 t.kernel = HIPTK_PERM_STRIP;
+            else if(!std::strcmp(tok, "grouped"))
+                t.kernel = HIPTK_PERM_GROUPED;
             tok = strtok_r(nullptr, ",", &save);
         }
         if(tok)

@@ -173,7 +173,66 @@ namespace hipta
         const bool shared = jB == 0;
         const bool stripJ = !shared && ext[jB] <= 64 && ext[jB] <= ext[0] && bs[0] == ext[jB]; // short j, B holds i right after it
         const bool stripI = !shared && ext[0] <= 64 && jB == 1 && !stripJ; // short i, A holds j right after it
+        // Many short modes: no single mode gives a long run.  A tile row then spans A's two
+        // fastest modes and a tile column B's two fastest modes, where those are free.
+        // Fills `out` and returns true when that kernel applies (force: even where the plain
+        // tiles would cover the extents well).
+        auto tryGrouped = [&](bool force) -> bool {
+            if(shared || ext[0] > 128 || ext[jB] > 128)
+                return false;
+            int mi2 = (r > 1 && jB != 1) ? 1 : -1;
+            int mj2 = -1;
+            for(int d = 0; d < r; ++d)
+                if(bs[d] == ext[jB])
+                    mj2 = d;
+            if(mj2 == 0)
+                mj2 = -1;
+            if(mi2 != -1 && mi2 == mj2) // both sides want mode 1: the side with the shorter run gets it
+                (ext[jB] < ext[0] ? mi2 : mj2) = -1;
+            if(mi2 == -1 && mj2 == -1)
+                return false;
+            const int    order[] = {0, 1, 2};
+            const int    st      = pickTile(in.elem_bytes, ext[0], ext[jB], order);
+            const Tile*  ts      = in.elem_bytes == 4 ? TILES4 : TILES2;
+            const double cov     = coverage(ext[0], ts[st].ti) * coverage(ext[jB], ts[st].tj);
+            if(cov >= 0.7 && !force)
+                return false;
+            const int64_t target = 128; // elements per tile row / column aimed at
+            int64_t       ci = mi2 == -1 ? 1 : std::max<int64_t>(1, std::min<int64_t>(ext[mi2], target / ext[0]));
+            int64_t       cj = mj2 == -1 ? 1 : std::max<int64_t>(1, std::min<int64_t>(ext[mj2], target / ext[jB]));
+            auto ldsBytes = [&]() { return (ext[jB] * cj) * (ext[0] * ci + 2) * in.elem_bytes; };
+            while(ldsBytes() > 56 * 1024 && (ci > 1 || cj > 1))
+                (ext[0] * ci >= ext[jB] * cj && ci > 1 ? ci : (cj > 1 ? cj : ci)) -= 1;
+            if(ldsBytes() > 56 * 1024)
+                return false;
+            std::vector<int64_t> aOth(as.begin() + 1, as.end()), bOth;
+            for(int d = 0; d < r; ++d)
+                if(d != jB)
+                    bOth.push_back(bs[d]);
+            int vr = pickVec(in.elem_bytes, cap, ext[0], aOth, in.A, false);
+            int vw = pickVec(in.elem_bytes, cap, ext[jB], bOth, in.B, false);
+            while(vr > 1 && ext[0] * ci / vr < 2)
+                vr = vr == 8 ? 2 : vr / 2;
+            while(vw > 1 && ext[jB] * cj / vw < 2)
+                vw = vw == 8 ? 2 : vw / 2;
+            if(ext[0] * ci / vr < 2 || ext[jB] * cj / vw < 2)
+                return false;
+            out.kernel  = HIPTK_PERM_GROUPED;
+            out.mode_i  = 0;
+            out.mode_j  = jB;
+            out.mode_i2 = mi2;
+            out.mode_j2 = mj2;
+            out.chunk_i = (int32_t)ci;
+            out.chunk_j = (int32_t)cj;
+            out.vec_r   = vr;
+            out.vec_w   = vw;
+            return true;
+        };
+        out.mode_i2 = out.mode_j2 = -1;
+        out.chunk_i = out.chunk_j = 1;
         int        kernel;
+        if(tune.kernel == HIPTK_PERM_GROUPED && tryGrouped(true))
+            return PermuteStatus::OK;
         if(tune.kernel == HIPTK_PERM_GATHER)
             kernel = HIPTK_PERM_GATHER;
         else if(tune.kernel == HIPTK_PERM_STRIP && (stripJ || stripI))
@@ -186,6 +245,8 @@ namespace hipta
             kernel = HIPTK_PERM_STRIP;
         else if(shared)
             kernel = ext[0] >= 16 ? HIPTK_PERM_ROWS : HIPTK_PERM_GATHER;
+        else if(tune.tile < 0 && tryGrouped(false))
+            return PermuteStatus::OK;
         else
             kernel = (ext[0] >= 16 && ext[jB] >= 16) ? HIPTK_PERM_TILED : HIPTK_PERM_GATHER;
         out.kernel = kernel;

@@ -14,6 +14,8 @@
 //             say) when the other tile mode follows it directly in memory on that side: a
 //             workgroup takes a strip of the long mode times the whole short mode, which is one
 //             contiguous run on the short mode's side, and moves it linearly there.
+//   * GROUPED TILED for tensors of many short modes: a tile row spans A's two fastest modes, a
+//             tile column B's two fastest modes, so that runs stay long when no single mode is.
 //   * GATHER  one thread per element of B; covers tiny tensors and awkward extents.
 // Element operation per Composable Kernel's UnaryCombinedOp<Aop, Scale, Bop>
 // (ck/tensor_operation/gpu/element/combined_element_wise_operation.hpp:14-32): every step is
@@ -343,6 +345,104 @@ namespace hiptk
             }
         }
 
+        struct QArgs
+        {
+            const void* A;
+            void*       B;
+            uint32_t    e_i0, e_i1, e_j0, e_j1; // extents of the row modes (0, i2) and the column modes (j, j2); 1 if absent
+            uint32_t    c_i, c_j; // indices of i2 / j2 per tile
+            uint32_t    a_j0, a_j1, b_i0, b_i1; // A strides of the column modes, B strides of the row modes
+            uint32_t    nt_i, nt_j; // tiles along i2 and j2
+            uint32_t    pitch; // LDS row pitch in elements: an odd number of 32-bit words
+            uint32_t    m_rv, m_ej0, m_cv, m_ei0; // floor(2^32 / d) + 1 for d = TI / VR, e_j0, TJ / VW, e_i0
+            int32_t     nb;
+            uint32_t    bext[PERM_BATCH], ba[PERM_BATCH], bb[PERM_BATCH];
+            float       alpha;
+            int32_t     op_a, op_b;
+        };
+
+        // Row x of a tile is (x0, x1) = (x mod e_i0, x div e_i0) over A's two fastest modes, which
+        // are contiguous in A; column y is (y0, y1) over B's two fastest modes, contiguous in B.
+        // Rows are read along x (one run of up to e_i0 * c_i elements of A per column), the tile is
+        // parked in LDS as [y][x], and columns are written along y.
+        template <typename T, int VR, int VW>
+        __global__ __launch_bounds__(PERM_THREADS) void permute_group_kernel(QArgs a)
+        {
+            constexpr int NT = PERM_THREADS;
+            constexpr int U  = 8;
+            extern __shared__ unsigned char group_smem[];
+            T* tile = reinterpret_cast<T*>(group_smem);
+
+            const T* __restrict__ A = static_cast<const T*>(a.A);
+            T* __restrict__ B       = static_cast<T*>(a.B);
+            const uint32_t tid      = threadIdx.x;
+
+            uint32_t       blk = blockIdx.x;
+            const uint32_t ti  = blk % a.nt_i;
+            blk /= a.nt_i;
+            const uint32_t tj = blk % a.nt_j;
+            blk /= a.nt_j;
+            uint32_t aoff = 0, boff = 0;
+            for(int d = 0; d < a.nb; ++d)
+            {
+                const uint32_t c = blk % a.bext[d];
+                blk /= a.bext[d];
+                aoff += c * a.ba[d];
+                boff += c * a.bb[d];
+            }
+            const uint32_t i1s = ti * a.c_i, j1s = tj * a.c_j;
+            const uint32_t ci = (a.e_i1 - i1s) < a.c_i ? (a.e_i1 - i1s) : a.c_i;
+            const uint32_t cj = (a.e_j1 - j1s) < a.c_j ? (a.e_j1 - j1s) : a.c_j;
+            const uint32_t nx = a.e_i0 * ci, ny = a.e_j0 * cj; // rows and columns inside the extents
+            const uint32_t RV = a.e_i0 * a.c_i / VR, CV = a.e_j0 * a.c_j / VW; // vectors per nominal row / column
+            aoff += i1s * a.e_i0 + j1s * a.a_j1;
+            boff += i1s * a.b_i1 + j1s * a.e_j0;
+            const T alpha = static_cast<T>(a.alpha);
+
+            const uint32_t total_r = RV * ny;
+            for(uint32_t u0 = 0; u0 < total_r; u0 += NT * U)
+            {
+                Vec<T, VR> r[U];
+                uint32_t   at[U];
+#pragma unroll
+                for(int k = 0; k < U; ++k)
+                {
+                    const uint32_t v  = u0 + tid + k * NT;
+                    const uint32_t y  = __umulhi(v, a.m_rv), xv = v - y * RV;
+                    const uint32_t y1 = __umulhi(y, a.m_ej0), y0 = y - y1 * a.e_j0;
+                    const bool     ok = v < total_r && xv * VR < nx;
+                    at[k]             = ok ? y * a.pitch + xv * VR : 0xFFFFFFFFu;
+                    // out-of-range lanes load the tile's first element: no branch, all loads in flight
+                    r[k] = *reinterpret_cast<const Vec<T, VR>*>(A + aoff + (ok ? xv * VR + y0 * a.a_j0 + y1 * a.a_j1 : 0u));
+                }
+#pragma unroll
+                for(int k = 0; k < U; ++k)
+                {
+                    if(at[k] != 0xFFFFFFFFu)
+                    {
+#pragma unroll
+                        for(int e = 0; e < VR; ++e)
+                            tile[at[k] + e] = element_op(r[k].v[e], alpha, a.op_a, a.op_b);
+                    }
+                }
+            }
+            __syncthreads();
+            const uint32_t total_w = CV * nx;
+            for(uint32_t v = tid; v < total_w; v += NT)
+            {
+                const uint32_t x = __umulhi(v, a.m_cv), yv = v - x * CV;
+                if(yv * VW < ny)
+                {
+                    const uint32_t x1 = __umulhi(x, a.m_ei0), x0 = x - x1 * a.e_i0;
+                    Vec<T, VW>     o;
+#pragma unroll
+                    for(int e = 0; e < VW; ++e)
+                        o.v[e] = tile[(yv * VW + e) * a.pitch + x];
+                    *reinterpret_cast<Vec<T, VW>*>(B + boff + yv * VW + x0 * a.b_i0 + x1 * a.b_i1) = o;
+                }
+            }
+        }
+
         template <typename T, int V>
         __global__ __launch_bounds__(PERM_THREADS) void permute_copy_kernel(
             const void* Av, void* Bv, uint32_t nvec, float alphaF, int op_a, int op_b)
@@ -515,6 +615,36 @@ namespace hiptk
             return launch_strip_len<T, VMAX, strip_len(sizeof(T), STRIP_MAX_SHORT)>(linear_write, vl, vs, a, grid, s);
         }
 
+        constexpr int GROUP_MAX_FAST = 128; // longest fastest mode the grouped kernel takes
+        constexpr int GROUP_MAX_LDS  = 60 * 1024;
+
+        uint32_t magic_of(uint32_t d)
+        {
+            return (uint32_t)((uint64_t(1) << 32) / d) + 1u;
+        }
+
+        template <typename T, int VMAX>
+        int launch_group(int vr, int vw, const QArgs& a, uint32_t grid, size_t lds, hipStream_t s)
+        {
+#define HIPTK_GROUP_CASE(R, W)                                                                                     \
+    if(vr == R && vw == W)                                                                                         \
+    {                                                                                                              \
+        hipLaunchKernelGGL((permute_group_kernel<T, R, W>), dim3(grid), dim3(PERM_THREADS), lds, s, a);              \
+        return (int)hipGetLastError();                                                                             \
+    }
+            HIPTK_GROUP_CASE(1, 1)
+            HIPTK_GROUP_CASE(1, 2)
+            HIPTK_GROUP_CASE(1, VMAX)
+            HIPTK_GROUP_CASE(2, 1)
+            HIPTK_GROUP_CASE(2, 2)
+            HIPTK_GROUP_CASE(2, VMAX)
+            HIPTK_GROUP_CASE(VMAX, 1)
+            HIPTK_GROUP_CASE(VMAX, 2)
+            HIPTK_GROUP_CASE(VMAX, VMAX)
+#undef HIPTK_GROUP_CASE
+            return -1;
+        }
+
         bool vec_allowed(int elem_bytes, int v)
         {
             return v == 1 || v == 2 || (elem_bytes == 4 ? v == 4 : v == 8);
@@ -612,6 +742,17 @@ extern "C" const char* hiptk_permute_kernel_name(const hiptk_permute_t* p)
         break;
     }
     case HIPTK_PERM_GATHER: snprintf(name, sizeof(name), "permute_gather_%s", type_tag(p->elem_bytes)); break;
+    case HIPTK_PERM_GROUPED:
+        if(vec_allowed(p->elem_bytes, p->vec_r) && vec_allowed(p->elem_bytes, p->vec_w) && p->chunk_i >= 1 && p->chunk_j >= 1)
+            snprintf(name,
+                     sizeof(name),
+                     "permute_grouped_%s_%dx%d_r%d_w%d",
+                     type_tag(p->elem_bytes),
+                     p->extent[0] * p->chunk_i,
+                     (p->mode_j >= 1 && p->mode_j < p->rank ? p->extent[p->mode_j] : 0) * p->chunk_j,
+                     p->vec_r,
+                     p->vec_w);
+        break;
     case HIPTK_PERM_STRIP:
         if((p->tile == 0 || p->tile == 1) && p->mode_j >= 1 && p->mode_j < p->rank && vec_allowed(p->elem_bytes, p->vec_r)
            && vec_allowed(p->elem_bytes, p->vec_w))
@@ -740,6 +881,81 @@ extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, v
             return HIPTK_ERR_ARG;
         rc = p->elem_bytes == 4 ? launch_tile_shape<float, 4>(p->tile, transpose, vr, vw, a, (uint32_t)grid, s)
                                 : launch_tile_shape<_Float16, 8>(p->tile, transpose, vr, vw, a, (uint32_t)grid, s);
+    }
+    else if(p->kernel == HIPTK_PERM_GROUPED)
+    {
+        const int mj = p->mode_j, mi2 = p->mode_i2, mj2 = p->mode_j2;
+        if(p->rank < 2 || p->mode_i != 0 || mj < 1 || mj >= p->rank || p->b_stride[mj] != 1)
+            return HIPTK_ERR_ARG;
+        if(!vec_allowed(p->elem_bytes, p->vec_r) || !vec_allowed(p->elem_bytes, p->vec_w))
+            return HIPTK_ERR_NO_KERNEL;
+        // the second modes, where present, directly follow the first ones in memory and are
+        // distinct from every other tile mode
+        if(mi2 != -1 && (mi2 < 1 || mi2 >= p->rank || mi2 == mj || mi2 == mj2 || p->a_stride[mi2] != p->extent[0]))
+            return HIPTK_ERR_ARG;
+        if(mj2 != -1 && (mj2 < 1 || mj2 >= p->rank || mj2 == mj || p->b_stride[mj2] != p->extent[mj]))
+            return HIPTK_ERR_ARG;
+        const int e_i1 = mi2 == -1 ? 1 : p->extent[mi2], e_j1 = mj2 == -1 ? 1 : p->extent[mj2];
+        if(p->extent[0] > GROUP_MAX_FAST || p->extent[mj] > GROUP_MAX_FAST || p->chunk_i < 1 || p->chunk_j < 1
+           || p->chunk_i > e_i1 || p->chunk_j > e_j1)
+            return HIPTK_ERR_ARG;
+        // vectors: whole vectors inside the fastest modes, every other stride and both bases aligned
+        const int vr = p->vec_r, vw = p->vec_w;
+        if(p->extent[0] % vr != 0 || p->extent[mj] % vw != 0 || !aligned(A, vr * p->elem_bytes) || !aligned(B, vw * p->elem_bytes))
+            return HIPTK_ERR_ARG;
+        for(int d = 1; d < p->rank; ++d)
+            if(p->a_stride[d] % vr != 0)
+                return HIPTK_ERR_ARG;
+        for(int d = 0; d < p->rank; ++d)
+            if(d != mj && p->b_stride[d] % vw != 0)
+                return HIPTK_ERR_ARG;
+
+        QArgs a;
+        memset(&a, 0, sizeof(a));
+        a.A    = A;
+        a.B    = B;
+        a.e_i0 = (uint32_t)p->extent[0];
+        a.e_i1 = (uint32_t)e_i1;
+        a.e_j0 = (uint32_t)p->extent[mj];
+        a.e_j1 = (uint32_t)e_j1;
+        a.c_i  = (uint32_t)p->chunk_i;
+        a.c_j  = (uint32_t)p->chunk_j;
+        a.a_j0 = (uint32_t)p->a_stride[mj];
+        a.a_j1 = mj2 == -1 ? 0u : (uint32_t)p->a_stride[mj2];
+        a.b_i0 = (uint32_t)p->b_stride[0];
+        a.b_i1 = mi2 == -1 ? 0u : (uint32_t)p->b_stride[mi2];
+        a.nt_i = (a.e_i1 + a.c_i - 1) / a.c_i;
+        a.nt_j = (a.e_j1 + a.c_j - 1) / a.c_j;
+        const uint32_t TI = a.e_i0 * a.c_i, TJ = a.e_j0 * a.c_j;
+        const uint32_t wordElems = 4u / (uint32_t)p->elem_bytes; // elements per 32-bit word
+        uint32_t       pitchWords = (TI + wordElems - 1) / wordElems;
+        pitchWords |= 1u; // odd: consecutive rows start in different banks
+        a.pitch          = pitchWords * wordElems;
+        const size_t lds = (size_t)TJ * a.pitch * p->elem_bytes;
+        if(lds > (size_t)GROUP_MAX_LDS || TI / vr == 0 || TJ / vw == 0)
+            return HIPTK_ERR_ARG;
+        a.m_rv  = magic_of(TI / vr);
+        a.m_ej0 = magic_of(a.e_j0);
+        a.m_cv  = magic_of(TJ / vw);
+        a.m_ei0 = magic_of(a.e_i0);
+        a.alpha = p->alpha;
+        a.op_a  = p->op_a;
+        a.op_b  = p->op_b;
+        int64_t grid = (int64_t)a.nt_i * a.nt_j;
+        for(int d = 1; d < p->rank; ++d)
+        {
+            if(d == mj || d == mi2 || d == mj2)
+                continue;
+            a.bext[a.nb] = (uint32_t)p->extent[d];
+            a.ba[a.nb]   = (uint32_t)p->a_stride[d];
+            a.bb[a.nb]   = (uint32_t)p->b_stride[d];
+            ++a.nb;
+            grid *= p->extent[d];
+        }
+        if(grid >= (int64_t(1) << 31))
+            return HIPTK_ERR_ARG;
+        rc = p->elem_bytes == 4 ? launch_group<float, 4>(vr, vw, a, (uint32_t)grid, lds, s)
+                                : launch_group<_Float16, 8>(vr, vw, a, (uint32_t)grid, lds, s);
     }
     else if(p->kernel == HIPTK_PERM_STRIP)
     {

@@ -150,11 +150,15 @@ enum
     HIPTK_PERM_ROWS   = 2, /* both tensors share the fastest mode (mode_i == 0): runs of that mode
                               are copied, tiles span it and one further mode (mode_j)             */
     HIPTK_PERM_GATHER = 3, /* one thread per element of B, any layout                             */
-    HIPTK_PERM_STRIP  = 4  /* TILED with one tile mode of at most 64 elements whose partner follows it
+    HIPTK_PERM_STRIP  = 4, /* TILED with one tile mode of at most 64 elements whose partner follows it
                               directly in memory on that side: a strip of the long mode times the
                               whole short mode is one contiguous run there.  tile == 0: mode_j is the
                               short one and the run lies in B; tile == 1: mode 0 is the short one and
                               the run lies in A                                                   */
+    HIPTK_PERM_GROUPED = 5 /* TILED for short fastest modes (both at most 128 elements): a tile row
+                              spans mode 0 and chunk_i indices of A's next mode (mode_i2, contiguous
+                              in A), a tile column mode_j and chunk_j indices of B's next mode
+                              (mode_j2, contiguous in B); a second mode may be absent (-1)        */
 };
 
 #define HIPTK_PERM_MAX_RANK 6
@@ -177,6 +181,8 @@ typedef struct hiptk_permute
     int32_t vec_w;      /* elements per global store                                              */
     int32_t group;      /* TILED / ROWS: workgroups walk the tile plane in bands of this many tiles
                            along mode_j, mode_j first inside a band (1: mode_i first throughout)  */
+    int32_t mode_i2, mode_j2; /* GROUPED: the second row / column mode, or -1                     */
+    int32_t chunk_i, chunk_j; /* GROUPED: indices of mode_i2 / mode_j2 per tile (1 when absent)   */
 } hiptk_permute_t;
 
 /* Name of the kernel a problem selects ("" if the combination is not instantiated). */

@@ -51,7 +51,8 @@ LARGE = [
     ([40, 50, 60], [0, 2, 1]),
     ([1024, 20, 4], [1, 0, 2]),           # long i, short j
     ([20, 1024, 4], [1, 0, 2]),           # short i, long j
-    ([6, 70, 80], [2, 1, 0]),             # short fastest mode: gather
+    ([6, 70, 80], [0, 2, 1]),             # short shared fastest mode: gather
+    ([6, 70, 80], [2, 1, 0]),
     ([8, 16, 8, 16, 8, 16], [5, 3, 1, 4, 2, 0]),
     ([32, 8, 16, 4, 8, 4], [1, 0, 3, 2, 5, 4]),
     ([512, 512], [1, 0]),
@@ -65,6 +66,11 @@ LARGE = [
     ([64, 300, 2], [1, 0, 2]),
     ([33, 290, 2], [1, 0, 2]),
     ([520, 64, 2], [1, 0, 2]),
+    ([16, 16, 16, 16, 16], [4, 3, 2, 1, 0]),   # many short modes: grouped tiles
+    ([24, 20, 12, 10, 6], [2, 4, 0, 3, 1]),
+    ([7, 9, 11, 13, 5], [3, 1, 4, 2, 0]),       # odd extents: scalar grouped tiles, ragged chunks
+    ([12, 5, 40, 30], [2, 3, 1, 0]),
+    ([6, 3, 2, 50, 40], [4, 3, 0, 1, 2]),
 ]
 
 

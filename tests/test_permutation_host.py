@@ -97,7 +97,7 @@ def test_fusion_and_kernel_choice(host_handle):
     i = _info(h, "f16", [128, 24, 96], [0, 2, 1])
     assert i["kernel"] == api.PERM_ROWS and i["vec_r"] == i["vec_w"] == 8 and i["mode_j"] == 2
     # short fastest mode, tiny tensors: one thread per element
-    assert _info(h, "f32", [6, 70, 80], [2, 1, 0])["kernel"] == api.PERM_GATHER
+    assert _info(h, "f32", [6, 70, 80], [0, 2, 1])["kernel"] == api.PERM_GATHER
     assert _info(h, "f32", [5, 2, 3, 4], [3, 2, 1, 0])["kernel"] == api.PERM_GATHER
     # a short tile mode whose partner follows it in memory: strips
     i = _info(h, "f32", [512, 512, 3, 16], [2, 0, 1, 3])
@@ -106,6 +106,10 @@ def test_fusion_and_kernel_choice(host_handle):
     assert i["kernel"] == api.PERM_STRIP and i["tile"] == 1 and (i["vec_r"], i["vec_w"]) == (8, 8)
     # ... but not when the partner is elsewhere in memory
     assert _info(h, "f32", [512, 3, 512, 16], [1, 3, 0, 2])["kernel"] == api.PERM_GATHER
+    # many short modes: rows span A's two fastest modes, columns B's two fastest
+    i = _info(h, "f32", [16] * 6, [5, 4, 3, 2, 1, 0])
+    assert i["kernel"] == api.PERM_GROUPED and i["kernel_name"] == "permute_grouped_f32_112x112_r4_w4"
+    assert _info(h, "f16", [16] * 6, [5, 4, 3, 2, 1, 0])["kernel_name"] == "permute_grouped_f16_128x128_r8_w8"
     # all extents one
     i = _info(h, "f16", [1, 1, 1], [2, 0, 1])
     assert (i["fused_rank"], i["kernel"], i["extent"]) == (1, api.PERM_COPY, [1])
