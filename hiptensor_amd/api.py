@@ -177,7 +177,7 @@ def hiptensorPermutation(handle, alpha, A, descA, modeA, B, descB, modeB, typeSc
 
 
 # kernel ids of the permutation path (HIPTK_PERM_* in include/hiptk_kernels.h)
-PERM_COPY, PERM_TILED, PERM_ROWS, PERM_GATHER, PERM_STRIP, PERM_GROUPED = 0, 1, 2, 3, 4, 5
+PERM_COPY, PERM_TILED, PERM_ROWS, PERM_GATHER, PERM_STRIP, PERM_GROUPED, PERM_SHARED = 0, 1, 2, 3, 4, 5, 6
 
 
 def permutationInfo(descA, modeA, descB, modeB, A=0, B=0):

@@ -38,7 +38,8 @@ namespace
 
     // HIPTENSOR_AMD_PERMUTE="kernel[,tile[,maxvec[,group]]]": kernel is auto | gather | tiled |
     // rows | strip | grouped (tiled and rows name the same preference: whichever of the two the
-    // layout admits; strip and grouped are taken wherever the layout admits them),
+    // layout admits; strip and grouped - which includes the shared-fastest-mode tiles - are
+    // taken wherever the layout admits them),
     // tile is 0..2 or -1, maxvec caps the vector width, group sets the band width of the
     // workgroup order.  For tests and experiments.
     hipta::PermuteTuning tuningFromEnv()

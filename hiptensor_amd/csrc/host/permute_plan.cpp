@@ -228,10 +228,48 @@ namespace hipta
             out.vec_w   = vw;
             return true;
         };
+        // A short shared fastest mode (interleaved channels): tiles of that mode times a chunk of
+        // A's next mode times a chunk of B's next mode, so that both sides see long runs.
+        auto tryShared = [&](bool force) -> bool {
+            if(!shared || r < 3 || ext[0] > 128)
+                return false;
+            if(ext[0] * in.elem_bytes >= 64 && !force)
+                return false; // from 64-byte runs on, plain rows do as well or better (measured)
+            const int mi2 = 1;
+            int       mj2 = -1;
+            for(int d = 1; d < r; ++d)
+                if(bs[d] == ext[0])
+                    mj2 = d;
+            if(mj2 == -1 || mj2 == mi2)
+                return false;
+            const int64_t target = 512 / in.elem_bytes; // elements per run aimed at
+            int64_t       ci = std::max<int64_t>(1, std::min<int64_t>(ext[mi2], target / ext[0]));
+            int64_t       cj = std::max<int64_t>(1, std::min<int64_t>(ext[mj2], target / ext[0]));
+            auto ldsBytes = [&]() { return cj * (ext[0] * ci + 2) * in.elem_bytes; };
+            while(ldsBytes() > 56 * 1024 && cj > 1)
+                cj -= 1;
+            if(ldsBytes() > 56 * 1024)
+                return false;
+            std::vector<int64_t> aOth(as.begin() + 1, as.end()), bOth(bs.begin() + 1, bs.end());
+            int v = std::min(pickVec(in.elem_bytes, cap, ext[0], aOth, in.A, false), pickVec(in.elem_bytes, cap, ext[0], bOth, in.B, false));
+            while(v > 1 && (ext[0] * ci / v < 2 || ext[0] * cj / v < 2))
+                v = v == 8 ? 2 : v / 2;
+            if(ext[0] * ci / v < 2 || ext[0] * cj / v < 2)
+                return false;
+            out.kernel  = HIPTK_PERM_SHARED;
+            out.mode_i  = 0;
+            out.mode_j  = 0;
+            out.mode_i2 = mi2;
+            out.mode_j2 = mj2;
+            out.chunk_i = (int32_t)ci;
+            out.chunk_j = (int32_t)cj;
+            out.vec_r = out.vec_w = v;
+            return true;
+        };
         out.mode_i2 = out.mode_j2 = -1;
         out.chunk_i = out.chunk_j = 1;
         int        kernel;
-        if(tune.kernel == HIPTK_PERM_GROUPED && tryGrouped(true))
+        if(tune.kernel == HIPTK_PERM_GROUPED && (tryGrouped(true) || tryShared(true)))
             return PermuteStatus::OK;
         if(tune.kernel == HIPTK_PERM_GATHER)
             kernel = HIPTK_PERM_GATHER;
@@ -243,6 +281,8 @@ namespace hipta
             kernel = HIPTK_PERM_GATHER; // a launch's worth of latency either way
         else if((stripJ && ext[0] >= 256) || (stripI && ext[jB] >= 256))
             kernel = HIPTK_PERM_STRIP;
+        else if(shared && tune.tile < 0 && tryShared(false))
+            return PermuteStatus::OK;
         else if(shared)
             kernel = ext[0] >= 16 ? HIPTK_PERM_ROWS : HIPTK_PERM_GATHER;
         else if(tune.tile < 0 && tryGrouped(false))

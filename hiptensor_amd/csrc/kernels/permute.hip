@@ -16,6 +16,8 @@
 //             contiguous run on the short mode's side, and moves it linearly there.
 //   * GROUPED TILED for tensors of many short modes: a tile row spans A's two fastest modes, a
 //             tile column B's two fastest modes, so that runs stay long when no single mode is.
+//   * SHARED  ROWS for a short shared fastest mode (interleaved channels): tiles of that mode
+//             times a chunk of A's next mode times a chunk of B's next mode, through LDS.
 //   * GATHER  one thread per element of B; covers tiny tensors and awkward extents.
 // Element operation per Composable Kernel's UnaryCombinedOp<Aop, Scale, Bop>
 // (ck/tensor_operation/gpu/element/combined_element_wise_operation.hpp:14-32): every step is
@@ -443,6 +445,101 @@ namespace hiptk
             }
         }
 
+        struct HArgs
+        {
+            const void* A;
+            void*       B;
+            uint32_t    e_c, e_i, e_j; // extents of mode 0, of A's next mode i and of B's next mode j
+            uint32_t    c_i, c_j; // indices of i / j per tile
+            uint32_t    a_j, b_i; // A stride of j, B stride of i (a_i == b_j == e_c)
+            uint32_t    nt_i, nt_j;
+            uint32_t    pitch; // LDS row pitch in elements: an odd number of 32-bit words
+            uint32_t    m_rv, m_cv, m_ec; // floor(2^32 / d) + 1 for d = e_c * c_i / VR, e_c * c_j / VW, e_c
+            int32_t     nb;
+            uint32_t    bext[PERM_BATCH], ba[PERM_BATCH], bb[PERM_BATCH];
+            float       alpha;
+            int32_t     op_a, op_b;
+        };
+
+        // A and B share the fastest mode c.  The tile (c, i-chunk, j-chunk) is read as c_j runs of
+        // e_c * c_i elements (c and i are contiguous in A), parked in LDS as [j][i * e_c + c], and
+        // written as c_i runs of e_c * c_j elements (c and j are contiguous in B).
+        template <typename T, int VR, int VW>
+        __global__ __launch_bounds__(PERM_THREADS) void permute_shared_kernel(HArgs a)
+        {
+            constexpr int NT = PERM_THREADS;
+            constexpr int U  = 8;
+            extern __shared__ unsigned char shared_smem[];
+            T* tile = reinterpret_cast<T*>(shared_smem);
+
+            const T* __restrict__ A = static_cast<const T*>(a.A);
+            T* __restrict__ B       = static_cast<T*>(a.B);
+            const uint32_t tid      = threadIdx.x;
+
+            uint32_t       blk = blockIdx.x;
+            const uint32_t ti  = blk % a.nt_i;
+            blk /= a.nt_i;
+            const uint32_t tj = blk % a.nt_j;
+            blk /= a.nt_j;
+            uint32_t aoff = 0, boff = 0;
+            for(int d = 0; d < a.nb; ++d)
+            {
+                const uint32_t c = blk % a.bext[d];
+                blk /= a.bext[d];
+                aoff += c * a.ba[d];
+                boff += c * a.bb[d];
+            }
+            const uint32_t is = ti * a.c_i, js = tj * a.c_j;
+            const uint32_t ci = (a.e_i - is) < a.c_i ? (a.e_i - is) : a.c_i;
+            const uint32_t cj = (a.e_j - js) < a.c_j ? (a.e_j - js) : a.c_j;
+            const uint32_t nx = a.e_c * ci, ny = a.e_c * cj; // run lengths inside the extents
+            const uint32_t RV = a.e_c * a.c_i / VR, CV = a.e_c * a.c_j / VW; // vectors per nominal run
+            aoff += is * a.e_c + js * a.a_j;
+            boff += is * a.b_i + js * a.e_c;
+            const T alpha = static_cast<T>(a.alpha);
+
+            const uint32_t total_r = RV * cj;
+            for(uint32_t u0 = 0; u0 < total_r; u0 += NT * U)
+            {
+                Vec<T, VR> r[U];
+                uint32_t   at[U];
+#pragma unroll
+                for(int k = 0; k < U; ++k)
+                {
+                    const uint32_t v  = u0 + tid + k * NT;
+                    const uint32_t y1 = __umulhi(v, a.m_rv), xv = v - y1 * RV;
+                    const bool     ok = v < total_r && xv * VR < nx;
+                    at[k]             = ok ? y1 * a.pitch + xv * VR : 0xFFFFFFFFu;
+                    r[k] = *reinterpret_cast<const Vec<T, VR>*>(A + aoff + (ok ? xv * VR + y1 * a.a_j : 0u));
+                }
+#pragma unroll
+                for(int k = 0; k < U; ++k)
+                {
+                    if(at[k] != 0xFFFFFFFFu)
+                    {
+#pragma unroll
+                        for(int e = 0; e < VR; ++e)
+                            tile[at[k] + e] = element_op(r[k].v[e], alpha, a.op_a, a.op_b);
+                    }
+                }
+            }
+            __syncthreads();
+            const uint32_t total_w = CV * ci;
+            for(uint32_t v = tid; v < total_w; v += NT)
+            {
+                const uint32_t x1 = __umulhi(v, a.m_cv), yv = v - x1 * CV;
+                if(yv * VW < ny)
+                {
+                    const uint32_t y1 = __umulhi(yv * VW, a.m_ec), c = yv * VW - y1 * a.e_c;
+                    Vec<T, VW>     o;
+#pragma unroll
+                    for(int e = 0; e < VW; ++e)
+                        o.v[e] = tile[y1 * a.pitch + x1 * a.e_c + c + e];
+                    *reinterpret_cast<Vec<T, VW>*>(B + boff + yv * VW + x1 * a.b_i) = o;
+                }
+            }
+        }
+
         template <typename T, int V>
         __global__ __launch_bounds__(PERM_THREADS) void permute_copy_kernel(
             const void* Av, void* Bv, uint32_t nvec, float alphaF, int op_a, int op_b)
@@ -645,6 +742,22 @@ namespace hiptk
             return -1;
         }
 
+        template <typename T, int VMAX>
+        int launch_shared(int v, const HArgs& a, uint32_t grid, size_t lds, hipStream_t s)
+        {
+#define HIPTK_SHARED_CASE(V)                                                                                  \
+    if(v == V)                                                                                                \
+    {                                                                                                         \
+        hipLaunchKernelGGL((permute_shared_kernel<T, V, V>), dim3(grid), dim3(PERM_THREADS), lds, s, a);        \
+        return (int)hipGetLastError();                                                                        \
+    }
+            HIPTK_SHARED_CASE(1)
+            HIPTK_SHARED_CASE(2)
+            HIPTK_SHARED_CASE(VMAX)
+#undef HIPTK_SHARED_CASE
+            return -1;
+        }
+
         bool vec_allowed(int elem_bytes, int v)
         {
             return v == 1 || v == 2 || (elem_bytes == 4 ? v == 4 : v == 8);
@@ -752,6 +865,17 @@ extern "C" const char* hiptk_permute_kernel_name(const hiptk_permute_t* p)
                      (p->mode_j >= 1 && p->mode_j < p->rank ? p->extent[p->mode_j] : 0) * p->chunk_j,
                      p->vec_r,
                      p->vec_w);
+        break;
+    case HIPTK_PERM_SHARED:
+        if(vec_allowed(p->elem_bytes, p->vec_r) && p->vec_r == p->vec_w && p->chunk_i >= 1 && p->chunk_j >= 1)
+            snprintf(name,
+                     sizeof(name),
+                     "permute_shared_%s_%dx%dx%d_v%d",
+                     type_tag(p->elem_bytes),
+                     p->extent[0],
+                     p->chunk_i,
+                     p->chunk_j,
+                     p->vec_r);
         break;
     case HIPTK_PERM_STRIP:
         if((p->tile == 0 || p->tile == 1) && p->mode_j >= 1 && p->mode_j < p->rank && vec_allowed(p->elem_bytes, p->vec_r)
@@ -956,6 +1080,65 @@ extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, v
             return HIPTK_ERR_ARG;
         rc = p->elem_bytes == 4 ? launch_group<float, 4>(vr, vw, a, (uint32_t)grid, lds, s)
                                 : launch_group<_Float16, 8>(vr, vw, a, (uint32_t)grid, lds, s);
+    }
+    else if(p->kernel == HIPTK_PERM_SHARED)
+    {
+        const int mi = p->mode_i2, mj = p->mode_j2, v = p->vec_r;
+        if(p->rank < 3 || p->mode_i != 0 || p->b_stride[0] != 1 || mi < 1 || mi >= p->rank || mj < 1 || mj >= p->rank || mi == mj)
+            return HIPTK_ERR_ARG;
+        if(p->a_stride[mi] != p->extent[0] || p->b_stride[mj] != p->extent[0])
+            return HIPTK_ERR_ARG;
+        if(!vec_allowed(p->elem_bytes, v) || p->vec_w != v)
+            return HIPTK_ERR_NO_KERNEL;
+        if(p->extent[0] > GROUP_MAX_FAST || p->chunk_i < 1 || p->chunk_j < 1 || p->chunk_i > p->extent[mi] || p->chunk_j > p->extent[mj])
+            return HIPTK_ERR_ARG;
+        if(p->extent[0] % v != 0 || !aligned(A, v * p->elem_bytes) || !aligned(B, v * p->elem_bytes))
+            return HIPTK_ERR_ARG;
+        for(int d = 1; d < p->rank; ++d)
+            if(p->a_stride[d] % v != 0 || p->b_stride[d] % v != 0)
+                return HIPTK_ERR_ARG;
+        HArgs a;
+        memset(&a, 0, sizeof(a));
+        a.A    = A;
+        a.B    = B;
+        a.e_c  = (uint32_t)p->extent[0];
+        a.e_i  = (uint32_t)p->extent[mi];
+        a.e_j  = (uint32_t)p->extent[mj];
+        a.c_i  = (uint32_t)p->chunk_i;
+        a.c_j  = (uint32_t)p->chunk_j;
+        a.a_j  = (uint32_t)p->a_stride[mj];
+        a.b_i  = (uint32_t)p->b_stride[mi];
+        a.nt_i = (a.e_i + a.c_i - 1) / a.c_i;
+        a.nt_j = (a.e_j + a.c_j - 1) / a.c_j;
+        const uint32_t TI = a.e_c * a.c_i, TJ = a.e_c * a.c_j;
+        const uint32_t wordElems  = 4u / (uint32_t)p->elem_bytes;
+        uint32_t       pitchWords = (TI + wordElems - 1) / wordElems;
+        pitchWords |= 1u;
+        a.pitch          = pitchWords * wordElems;
+        const size_t lds = (size_t)a.c_j * a.pitch * p->elem_bytes;
+        if(lds > (size_t)GROUP_MAX_LDS || TI / v < 2 || TJ / v < 2)
+            return HIPTK_ERR_ARG;
+        a.m_rv  = magic_of(TI / v);
+        a.m_cv  = magic_of(TJ / v);
+        a.m_ec  = magic_of(a.e_c);
+        a.alpha = p->alpha;
+        a.op_a  = p->op_a;
+        a.op_b  = p->op_b;
+        int64_t grid = (int64_t)a.nt_i * a.nt_j;
+        for(int d = 1; d < p->rank; ++d)
+        {
+            if(d == mi || d == mj)
+                continue;
+            a.bext[a.nb] = (uint32_t)p->extent[d];
+            a.ba[a.nb]   = (uint32_t)p->a_stride[d];
+            a.bb[a.nb]   = (uint32_t)p->b_stride[d];
+            ++a.nb;
+            grid *= p->extent[d];
+        }
+        if(grid >= (int64_t(1) << 31))
+            return HIPTK_ERR_ARG;
+        rc = p->elem_bytes == 4 ? launch_shared<float, 4>(v, a, (uint32_t)grid, lds, s)
+                                : launch_shared<_Float16, 8>(v, a, (uint32_t)grid, lds, s);
     }
     else if(p->kernel == HIPTK_PERM_STRIP)
     {

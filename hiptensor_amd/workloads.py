@@ -375,6 +375,9 @@ def permutation_configs():
         "perm_f32_copy": permutation("f32", [512, 64, 128, 64], [0, 1, 2, 3], 1.5, name="perm_f32_512x64x128x64_0123"),
         "perm_f16_nchw_to_nhwc": permutation("f16", [224, 224, 64, 256], [2, 0, 1, 3], 1.0, name="perm_f16_224x224x64x256_2013"),
         "perm_f32_channels3": permutation("f32", [512, 512, 3, 256], [2, 0, 1, 3], 1.0, name="perm_f32_512x512x3x256_2013"),
+        "perm_f32_short_modes": permutation("f32", [32, 32, 32, 32, 32, 8], [4, 3, 2, 1, 0, 5], 1.0, name="perm_f32_32x32x32x32x32x8_432105"),
+        "perm_f16_short_modes": permutation("f16", [16, 16, 16, 16, 16, 256], [4, 3, 2, 1, 0, 5], 1.0, name="perm_f16_16x16x16x16x16x256_432105"),
+        "perm_f32_rgba_transpose": permutation("f32", [4, 2048, 2048, 16], [0, 2, 1, 3], 1.0, name="perm_f32_4x2048x2048x16_0213"),
         "perm_f32_sample": permutation("f32", [33, 32, 34, 35], [2, 3, 1, 0], 1.0, name="perm_f32_33x32x34x35_2310"),
     }
 

@@ -155,10 +155,15 @@ enum
                               whole short mode is one contiguous run there.  tile == 0: mode_j is the
                               short one and the run lies in B; tile == 1: mode 0 is the short one and
                               the run lies in A                                                   */
-    HIPTK_PERM_GROUPED = 5 /* TILED for short fastest modes (both at most 128 elements): a tile row
+    HIPTK_PERM_GROUPED = 5, /* TILED for short fastest modes (both at most 128 elements): a tile row
                               spans mode 0 and chunk_i indices of A's next mode (mode_i2, contiguous
                               in A), a tile column mode_j and chunk_j indices of B's next mode
                               (mode_j2, contiguous in B); a second mode may be absent (-1)        */
+    HIPTK_PERM_SHARED = 6  /* ROWS for a short shared fastest mode (at most 128 elements, e.g. the
+                              four channels of RGBA pixels): a tile is mode 0 times chunk_i indices of
+                              A's next mode (mode_i2) times chunk_j indices of B's next mode (mode_j2);
+                              it is read in runs of extent[0] * chunk_i and, through LDS, written in
+                              runs of extent[0] * chunk_j                                        */
 };
 
 #define HIPTK_PERM_MAX_RANK 6

@@ -51,7 +51,11 @@ LARGE = [
     ([40, 50, 60], [0, 2, 1]),
     ([1024, 20, 4], [1, 0, 2]),           # long i, short j
     ([20, 1024, 4], [1, 0, 2]),           # short i, long j
-    ([6, 70, 80], [0, 2, 1]),             # short shared fastest mode: gather
+    ([6, 70, 80], [0, 2, 1]),             # short shared fastest mode: shared tiles
+    ([4, 130, 70, 3], [0, 2, 1, 3]),
+    ([2, 300, 33], [0, 2, 1]),
+    ([3, 5, 7, 9, 11, 5], [0, 4, 2, 3, 1, 5]),  # nothing lines up: gather
+    ([40, 50, 60], [0, 2, 1]),            # long shared fastest mode: rows
     ([6, 70, 80], [2, 1, 0]),
     ([8, 16, 8, 16, 8, 16], [5, 3, 1, 4, 2, 0]),
     ([32, 8, 16, 4, 8, 4], [1, 0, 3, 2, 5, 4]),

@@ -84,7 +84,7 @@ def test_large_shapes_default_selection(gpu_handle, oracle_mod, dtype, scalar):
         for w in perm_cases.large(dtype, scalar, 1.7, ops):
             _check(gpu_handle, oracle_mod, w, names)
     kinds = {n.split("_")[1] for n in names}
-    assert kinds == {"copy", "tiled", "rows", "gather", "strip", "grouped"}, names
+    assert kinds == {"copy", "tiled", "rows", "gather", "strip", "grouped", "shared"}, names
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
@@ -115,14 +115,15 @@ def test_grouped_kernels_at_every_vector_width(gpu_handle, oracle_mod, dtype, ma
     with _Override(f"grouped,-1,{maxvec}"):
         for w in perm_cases.large(dtype, alpha=1.5, ops=perm_cases.OPS[3]):
             _check(gpu_handle, oracle_mod, w, names)
-    assert sum(n.startswith("permute_grouped") for n in names) >= 4, names
+    assert sum(n.startswith("permute_grouped") for n in names) >= 4 and sum(n.startswith("permute_shared") for n in names) >= 3, names
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 def test_pointers_off_their_alignment(gpu_handle, oracle_mod, dtype):
     for a_shift, b_shift in ((1, 0), (0, 1), (2, 2), (1, 3), (4, 2)):
         for lens, perm in (([256, 192], [1, 0]), ([128, 24, 96], [0, 2, 1]), ([64, 64, 64], [0, 1, 2]),
-                           ([3000, 4, 5], [1, 0, 2]), ([4, 3000, 5], [1, 0, 2]), ([16, 16, 16, 16, 16], [4, 3, 2, 1, 0])):
+                           ([3000, 4, 5], [1, 0, 2]), ([4, 3000, 5], [1, 0, 2]), ([16, 16, 16, 16, 16], [4, 3, 2, 1, 0]),
+                           ([4, 130, 70, 3], [0, 2, 1, 3])):
             _check(gpu_handle, oracle_mod, wl.permutation(dtype, lens, perm, 1.25), a_shift=a_shift, b_shift=b_shift)
 
 

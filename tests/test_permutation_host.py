@@ -94,10 +94,13 @@ def test_fusion_and_kernel_choice(host_handle):
     i = _info(h, "f32", [33, 32, 34, 35], [2, 3, 1, 0])
     assert i["kernel"] == api.PERM_TILED and i["extent"] == [33, 32, 34 * 35] and (i["vec_r"], i["vec_w"]) == (1, 2)
     # shared fastest mode
-    i = _info(h, "f16", [128, 24, 96], [0, 2, 1])
+    i = _info(h, "f16", [512, 24, 96], [0, 2, 1])
     assert i["kernel"] == api.PERM_ROWS and i["vec_r"] == i["vec_w"] == 8 and i["mode_j"] == 2
+    # ... a short one (interleaved channels): tiles of it times chunks of A's and B's next modes
+    i = _info(h, "f32", [4, 512, 512, 8], [0, 2, 1, 3])
+    assert i["kernel"] == api.PERM_SHARED and i["kernel_name"] == "permute_shared_f32_4x32x32_v4"
     # short fastest mode, tiny tensors: one thread per element
-    assert _info(h, "f32", [6, 70, 80], [0, 2, 1])["kernel"] == api.PERM_GATHER
+    assert _info(h, "f32", [3, 5, 7, 9, 11], [0, 4, 2, 3, 1])["kernel"] == api.PERM_GATHER
     assert _info(h, "f32", [5, 2, 3, 4], [3, 2, 1, 0])["kernel"] == api.PERM_GATHER
     # a short tile mode whose partner follows it in memory: strips
     i = _info(h, "f32", [512, 512, 3, 16], [2, 0, 1, 3])
