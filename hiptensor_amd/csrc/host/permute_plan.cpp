@@ -151,7 +151,7 @@ namespace hipta
             out.b_stride[d] = (int32_t)bs[d];
         }
         out.vec_r = out.vec_w = 1;
-        out.group             = tune.group >= 1 ? tune.group : 1;
+        out.group             = tune.group >= 0 ? tune.group : 1;
         const int cap         = std::max(1, tune.max_vec);
 
         if(r == 1)
