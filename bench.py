@@ -35,7 +35,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("cfg2_f16_scale_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue"): (2.0 * 98533.9 + 1.0 * 32768.0) * 1024,
     ("cfg2_f16_scale_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue_pipe2x2"): (2.0 * 98563.0 + 1.0 * 32768.0) * 1024,
     # profiles/permute_kernels_1GiB_tensors.md
-    ("perm_f32_512x64x128x64_2031", "permute_tiled_f32_128x128_r4_w4"): (2.0 * 524327.4 + 1.0 * 1048576.1) * 1024,
+    ("perm_f32_512x64x128x64_2031", "permute_tiled_f32_128x128_r4_w4"): (2.0 * 524329.9 + 1.0 * 1049097.7) * 1024,
 }
 
 
