@@ -35,6 +35,10 @@ namespace hiptk
     typedef float    f32x16_t __attribute__((ext_vector_type(16)));
     typedef short    short4_t __attribute__((ext_vector_type(4)));
     typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+// D is written once and not read again by this launch: its vector stores are non-temporal, which
+// leaves the L2 to the operand panels (4096^3 f16: scale 123.4 -> 121.5 us, bilinear 128.3 -> 127.2 us).
+// Reading C the same way costs 5 % (135.0 us) and is not done.
+#define HIPTK_STORE_D(ptr, val) __builtin_nontemporal_store((val), (ptr))
     typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
     typedef float    f32x4_t __attribute__((ext_vector_type(4)));
 
@@ -733,7 +737,7 @@ namespace hiptk
 #pragma unroll
                 for(int v = 0; v < NVEC; v++)
                     if(qok[v] && pw + i * 32 + prow[v] < a.P)
-                        *(u32x4_t*)(Dp + doff[i & 1][v]) = o[v];
+                        HIPTK_STORE_D((u32x4_t*)(Dp + doff[i & 1][v]), o[v]);
                 wave_lds_fence();
             }
 #ifdef HIPTK_CLOCK_PROBE
@@ -876,7 +880,7 @@ namespace hiptk
 #pragma unroll
                 for(int v = 0; v < NVEC; v++)
                     if(cur.ok[v])
-                        *(u32x4_t*)(Dp + cur.doff[v]) = o[v];
+                        HIPTK_STORE_D((u32x4_t*)(Dp + cur.doff[v]), o[v]);
                 wave_lds_fence();
             }
 #ifdef HIPTK_CLOCK_PROBE
