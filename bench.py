@@ -12,7 +12,9 @@ f16 scale contraction at M = N = K = 4096 (extents 64^6, packed column-major).  
 prints ONE JSON line: metric / value (TFLOP/s of the headline workload), a `roofline` object
 for its kernel (average launch duration measured with HIP events on the launch stream), a
 `cpu_baseline` object (the reference's own CPU contraction, or the oracle port, timed on a
-bounded slab of the same workload on this host) and, with --all, the other configurations.
+bounded slab of the same workload on this host), a short `permutation` object (GB/s of one
+hiptensorPermutation workload; --permutation gives that operation its own full line) and, with
+--all, the other configurations.
 """
 import argparse
 import json
@@ -379,6 +381,12 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         out["copy_calibration"] = {"bytes_read": 1 << 28, "bytes_written": 1 << 28, "launches": 3}
+    # the permutation beside the contraction (its own line: --permutation): one workload, briefly
+    pw = wl.permutation_configs()["perm_f32_rank4"]
+    pr = measure_permutation(handle, pw, 50, 10, 0.1)
+    pgbs = wl.permutation_bytes(pw) / (pr["kernel_ms"] * 1e-3) / 1e9
+    out["permutation"] = {"workload": pw["name"], "kernel": pr["info"]["kernel_name"], "kernel_ms": pr["kernel_ms"],
+                          "GBs": pgbs, "frac_hbm_peak": pgbs / HBM_PEAK_GBS}
     if not a.no_cpu:
         out["cpu_baseline"] = cpu_baseline(w)
     api.hiptensorDestroy(handle)

@@ -114,7 +114,7 @@ typedef struct hiptensorAmdPermutationInfo
     int32_t fused_rank;   /* modes left after extent-1 modes are dropped and neighbours fused */
     int32_t extent[6];    /* fused extents in A's order, fastest first                        */
     int32_t a_stride[6], b_stride[6];
-    int32_t kernel;       /* HIPTK_PERM_COPY / TILED / ROWS / GATHER                          */
+    int32_t kernel;       /* HIPTK_PERM_COPY / TILED / ROWS / GATHER / STRIP / GROUPED / SHARED */
     int32_t mode_i, mode_j, tile, vec_r, vec_w;
     int32_t empty;        /* 1: an extent is zero, nothing would be launched                  */
     char    kernel_name[96];
