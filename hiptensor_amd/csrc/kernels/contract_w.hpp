@@ -580,7 +580,11 @@ namespace hiptk
                     if(qw + j * TILE < a.Q)
                     {
                         const E* cptr = bil ? Cp + (cpo + cqo[j]) : nullptr;
-                        Dp[dpo + dqo[j]] = Tr::finish(Tr::get(acc[i][j], r), a.alpha, a.beta, bil, cptr);
+                        const E val = Tr::finish(Tr::get(acc[i][j], r), a.alpha, a.beta, bil, cptr);
+                        if constexpr(std::is_arithmetic<E>::value)
+                            __builtin_nontemporal_store(val, Dp + (dpo + dqo[j]));
+                        else
+                            Dp[dpo + dqo[j]] = val;
                     }
                 }
             }
