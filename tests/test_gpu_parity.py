@@ -121,3 +121,25 @@ def test_invariants(gpu_handle, oracle_mod):
         ref = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
         got = gpu_util.run_gpu(gpu_handle, w, inp, d_alias_c=True)
         cases.assert_parity(w, got, ref, "D aliasing C")
+
+
+def test_non_finite_values_propagate_like_the_reference(gpu_handle, oracle_mod):
+    """The reference multiplies by alpha and beta unconditionally: beta = 0 does not hide a NaN or
+    an infinity held by C, alpha = 0 does not hide one produced by A x B.  The result must have
+    NaN exactly where the oracle has NaN, and agree elsewhere."""
+    for dtype in ("f32", "f16", "f64"):
+        for alpha, beta in ((1.0, 0.0), (0.0, 1.0), (1.5, 0.5)):
+            w = wl._rank4(dtype, cases.COMPUTE[dtype], (8, 5), (8, 7), (8, 6), alpha, beta, f"nonfinite_{dtype}")
+            inp = wl.host_inputs(w)
+            t = wl.NP_STORE[dtype]
+            inp["C"][3] = t(np.nan)
+            inp["C"][17] = t(np.inf)
+            inp["C"][40] = t(-np.inf)
+            inp["A"][5] = t(np.nan)
+            inp["B"][11] = t(np.inf)
+            got = wl.to_float(dtype, gpu_util.run_gpu(gpu_handle, w, inp))
+            ref = wl.to_float(dtype, oracle_mod.contract(w, inp["A"], inp["B"], inp["C"]))
+            assert np.array_equal(np.isnan(got), np.isnan(ref)), (dtype, alpha, beta)
+            assert np.array_equal(np.isinf(got), np.isinf(ref)) and np.array_equal(np.sign(got[np.isinf(got)]), np.sign(ref[np.isinf(ref)]))
+            fin = np.isfinite(ref)
+            assert fin.sum() > 0 and np.allclose(got[fin], ref[fin], rtol=cases.contract_tolerance(w), atol=cases.contract_tolerance(w))
