@@ -177,33 +177,25 @@ namespace hipta
         // fastest modes and a tile column B's two fastest modes, where those are free.
         // Fills `out` and returns true when that kernel applies (force: even where the plain
         // tiles would cover the extents well).
-        auto tryGrouped = [&](bool force) -> bool {
-            if(shared || ext[0] > 128 || ext[jB] > 128)
+        auto tryGrouped = [&](bool force, bool anySize) -> bool {
+            if(shared)
                 return false;
-            int mi2 = (r > 1 && jB != 1) ? 1 : -1;
+            const int64_t target = 128; // elements per tile row / column aimed at
+            // a side whose fastest mode is short takes a chunk of the next mode along; a long one
+            // is tiled by itself
+            int mi2 = (ext[0] <= target && r > 1 && jB != 1) ? 1 : -1;
             int mj2 = -1;
-            for(int d = 0; d < r; ++d)
-                if(bs[d] == ext[jB])
-                    mj2 = d;
-            if(mj2 == 0)
-                mj2 = -1;
+            if(ext[jB] <= target)
+                for(int d = 1; d < r; ++d)
+                    if(bs[d] == ext[jB])
+                        mj2 = d;
             if(mi2 != -1 && mi2 == mj2) // both sides want mode 1: the side with the shorter run gets it
                 (ext[jB] < ext[0] ? mi2 : mj2) = -1;
-            if(mi2 == -1 && mj2 == -1)
-                return false;
             const int    order[] = {0, 1, 2};
             const int    st      = pickTile(in.elem_bytes, ext[0], ext[jB], order);
             const Tile*  ts      = in.elem_bytes == 4 ? TILES4 : TILES2;
             const double cov     = coverage(ext[0], ts[st].ti) * coverage(ext[jB], ts[st].tj);
             if(cov >= 0.7 && !force)
-                return false;
-            const int64_t target = 128; // elements per tile row / column aimed at
-            int64_t       ci = mi2 == -1 ? 1 : std::max<int64_t>(1, std::min<int64_t>(ext[mi2], target / ext[0]));
-            int64_t       cj = mj2 == -1 ? 1 : std::max<int64_t>(1, std::min<int64_t>(ext[mj2], target / ext[jB]));
-            auto ldsBytes = [&]() { return (ext[jB] * cj) * (ext[0] * ci + 2) * in.elem_bytes; };
-            while(ldsBytes() > 56 * 1024 && (ci > 1 || cj > 1))
-                (ext[0] * ci >= ext[jB] * cj && ci > 1 ? ci : (cj > 1 ? cj : ci)) -= 1;
-            if(ldsBytes() > 56 * 1024)
                 return false;
             std::vector<int64_t> aOth(as.begin() + 1, as.end()), bOth;
             for(int d = 0; d < r; ++d)
@@ -211,12 +203,57 @@ namespace hipta
                     bOth.push_back(bs[d]);
             int vr = pickVec(in.elem_bytes, cap, ext[0], aOth, in.A, false);
             int vw = pickVec(in.elem_bytes, cap, ext[jB], bOth, in.B, false);
-            while(vr > 1 && ext[0] * ci / vr < 2)
+            int64_t wi = std::min<int64_t>(ext[0], target), wj = std::min<int64_t>(ext[jB], target);
+            int64_t ci = mi2 == -1 ? 1 : std::max<int64_t>(1, std::min<int64_t>(ext[mi2], target / ext[0]));
+            int64_t cj = mj2 == -1 ? 1 : std::max<int64_t>(1, std::min<int64_t>(ext[mj2], target / ext[jB]));
+            auto ldsBytes = [&]() { return (wj * cj) * (wi * ci + 2) * in.elem_bytes; };
+            while(ldsBytes() > 56 * 1024)
+            {
+                // shrink the longer side: first its chunk, then (a tiled side) its width
+                const bool iSide = wi * ci >= wj * cj;
+                int64_t&   c     = iSide ? ci : cj;
+                int64_t&   w     = iSide ? wi : wj;
+                const int  v     = iSide ? vr : vw;
+                if(c > 1)
+                    c -= 1;
+                else if(w > 2 * v && w > 16)
+                    w = (w / 2 + v - 1) / v * v;
+                else
+                    return false;
+            }
+            // a small problem needs more workgroups than long runs: halve the larger side of the
+            // tile until there are two workgroups per compute unit (256 of them) or the tile is small
+            auto groups = [&]() {
+                int64_t g = ((ext[0] + wi - 1) / wi) * ((ext[jB] + wj - 1) / wj);
+                for(int d = 1; d < r; ++d)
+                {
+                    if(d == jB)
+                        continue;
+                    g *= d == mi2 ? (ext[d] + ci - 1) / ci : d == mj2 ? (ext[d] + cj - 1) / cj : ext[d];
+                }
+                return g;
+            };
+            while(groups() < 512 && wi * ci * wj * cj >= 2 * 2048)
+            {
+                const bool iSide = wi * ci >= wj * cj;
+                int64_t&   c     = iSide ? ci : cj;
+                int64_t&   w     = iSide ? wi : wj;
+                const int  v     = iSide ? vr : vw;
+                if(c > 1)
+                    c = (c + 1) / 2;
+                else if(w > 2 * v && w > 16)
+                    w = (w / 2 + v - 1) / v * v;
+                else
+                    break;
+            }
+            while(vr > 1 && (wi * ci / vr < 2 || wi % vr != 0))
                 vr = vr == 8 ? 2 : vr / 2;
-            while(vw > 1 && ext[jB] * cj / vw < 2)
+            while(vw > 1 && (wj * cj / vw < 2 || wj % vw != 0))
                 vw = vw == 8 ? 2 : vw / 2;
-            if(ext[0] * ci / vr < 2 || ext[jB] * cj / vw < 2)
+            if(wi < 2 || wj < 2 || wi * ci / vr < 2 || wj * cj / vw < 2)
                 return false;
+            if(wi * ci * wj * cj < 2048 && !anySize)
+                return false; // tiles of a few hundred elements: one thread per element does better
             out.kernel  = HIPTK_PERM_GROUPED;
             out.mode_i  = 0;
             out.mode_j  = jB;
@@ -224,6 +261,8 @@ namespace hipta
             out.mode_j2 = mj2;
             out.chunk_i = (int32_t)ci;
             out.chunk_j = (int32_t)cj;
+            out.width_i = (int32_t)wi;
+            out.width_j = (int32_t)wj;
             out.vec_r   = vr;
             out.vec_w   = vw;
             return true;
@@ -269,7 +308,7 @@ namespace hipta
         out.mode_i2 = out.mode_j2 = -1;
         out.chunk_i = out.chunk_j = 1;
         int        kernel;
-        if(tune.kernel == HIPTK_PERM_GROUPED && (tryGrouped(true) || tryShared(true)))
+        if(tune.kernel == HIPTK_PERM_GROUPED && (tryGrouped(true, true) || tryShared(true)))
             return PermuteStatus::OK;
         if(tune.kernel == HIPTK_PERM_GATHER)
             kernel = HIPTK_PERM_GATHER;
@@ -279,13 +318,13 @@ namespace hipta
             kernel = shared ? HIPTK_PERM_ROWS : HIPTK_PERM_TILED;
         else if(count <= 16384)
             kernel = HIPTK_PERM_GATHER; // a launch's worth of latency either way
-        else if((stripJ && ext[0] >= 256) || (stripI && ext[jB] >= 256))
+        else if((stripJ && ext[0] >= 64) || (stripI && ext[jB] >= 64))
             kernel = HIPTK_PERM_STRIP;
         else if(shared && tune.tile < 0 && tryShared(false))
             return PermuteStatus::OK;
         else if(shared)
             kernel = ext[0] >= 16 ? HIPTK_PERM_ROWS : HIPTK_PERM_GATHER;
-        else if(tune.tile < 0 && tryGrouped(false))
+        else if(tune.tile < 0 && tryGrouped(ext[0] < 16 || ext[jB] < 16, false)) // (the plain tiles need 16 and more)
             return PermuteStatus::OK;
         else
             kernel = (ext[0] >= 16 && ext[jB] >= 16) ? HIPTK_PERM_TILED : HIPTK_PERM_GATHER;

@@ -405,21 +405,23 @@ namespace hiptk
             const void* A;
             void*       B;
             uint32_t    e_i0, e_i1, e_j0, e_j1; // extents of the row modes (0, i2) and the column modes (j, j2); 1 if absent
+            uint32_t    w_i, w_j; // elements of mode 0 / mode j per tile (== the extent when c > 1)
             uint32_t    c_i, c_j; // indices of i2 / j2 per tile
             uint32_t    a_j0, a_j1, b_i0, b_i1; // A strides of the column modes, B strides of the row modes
-            uint32_t    nt_i, nt_j; // tiles along i2 and j2
+            uint32_t    nt_i0, nt_j0, nt_i, nt_j; // tiles along mode 0, mode j, i2 and j2
             uint32_t    pitch; // LDS row pitch in elements: an odd number of 32-bit words
-            uint32_t    m_rv, m_ej0, m_cv, m_ei0; // floor(2^32 / d) + 1 for d = TI / VR, e_j0, TJ / VW, e_i0
+            uint32_t    m_rv, m_wj, m_cv, m_wi; // floor(2^32 / d) + 1 for d = TI / VR, w_j, TJ / VW, w_i
             int32_t     nb;
             uint32_t    bext[PERM_BATCH], ba[PERM_BATCH], bb[PERM_BATCH];
             float       alpha;
             int32_t     op_a, op_b;
         };
 
-        // Row x of a tile is (x0, x1) = (x mod e_i0, x div e_i0) over A's two fastest modes, which
-        // are contiguous in A; column y is (y0, y1) over B's two fastest modes, contiguous in B.
-        // Rows are read along x (one run of up to e_i0 * c_i elements of A per column), the tile is
-        // parked in LDS as [y][x], and columns are written along y.
+        // Row x of a tile is (x0, x1) = (x mod w_i, x div w_i): x0 walks w_i elements of mode 0 and,
+        // when the tile takes all of mode 0, x1 walks c_i indices of A's next mode - the two are
+        // contiguous in A, so a row is one run of A.  Column y is (y0, y1) over mode j and B's next
+        // mode in the same way, one run of B.  Rows are read along x, the tile is parked in LDS as
+        // [y][x], and columns are written along y.
         template <typename T, int VR, int VW>
         __global__ __launch_bounds__(PERM_THREADS) void permute_group_kernel(QArgs a)
         {
@@ -433,7 +435,11 @@ namespace hiptk
             const uint32_t tid      = threadIdx.x;
 
             uint32_t       blk = blockIdx.x;
-            const uint32_t ti  = blk % a.nt_i;
+            const uint32_t ti0 = blk % a.nt_i0;
+            blk /= a.nt_i0;
+            const uint32_t tj0 = blk % a.nt_j0;
+            blk /= a.nt_j0;
+            const uint32_t ti = blk % a.nt_i;
             blk /= a.nt_i;
             const uint32_t tj = blk % a.nt_j;
             blk /= a.nt_j;
@@ -445,13 +451,17 @@ namespace hiptk
                 aoff += c * a.ba[d];
                 boff += c * a.bb[d];
             }
+            const uint32_t i0s = ti0 * a.w_i, j0s = tj0 * a.w_j;
+            const uint32_t wi = (a.e_i0 - i0s) < a.w_i ? (a.e_i0 - i0s) : a.w_i;
+            const uint32_t wj = (a.e_j0 - j0s) < a.w_j ? (a.e_j0 - j0s) : a.w_j;
             const uint32_t i1s = ti * a.c_i, j1s = tj * a.c_j;
             const uint32_t ci = (a.e_i1 - i1s) < a.c_i ? (a.e_i1 - i1s) : a.c_i;
             const uint32_t cj = (a.e_j1 - j1s) < a.c_j ? (a.e_j1 - j1s) : a.c_j;
-            const uint32_t nx = a.e_i0 * ci, ny = a.e_j0 * cj; // rows and columns inside the extents
-            const uint32_t RV = a.e_i0 * a.c_i / VR, CV = a.e_j0 * a.c_j / VW; // vectors per nominal row / column
-            aoff += i1s * a.e_i0 + j1s * a.a_j1;
-            boff += i1s * a.b_i1 + j1s * a.e_j0;
+            // rows and columns inside the extents (c > 1 only with the whole first mode: w == e)
+            const uint32_t nx = a.w_i * (ci - 1) + wi, ny = a.w_j * (cj - 1) + wj;
+            const uint32_t RV = a.w_i * a.c_i / VR, CV = a.w_j * a.c_j / VW; // vectors per nominal row / column
+            aoff += i0s + i1s * a.e_i0 + j0s * a.a_j0 + j1s * a.a_j1;
+            boff += i0s * a.b_i0 + i1s * a.b_i1 + j0s + j1s * a.e_j0;
             const T alpha = static_cast<T>(a.alpha);
 
             const uint32_t total_r = RV * ny;
@@ -464,7 +474,7 @@ namespace hiptk
                 {
                     const uint32_t v  = u0 + tid + k * NT;
                     const uint32_t y  = __umulhi(v, a.m_rv), xv = v - y * RV;
-                    const uint32_t y1 = __umulhi(y, a.m_ej0), y0 = y - y1 * a.e_j0;
+                    const uint32_t y1 = __umulhi(y, a.m_wj), y0 = y - y1 * a.w_j;
                     const bool     ok = v < total_r && xv * VR < nx;
                     at[k]             = ok ? y * a.pitch + xv * VR : 0xFFFFFFFFu;
                     // out-of-range lanes load the tile's first element: no branch, all loads in flight
@@ -488,7 +498,7 @@ namespace hiptk
                 const uint32_t x = __umulhi(v, a.m_cv), yv = v - x * CV;
                 if(yv * VW < ny)
                 {
-                    const uint32_t x1 = __umulhi(x, a.m_ei0), x0 = x - x1 * a.e_i0;
+                    const uint32_t x1 = __umulhi(x, a.m_wi), x0 = x - x1 * a.w_i;
                     Vec<T, VW>     o;
 #pragma unroll
                     for(int e = 0; e < VW; ++e)
@@ -914,8 +924,8 @@ extern "C" const char* hiptk_permute_kernel_name(const hiptk_permute_t* p)
                      sizeof(name),
                      "permute_grouped_%s_%dx%d_r%d_w%d",
                      type_tag(p->elem_bytes),
-                     p->extent[0] * p->chunk_i,
-                     (p->mode_j >= 1 && p->mode_j < p->rank ? p->extent[p->mode_j] : 0) * p->chunk_j,
+                     p->width_i * p->chunk_i,
+                     p->width_j * p->chunk_j,
                      p->vec_r,
                      p->vec_w);
         break;
@@ -1073,12 +1083,18 @@ extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, v
         if(mj2 != -1 && (mj2 < 1 || mj2 >= p->rank || mj2 == mj || p->b_stride[mj2] != p->extent[mj]))
             return HIPTK_ERR_ARG;
         const int e_i1 = mi2 == -1 ? 1 : p->extent[mi2], e_j1 = mj2 == -1 ? 1 : p->extent[mj2];
-        if(p->extent[0] > GROUP_MAX_FAST || p->extent[mj] > GROUP_MAX_FAST || p->chunk_i < 1 || p->chunk_j < 1
+        const int w_i = p->width_i, w_j = p->width_j;
+        if(w_i < 1 || w_i > p->extent[0] || w_j < 1 || w_j > p->extent[mj] || p->chunk_i < 1 || p->chunk_j < 1
            || p->chunk_i > e_i1 || p->chunk_j > e_j1)
             return HIPTK_ERR_ARG;
-        // vectors: whole vectors inside the fastest modes, every other stride and both bases aligned
+        // a tile takes several indices of a second mode only together with the whole first mode
+        if((p->chunk_i > 1 && w_i != p->extent[0]) || (p->chunk_j > 1 && w_j != p->extent[mj]))
+            return HIPTK_ERR_ARG;
+        // vectors: whole vectors inside the tile widths and the fastest modes, every other stride
+        // and both bases aligned
         const int vr = p->vec_r, vw = p->vec_w;
-        if(p->extent[0] % vr != 0 || p->extent[mj] % vw != 0 || !aligned(A, vr * p->elem_bytes) || !aligned(B, vw * p->elem_bytes))
+        if(p->extent[0] % vr != 0 || p->extent[mj] % vw != 0 || w_i % vr != 0 || w_j % vw != 0 || !aligned(A, vr * p->elem_bytes)
+           || !aligned(B, vw * p->elem_bytes))
             return HIPTK_ERR_ARG;
         for(int d = 1; d < p->rank; ++d)
             if(p->a_stride[d] % vr != 0)
@@ -1095,30 +1111,34 @@ extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, v
         a.e_i1 = (uint32_t)e_i1;
         a.e_j0 = (uint32_t)p->extent[mj];
         a.e_j1 = (uint32_t)e_j1;
+        a.w_i  = (uint32_t)w_i;
+        a.w_j  = (uint32_t)w_j;
         a.c_i  = (uint32_t)p->chunk_i;
         a.c_j  = (uint32_t)p->chunk_j;
         a.a_j0 = (uint32_t)p->a_stride[mj];
         a.a_j1 = mj2 == -1 ? 0u : (uint32_t)p->a_stride[mj2];
         a.b_i0 = (uint32_t)p->b_stride[0];
         a.b_i1 = mi2 == -1 ? 0u : (uint32_t)p->b_stride[mi2];
-        a.nt_i = (a.e_i1 + a.c_i - 1) / a.c_i;
-        a.nt_j = (a.e_j1 + a.c_j - 1) / a.c_j;
-        const uint32_t TI = a.e_i0 * a.c_i, TJ = a.e_j0 * a.c_j;
+        a.nt_i0 = (a.e_i0 + a.w_i - 1) / a.w_i;
+        a.nt_j0 = (a.e_j0 + a.w_j - 1) / a.w_j;
+        a.nt_i  = (a.e_i1 + a.c_i - 1) / a.c_i;
+        a.nt_j  = (a.e_j1 + a.c_j - 1) / a.c_j;
+        const uint32_t TI = a.w_i * a.c_i, TJ = a.w_j * a.c_j;
         const uint32_t wordElems = 4u / (uint32_t)p->elem_bytes; // elements per 32-bit word
         uint32_t       pitchWords = (TI + wordElems - 1) / wordElems;
         pitchWords |= 1u; // odd: consecutive rows start in different banks
         a.pitch          = pitchWords * wordElems;
         const size_t lds = (size_t)TJ * a.pitch * p->elem_bytes;
-        if(lds > (size_t)GROUP_MAX_LDS || TI / vr == 0 || TJ / vw == 0)
-            return HIPTK_ERR_ARG;
-        a.m_rv  = magic_of(TI / vr);
-        a.m_ej0 = magic_of(a.e_j0);
-        a.m_cv  = magic_of(TJ / vw);
-        a.m_ei0 = magic_of(a.e_i0);
+        if(lds > (size_t)GROUP_MAX_LDS || TI / vr < 2 || TJ / vw < 2 || w_i < 2 || w_j < 2)
+            return HIPTK_ERR_ARG; // (the reciprocals below are exact for divisors of 2 and more)
+        a.m_rv = magic_of(TI / vr);
+        a.m_wj = magic_of(a.w_j);
+        a.m_cv = magic_of(TJ / vw);
+        a.m_wi = magic_of(a.w_i);
         a.alpha = p->alpha;
         a.op_a  = p->op_a;
         a.op_b  = p->op_b;
-        int64_t grid = (int64_t)a.nt_i * a.nt_j;
+        int64_t grid = (int64_t)a.nt_i0 * a.nt_j0 * a.nt_i * a.nt_j;
         for(int d = 1; d < p->rank; ++d)
         {
             if(d == mj || d == mi2 || d == mj2)

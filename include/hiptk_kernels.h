@@ -155,10 +155,12 @@ enum
                               whole short mode is one contiguous run there.  tile == 0: mode_j is the
                               short one and the run lies in B; tile == 1: mode 0 is the short one and
                               the run lies in A                                                   */
-    HIPTK_PERM_GROUPED = 5, /* TILED for short fastest modes (both at most 128 elements): a tile row
-                              spans mode 0 and chunk_i indices of A's next mode (mode_i2, contiguous
-                              in A), a tile column mode_j and chunk_j indices of B's next mode
-                              (mode_j2, contiguous in B); a second mode may be absent (-1)        */
+    HIPTK_PERM_GROUPED = 5, /* TILED with run-time tile shapes, for short fastest modes: a tile row
+                              spans width_i elements of mode 0 and, when width_i == extent[0],
+                              chunk_i indices of A's next mode (mode_i2, contiguous in A); a tile
+                              column width_j elements of mode_j and, when width_j == extent[mode_j],
+                              chunk_j indices of B's next mode (mode_j2, contiguous in B); a second
+                              mode may be absent (-1, chunk 1)                                    */
     HIPTK_PERM_SHARED = 6  /* ROWS for a short shared fastest mode (at most 128 elements, e.g. the
                               four channels of RGBA pixels): a tile is mode 0 times chunk_i indices of
                               A's next mode (mode_i2) times chunk_j indices of B's next mode (mode_j2);
@@ -188,6 +190,7 @@ typedef struct hiptk_permute
                            along mode_j, mode_j first inside a band (1: mode_i first throughout)  */
     int32_t mode_i2, mode_j2; /* GROUPED: the second row / column mode, or -1                     */
     int32_t chunk_i, chunk_j; /* GROUPED: indices of mode_i2 / mode_j2 per tile (1 when absent)   */
+    int32_t width_i, width_j; /* GROUPED: elements of mode 0 / mode_j per tile                    */
 } hiptk_permute_t;
 
 /* Name of the kernel a problem selects ("" if the combination is not instantiated). */

@@ -54,7 +54,9 @@ LARGE = [
     ([6, 70, 80], [0, 2, 1]),             # short shared fastest mode: shared tiles
     ([4, 130, 70, 3], [0, 2, 1, 3]),
     ([2, 300, 33], [0, 2, 1]),
-    ([3, 5, 7, 9, 11, 5], [0, 4, 2, 3, 1, 5]),  # nothing lines up: gather
+    ([3, 5, 7, 9, 11, 5], [0, 4, 2, 3, 1, 5]),
+    ([5, 7, 9, 4], [3, 1, 0, 2]),         # small: one thread per element
+    ([6, 32, 300], [1, 0, 2]),            # 192-element blocks transposed in place: one thread per element
     ([40, 50, 60], [0, 2, 1]),            # long shared fastest mode: rows
     ([6, 70, 80], [2, 1, 0]),
     ([8, 16, 8, 16, 8, 16], [5, 3, 1, 4, 2, 0]),

@@ -203,3 +203,37 @@ def test_permutation_inside_a_hip_graph(gpu_handle, oracle_mod):
             got = B.cpu().numpy().view(np.float32)
             assert _same(got, oracle_mod.permute(w, newA)), f"{w['name']} replay {rep}"
         p.close()
+
+
+def _random_cases(seed, count):
+    """Seeded random permutation problems: ranks 2..6, extents drawn to land on every kernel
+    (runs of 1..4 short modes next to long ones, powers of two and odd sizes), any mode order."""
+    rng = np.random.default_rng(seed)
+    pools = ([2, 3, 4, 5, 6, 7, 8], [9, 12, 16, 17, 24, 31, 32, 33], [48, 64, 65, 96, 100, 128, 130], [255, 256, 300, 513, 1000])
+    out = []
+    while len(out) < count:
+        rank = int(rng.integers(2, 7))
+        lens = [int(rng.choice(pools[int(rng.choice(4, p=[0.35, 0.3, 0.25, 0.1]))])) for _ in range(rank)]
+        n = int(np.prod(lens))
+        if not 2000 <= n <= 3_000_000:
+            continue
+        perm = [int(x) for x in rng.permutation(rank)]
+        dtype, scalar = perm_cases.TYPE_ROWS[int(rng.integers(0, 3))]
+        ops = perm_cases.OPS[int(rng.integers(0, 4))]
+        out.append((wl.permutation(dtype, lens, perm, float(rng.choice([1.0, -0.75, 2.3])), scalar, ops[0], ops[1]),
+                    int(rng.choice([0, 0, 1, 2, 4])), int(rng.choice([0, 0, 1, 2, 4]))))
+    return out
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_problems(gpu_handle, oracle_mod, seed):
+    names = {}
+    for w, a_shift, b_shift in _random_cases(seed, 150):
+        A = wl.permutation_input(w)
+        got, info = gpu_util.run_gpu_permutation(gpu_handle, w, A, a_shift=a_shift, b_shift=b_shift, return_info=True)
+        want = oracle_mod.permute(w, A)
+        assert _same(got, want), (w["dtype"], w["lensA"], w["perm"], a_shift, b_shift, info["kernel_name"])
+        kind = info["kernel_name"].split("_")[1]
+        names[kind] = names.get(kind, 0) + 1
+    print(f"[case] seed {seed}: kernels used {names}", flush=True)
+    assert len(names) >= 5, names

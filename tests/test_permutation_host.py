@@ -92,7 +92,8 @@ def test_fusion_and_kernel_choice(host_handle):
     assert i["kernel"] == api.PERM_TILED and (i["mode_i"], i["mode_j"]) == (0, 1) and (i["vec_r"], i["vec_w"]) == (4, 4)
     # the sample program's shape: 33 is odd, so loads are scalar; stores run along 34 * 35
     i = _info(h, "f32", [33, 32, 34, 35], [2, 3, 1, 0])
-    assert i["kernel"] == api.PERM_TILED and i["extent"] == [33, 32, 34 * 35] and (i["vec_r"], i["vec_w"]) == (1, 2)
+    assert i["kernel"] == api.PERM_GROUPED and i["extent"] == [33, 32, 34 * 35] and (i["vec_r"], i["vec_w"]) == (1, 2)
+    assert i["kernel_name"] == "permute_grouped_f32_33x64_r1_w2"  # a small tensor: tiles shrunk until 512 workgroups
     # shared fastest mode
     i = _info(h, "f16", [512, 24, 96], [0, 2, 1])
     assert i["kernel"] == api.PERM_ROWS and i["vec_r"] == i["vec_w"] == 8 and i["mode_j"] == 2
@@ -107,8 +108,9 @@ def test_fusion_and_kernel_choice(host_handle):
     assert i["kernel"] == api.PERM_STRIP and i["tile"] == 0 and i["extent"][:2] == [512 * 512, 3] and (i["vec_r"], i["vec_w"]) == (4, 4)
     i = _info(h, "f16", [3, 512, 512, 16], [1, 2, 0, 3])
     assert i["kernel"] == api.PERM_STRIP and i["tile"] == 1 and (i["vec_r"], i["vec_w"]) == (8, 8)
-    # ... but not when the partner is elsewhere in memory
-    assert _info(h, "f32", [512, 3, 512, 16], [1, 3, 0, 2])["kernel"] == api.PERM_GATHER
+    # ... when the partner is elsewhere in memory, grouped tiles take B's next mode along instead
+    i = _info(h, "f32", [512, 3, 512, 16], [1, 3, 0, 2])
+    assert i["kernel"] == api.PERM_GROUPED and i["kernel_name"] == "permute_grouped_f32_128x48_r4_w1"
     # many short modes: rows span A's two fastest modes, columns B's two fastest
     i = _info(h, "f32", [16] * 6, [5, 4, 3, 2, 1, 0])
     assert i["kernel"] == api.PERM_GROUPED and i["kernel_name"] == "permute_grouped_f32_112x112_r4_w4"
