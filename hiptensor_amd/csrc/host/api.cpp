@@ -764,6 +764,8 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         p.dq_stride = (int32_t)v.dq_stride;
         p.cp_stride = (int32_t)v.cp_stride;
         p.cq_stride = (int32_t)v.cq_stride;
+        p.shift_p   = v.shift_p;
+        p.shift_q   = v.shift_q;
         p.xk_stride            = (int32_t)v.xk_stride;
         p.yk_stride            = (int32_t)v.yk_stride;
         fresh->kernel_name     = hiptk_kernel_name(&p);

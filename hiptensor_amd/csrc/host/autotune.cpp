@@ -88,6 +88,8 @@ namespace hipta
         p.dq_stride = (int32_t)v.dq_stride;
         p.cp_stride = (int32_t)v.cp_stride;
         p.cq_stride = (int32_t)v.cq_stride;
+        p.shift_p   = v.shift_p;
+        p.shift_q   = v.shift_q;
         p.xk_stride = (int32_t)v.xk_stride;
         p.yk_stride = (int32_t)v.yk_stride;
         p.xp      = base + offs[0];

@@ -115,22 +115,30 @@ namespace hipta
             return true;
         }
 
-        // Widest power-of-two vector (<= maxv elements) that stays inside the leading
-        // dim's contiguous run and keeps every vector start aligned.
-        int vector_width(int64_t lead_len, const std::vector<int64_t>& other_strides, uint32_t align_bytes, int elem_bytes, int maxv)
+        // Extent from which a sole row / column dim may carry vectors although it is not a multiple
+        // of them: every tile (at most 256 rows or columns) then fits and can be moved back.
+        constexpr int64_t RAGGED_MIN = 256;
+
+        // Widest power-of-two vector (<= maxv elements) along a contiguous leading dim.  Vectors
+        // must not straddle the end of that dim's run: its length is a multiple of the vector, or
+        // (`sole`: it is its group's only dim, at least RAGGED_MIN long) the kernels move the last
+        // tile back so that every vector of it lies inside; *ragged says that this is relied on.
+        // Neither the base address nor the other strides need to be multiples of the vector:
+        // global memory takes vector loads and stores at any element-aligned address on this
+        // target (the compiler itself emits them for under-aligned types).
+        int vector_width(int64_t lead_len, bool sole, int maxv, bool* ragged)
         {
+            if(ragged)
+                *ragged = false;
             for(int v = maxv; v > 1; v /= 2)
             {
-                if(lead_len % v != 0)
-                    continue;
-                if((uint32_t)(v * elem_bytes) > align_bytes)
-                    continue;
-                bool ok = true;
-                for(int64_t s : other_strides)
-                    if(s % v != 0)
-                        ok = false;
-                if(ok)
+                if(lead_len % v == 0)
                     return v;
+                if(ragged && sole && lead_len >= RAGGED_MIN)
+                {
+                    *ragged = true;
+                    return v;
+                }
             }
             return 1;
         }
@@ -363,22 +371,13 @@ namespace hipta
 
         // ---- gather direction and vector width per operand ----
         const int maxv = class_max_vec(v.cls);
-        const TensorIn& Xt = v.swapped ? B : A;
-        const TensorIn& Yt = v.swapped ? A : B;
-        auto strides_except = [](const std::vector<Dim>& a, const std::vector<Dim>& b, bool use_x, const Dim* skip) {
-            std::vector<int64_t> s;
-            for(const std::vector<Dim>* g : {&a, &b})
-                for(const Dim& d : *g)
-                    if(&d != skip)
-                        s.push_back(use_x ? d.sx : d.sy);
-            return s;
-        };
-        auto pick = [&](bool use_x, const std::vector<Dim>& rows, uint32_t align, int& kfast, int& vec) {
-            int vk = 1, vr = 1;
+        auto pick = [&](bool use_x, const std::vector<Dim>& rows, int& kfast, int& vec, bool& ragged) {
+            int  vk = 1, vr = 1;
+            bool rr = false;
             if(!v.kdims.empty() && (use_x ? v.kdims[0].sx : v.kdims[0].sy) == 1)
-                vk = vector_width(v.kdims[0].len, strides_except(rows, v.kdims, use_x, &v.kdims[0]), align, v.elem_bytes, maxv);
+                vk = vector_width(v.kdims[0].len, false, maxv, nullptr);
             if(!rows.empty() && (use_x ? rows[0].sx : rows[0].sy) == 1)
-                vr = vector_width(rows[0].len, strides_except(rows, v.kdims, use_x, &rows[0]), align, v.elem_bytes, maxv);
+                vr = vector_width(rows[0].len, rows.size() == 1, maxv, &rr);
             // the wide classes are instantiated for full-width vectors and for scalars; the
             // 16-bit classes also for 8- and 4-byte vectors (narrowed jointly below)
             if(maxv != 8)
@@ -390,17 +389,20 @@ namespace hipta
             }
             if(vr > vk)
             {
-                kfast = 0;
-                vec   = vr;
+                kfast  = 0;
+                vec    = vr;
+                ragged = rr;
             }
             else
             {
-                kfast = 1;
-                vec   = vk;
+                kfast  = 1;
+                vec    = vk;
+                ragged = false;
             }
         };
-        pick(true, v.pdims, Xt.align, v.x_kfast, v.x_vec);
-        pick(false, v.qdims, Yt.align, v.y_kfast, v.y_vec);
+        bool xRagged = false, yRagged = false, cdRagged = false;
+        pick(true, v.pdims, v.x_kfast, v.x_vec, xRagged);
+        pick(false, v.qdims, v.y_kfast, v.y_vec, yRagged);
         if(maxv == 8 && !(v.x_vec == 8 && v.y_vec == 8))
         {
             // 16-bit kernels exist for (8,8), (4,4), (2,2), (1,8), (8,1) and (1,1) elements per
@@ -415,31 +417,21 @@ namespace hipta
                 {
                     v.x_vec   = 1;
                     v.x_kfast = 1;
+                    xRagged   = false;
                 }
                 if(v.y_vec < 8)
                 {
                     v.y_vec   = 1;
                     v.y_kfast = 1;
+                    yRagged   = false;
                 }
             }
         }
         v.cd_vec = 1;
         if(!v.qdims.empty() && v.qdims[0].sd == 1 && (!in.bilinear || v.qdims[0].sc == 1))
-        {
-            std::vector<int64_t> others;
-            for(const std::vector<Dim>* g : {&v.pdims, &v.qdims})
-                for(const Dim& d : *g)
-                    if(&d != &v.qdims[0])
-                    {
-                        others.push_back(d.sd);
-                        if(in.bilinear)
-                            others.push_back(d.sc);
-                    }
-            uint32_t al = D.align;
-            if(in.bilinear)
-                al = std::min(al, C.align);
-            v.cd_vec = vector_width(v.qdims[0].len, others, al, v.elem_bytes, maxv);
-        }
+            v.cd_vec = vector_width(v.qdims[0].len, v.qdims.size() == 1, maxv, &cdRagged);
+        v.shift_p = xRagged ? 1 : 0;
+        v.shift_q = (yRagged || cdRagged) ? 1 : 0;
 
         // ---- offset tables ----
         // Row / column tables cover every index a tile may overhang to: the largest tile edge is

@@ -61,6 +61,9 @@ namespace hipta
         // P and Q each fused into (at most) one dim in C and D: offsets are index * stride
         int     cd_affine = 0;
         int64_t dp_stride = 0, dq_stride = 0, cp_stride = 0, cq_stride = 0;
+        // vectors run along a row (column) index that is one contiguous run whose extent is not a
+        // multiple of the vector: tiles that would overhang are moved back to end at P (Q)
+        int shift_p = 0, shift_q = 0;
         int elem_bytes = 0;
         // bytes each tensor spans in memory (1 + sum (len-1)*stride elements)
         int64_t spanA = 0, spanB = 0, spanC = 0, spanD = 0;

@@ -75,6 +75,10 @@ namespace hipta
         p.x_vec   = v.x_vec;
         p.y_vec   = v.y_vec;
         p.k_affine = v.k_affine;
+        p.P        = v.P;
+        p.Q        = v.Q;
+        p.shift_p  = v.shift_p;
+        p.shift_q  = v.shift_q;
         return hiptk_kernel_available(&p) != 0;
     }
 

@@ -369,8 +369,16 @@ namespace hiptk
 
         int tp, tq;
         tile_coords(blockIdx.x, a.tiles_p, a.tiles_q, tp, tq);
-        const int p0 = tp * BP;
-        const int q0 = tq * BQ;
+        // rows / columns from p_own / q_own on are this tile's to store; with shift_p / shift_q the
+        // last tile is moved back to end exactly at P / Q (and recomputes some of its neighbour's)
+        const int p_own = tp * BP, q_own = tq * BQ;
+        const int p0    = (a.shift_p && p_own + BP > a.P) ? a.P - BP : p_own;
+        const int q0    = (a.shift_q && q_own + BQ > a.Q) ? a.Q - BQ : q_own;
+        auto      p_in  = [&](int p) { return p >= p_own && p < a.P; };
+        auto      q_in  = [&](int q) { return q >= q_own && q < a.Q; };
+        // a vector of 8 columns is stored when any of it is this tile's (the others are the
+        // neighbour's, recomputed here to the same values)
+        auto q_in8 = [&](int q) { return q + 8 > q_own && q < a.Q; };
 
         const int kt_begin = blockIdx.z * a.ktiles_per_split;
         int       kt_end   = kt_begin + a.ktiles_per_split;
@@ -630,7 +638,7 @@ namespace hiptk
             for(int j = 0; j < TQ; j++)
             {
                 const int q = qw + j * 32;
-                if(q >= a.Q)
+                if(!q_in(q))
                     continue;
 #pragma unroll
                 for(int i = 0; i < TP; i++)
@@ -638,7 +646,7 @@ namespace hiptk
                     for(int r = 0; r < 16; r++)
                     {
                         const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
-                        if(p < a.P)
+                        if(p_in(p))
                             ws[(size_t)p * a.Q + q] = acc[i][j][r];
                     }
             }
@@ -681,7 +689,7 @@ namespace hiptk
                 prow[v]     = 4 * (u / QB) + (L & 3);
                 qcol[v]     = 32 * (u % QB) + 8 * (L >> 2);
                 const int q = qw + qcol[v];
-                qok[v]      = q < a.Q;
+                qok[v]      = q_in8(q);
                 dqo[v]      = !qok[v] ? 0u : aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
             }
             uint32_t doff[2][NVEC];
@@ -690,7 +698,7 @@ namespace hiptk
                 for(int v = 0; v < NVEC; v++)
                 {
                     const int p = pw + i * 32 + prow[v];
-                    d[v] = !(qok[v] && p < a.P) ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
+                    d[v] = !(qok[v] && p_in(p)) ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
                 }
             };
             auto write_slab = [&](int i, uint16_t* dst) {
@@ -736,7 +744,7 @@ namespace hiptk
                     __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
 #pragma unroll
                 for(int v = 0; v < NVEC; v++)
-                    if(qok[v] && pw + i * 32 + prow[v] < a.P)
+                    if(qok[v] && p_in(pw + i * 32 + prow[v]))
                         HIPTK_STORE_D((u32x4_t*)(Dp + doff[i & 1][v]), o[v]);
                 wave_lds_fence();
             }
@@ -771,7 +779,7 @@ namespace hiptk
             for(int v = 0; v < NVEC; v++)
             {
                 const int q = qw + ((v * 64 + lane) % VPR) * 8;
-                qok[v]      = q < a.Q;
+                qok[v]      = q_in8(q);
                 // affine C / D (every benchmark-style packed layout): offsets are computed, so the
                 // epilogue starts without a round trip to the offset tables
                 dqo[v] = !qok[v] ? 0u : aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
@@ -789,7 +797,7 @@ namespace hiptk
                 for(int v = 0; v < NVEC; v++)
                 {
                     const int p = pw + i * 32 + (v * 64 + lane) / VPR;
-                    s.ok[v]     = qok[v] && p < a.P;
+                    s.ok[v]     = qok[v] && p_in(p);
                     s.doff[v]   = !s.ok[v] ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
                     u32x4_t c4  = {0u, 0u, 0u, 0u};
                     if(s.ok[v] && bil)
@@ -895,7 +903,7 @@ namespace hiptk
             for(int j = 0; j < TQ; j++)
             {
                 const int q = qw + j * 32;
-                if(q >= a.Q)
+                if(!q_in(q))
                     continue;
                 const uint32_t dqo = (uint32_t)a.dq[q];
                 const uint32_t cqo = a.bilinear ? (uint32_t)a.cq[q] : 0u;
@@ -905,7 +913,7 @@ namespace hiptk
                     for(int r = 0; r < 16; r++)
                     {
                         const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
-                        if(p < a.P)
+                        if(p_in(p))
                         {
                             const float c = a.bilinear ? Tr::out_to_f32(Cp[(uint32_t)a.cp[p] + cqo]) : 0.f;
                             Dp[(uint32_t)a.dp[p] + dqo]

@@ -391,8 +391,13 @@ namespace hiptk
 
         int tp, tq;
         tile_coords(blockIdx.x, a.tiles_p, a.tiles_q, tp, tq);
-        const int p0 = tp * BP;
-        const int q0 = tq * BQ;
+        // rows / columns from p_own / q_own on are this tile's to store; with shift_p / shift_q the
+        // last tile is moved back to end exactly at P / Q (and recomputes some of its neighbour's)
+        const int p_own = tp * BP, q_own = tq * BQ;
+        const int p0    = (a.shift_p && p_own + BP > a.P) ? a.P - BP : p_own;
+        const int q0    = (a.shift_q && q_own + BQ > a.Q) ? a.Q - BQ : q_own;
+        auto      p_in  = [&](int p) { return p >= p_own && p < a.P; };
+        auto      q_in  = [&](int q) { return q >= q_own && q < a.Q; };
 
         const int kt_begin = blockIdx.z * a.ktiles_per_split;
         int       kt_end   = kt_begin + a.ktiles_per_split;
@@ -538,14 +543,14 @@ namespace hiptk
                 for(int r = 0; r < Tr::NREG; r++)
                 {
                     const int p = pw + i * TILE + Tr::p_of(r, lane);
-                    if(p >= a.P)
+                    if(!p_in(p))
                         continue;
                     O* wrow = ws + (size_t)p * a.Q;
 #pragma unroll
                     for(int j = 0; j < TQ; j++)
                     {
                         const int q = qw + j * TILE;
-                        if(q < a.Q)
+                        if(q_in(q))
                             wrow[q] = Tr::get(acc[i][j], r);
                     }
                 }
@@ -570,14 +575,14 @@ namespace hiptk
             for(int r = 0; r < Tr::NREG; r++)
             {
                 const int p = pw + i * TILE + Tr::p_of(r, lane);
-                if(p >= a.P)
+                if(!p_in(p))
                     continue;
                 const uint32_t dpo = aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p];
                 const uint32_t cpo = !bil ? 0u : aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p];
 #pragma unroll
                 for(int j = 0; j < TQ; j++)
                 {
-                    if(qw + j * TILE < a.Q)
+                    if(q_in(qw + j * TILE))
                     {
                         const E* cptr = bil ? Cp + (cpo + cqo[j]) : nullptr;
                         const E val = Tr::finish(Tr::get(acc[i][j], r), a.alpha, a.beta, bil, cptr);

@@ -25,6 +25,10 @@ namespace hiptk
         int32_t cd_affine; // 1: C / D offsets are p * stride + q * stride, no table lookups
         int32_t dp_stride, dq_stride, cp_stride, cq_stride;
         int32_t cd_vec; // contiguous elements along q shared by C and D
+        // 1: a tile that would overhang P (Q) is moved back so that it ends at P (Q); it still
+        // stores only the rows (columns) of its own range.  Lets vectors run along a contiguous
+        // row (column) index whose extent is not a multiple of the vector.
+        int32_t shift_p, shift_q;
         double  alpha[2], beta[2];
     };
 

@@ -164,6 +164,9 @@ namespace hiptk
                 if(e.cls == p->cls && e.tile_id == p->tile_id && e.x_kfast == (p->x_kfast != 0)
                    && e.y_kfast == (p->y_kfast != 0) && e.x_vec == p->x_vec && e.y_vec == p->y_vec)
                 {
+                    // a tile can only be moved back to end at P / Q if it fits into P / Q
+                    if((p->shift_p && p->P < e.bp) || (p->shift_q && p->Q < e.bq))
+                        continue;
                     if(e.k_affine && p->k_affine)
                         return &e;
                     if(!e.k_affine && !table)
@@ -280,6 +283,13 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
     a.xk_stride = prob->xk_stride;
     a.yk_stride = prob->yk_stride;
     a.cd_vec    = prob->cd_vec;
+    a.shift_p   = prob->shift_p ? 1 : 0;
+    a.shift_q   = prob->shift_q ? 1 : 0;
+    // A moved-back tile stores whole 8-element vectors of D that reach into its neighbour's
+    // columns (same values).  When D is updated in place (C == D) the neighbour's elements must
+    // not be read and written twice, so that case stores element by element.
+    if(a.shift_q && bil && C == D && prob->Q % 8 != 0)
+        a.cd_vec = 1;
     a.tiles_p  = (int32_t)((prob->P + e->bp - 1) / e->bp);
     a.tiles_q  = (int32_t)((prob->Q + e->bq - 1) / e->bq);
     const int ktiles = (int)((prob->K + e->bk - 1) / e->bk);

@@ -89,6 +89,12 @@ typedef struct hiptk_problem
                           for a bilinear problem) for all p < P, q < Q: the epilogue then computes
                           offsets instead of reading the tables (which must still be valid)      */
     int32_t dp_stride, dq_stride, cp_stride, cq_stride;
+    int32_t shift_p; /* 1: the rows are one contiguous run of P elements in every tensor that is read
+                        or written in vectors along them, P need not be a multiple of the vector: a
+                        tile that would overhang P is moved back to end at P (it recomputes some of
+                        its neighbour's rows and stores only its own).  Needs P >= the tile's rows;
+                        tiles that do not fit are reported as unavailable                          */
+    int32_t shift_q; /* likewise for the columns                                                    */
 } hiptk_problem_t;
 
 /* Number of tile configurations of a class, and their description. */

@@ -182,54 +182,92 @@ def test_contraction_inside_a_hip_graph(gpu_handle, oracle_mod):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "f32", "f64"])
-def test_pointer_alignment_drives_the_vector_width(gpu_handle, oracle_mod, dtype):
-    """Operands at addresses that are only 8-, 4- or 2-byte aligned: the alignment reported by
-    hiptensorGetAlignmentRequirement goes into the descriptor, the planner narrows the gathers
-    to it (16-bit classes: 8 -> 4 -> 2 -> 1 elements; wide classes: full width or scalar),
-    and the result still matches the oracle."""
+def test_operands_at_any_element_aligned_address(gpu_handle, oracle_mod, dtype):
+    """Operands at addresses that are only 8-, 4- or 2-byte aligned, and with an odd row pitch:
+    the gathers and the stores of D keep their full vector width (global memory takes vector
+    accesses at any element-aligned address) and the result matches the oracle."""
     import torch
 
     a, b = 1.5, 0.75
-    w = wl._rank4(dtype, cases.COMPUTE[dtype], (16, 6), (8, 10), (8, 9), a, b, f"misaligned_{dtype}")
+    eb = wl.ELEM_BYTES[dtype]
+    full = {"f16": 8, "f32": 4, "f64": 2}[dtype]
+    ext = {0: 16, 1: 6, 10: 8, 11: 10, 20: 8, 21: 9}
+    packed = wl._rank4(dtype, cases.COMPUTE[dtype], (16, 6), (8, 10), (8, 9), a, b, f"misaligned_{dtype}")
+    # leading dimensions padded by one element: every row of A, B, C, D starts one element further off
+    odd_pitch = wl.make_workload(dtype, cases.COMPUTE[dtype], [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, a, b,
+                                 strideA=[1, 16, 97, 97 * 8], strideB=[1, 8, 81, 81 * 8],
+                                 strideC=[1, 16, 97, 97 * 8], strideD=[1, 16, 97, 97 * 8], name=f"odd_pitch_{dtype}")
+    for w in (packed, odd_pitch):
+        inp = wl.host_inputs(w)
+        exp = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
+        for shift in (0, 8, 4, 2):
+            if shift % eb:
+                continue
+            bufs = {}
+            for k in ("A", "B", "C"):
+                raw = torch.zeros(inp[k].nbytes + 64, dtype=torch.uint8, device="cuda")
+                base = (-raw.data_ptr()) % 16 + shift  # exactly `shift` beyond a 16-byte boundary
+                view = raw[base:base + inp[k].nbytes]
+                view.copy_(gpu_util.to_device(inp[k]))
+                bufs[k] = (raw, view)
+            nanD = wl.nan_buffer(dtype, inp["spanD"])
+            rawD = torch.zeros(nanD.nbytes + 64, dtype=torch.uint8, device="cuda")
+            baseD = (-rawD.data_ptr()) % 16 + shift
+            viewD = rawD[baseD:baseD + nanD.nbytes]
+            viewD.copy_(gpu_util.to_device(nanD))
+            probe = wl.Contraction(gpu_handle, w)
+            al = {}
+            for k, (d, ptr) in {"A": (probe.dA, bufs["A"][1].data_ptr()), "B": (probe.dB, bufs["B"][1].data_ptr()),
+                                "C": (probe.dC, bufs["C"][1].data_ptr()), "D": (probe.dD, viewD.data_ptr())}.items():
+                al[k] = api.check(api.hiptensorGetAlignmentRequirement(gpu_handle, ptr, d), "alignment")
+                assert al[k] == (16 if shift == 0 else shift), (k, shift, al[k])
+            probe.close()
+            c = wl.Contraction(gpu_handle, w, align=al)
+            assert (c.info["x_vec"], c.info["y_vec"], c.info["cd_vec"]) == (full, full, full), (shift, c.info)
+            ws = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+            print(f"[case] {w['name']} shift {shift} {c.info['kernel_name']}", flush=True)
+            st = c.run(bufs["A"][1].data_ptr(), bufs["B"][1].data_ptr(), bufs["C"][1].data_ptr(), viewD.data_ptr(),
+                       ws.data_ptr() if c.workspace_bytes else None, torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
+            assert st == 0
+            got = viewD.cpu().numpy().view(wl.NP_STORE[dtype])
+            cases.assert_parity(w, cases.logical_view(w, got), cases.logical_view(w, exp), f"shift {shift} {c.info['kernel_name']}")
+            c.close()
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32", "f64", "c32"])
+def test_ragged_extents_in_place(gpu_handle, oracle_mod, dtype):
+    """Odd extents of 256 and more on contiguous row and column indices: vectors are kept and the
+    last tiles are moved back.  D updated in place (D aliases C) must still see every element of
+    C exactly once, with and without split-K and on every tile of the class."""
+    import os
+
+    from hiptensor_amd._lib import lib
+
+    a, b = (1.1 + 1.2j, 0.5 - 0.25j) if dtype.startswith("c") else (1.5, 0.75)
+    ext = {0: 15, 1: 19, 10: 17, 11: 21, 20: 8, 21: 9}
+    w = wl.make_workload(dtype, cases.COMPUTE[dtype], [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, a, b,
+                         name=f"ragged_in_place_{dtype}")
     inp = wl.host_inputs(w)
     exp = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
-    eb = wl.ELEM_BYTES[dtype]
-    seen = set()
-    for shift in (0, 8, 4, 2):
-        if shift % eb:
-            continue
-        bufs = {}
-        for k in ("A", "B", "C"):
-            raw = torch.zeros(inp[k].nbytes + 64, dtype=torch.uint8, device="cuda")
-            base = (-raw.data_ptr()) % 16 + shift  # exactly `shift` beyond a 16-byte boundary
-            view = raw[base:base + inp[k].nbytes]
-            view.copy_(gpu_util.to_device(inp[k]))
-            bufs[k] = (raw, view)
-        nanD = wl.nan_buffer(dtype, inp["spanD"])
-        rawD = torch.zeros(nanD.nbytes + 64, dtype=torch.uint8, device="cuda")
-        baseD = (-rawD.data_ptr()) % 16 + shift
-        viewD = rawD[baseD:baseD + nanD.nbytes]
-        viewD.copy_(gpu_util.to_device(nanD))
-        probe = wl.Contraction(gpu_handle, w)
-        al = {}
-        for k, (d, ptr) in {"A": (probe.dA, bufs["A"][1].data_ptr()), "B": (probe.dB, bufs["B"][1].data_ptr()),
-                            "C": (probe.dC, bufs["C"][1].data_ptr()), "D": (probe.dD, viewD.data_ptr())}.items():
-            al[k] = api.check(api.hiptensorGetAlignmentRequirement(gpu_handle, ptr, d), "alignment")
-            assert al[k] == (16 if shift == 0 else shift), (k, shift, al[k])
-        probe.close()
-        c = wl.Contraction(gpu_handle, w, align=al)
-        full = {"f16": 8, "f32": 4, "f64": 2}[dtype]
-        want = max(1, min(full, (16 if shift == 0 else shift) // eb))
-        if dtype != "f16" and want < full:
-            want = 1
-        assert (c.info["x_vec"], c.info["y_vec"]) == (want, want), (shift, c.info)
-        seen.add(want)
-        ws = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
-        st = c.run(bufs["A"][1].data_ptr(), bufs["B"][1].data_ptr(), bufs["C"][1].data_ptr(), viewD.data_ptr(),
-                   ws.data_ptr() if c.workspace_bytes else None, torch.cuda.current_stream().cuda_stream)
-        torch.cuda.synchronize()
-        assert st == 0
-        got = viewD.cpu().numpy().view(wl.NP_STORE[dtype])
-        cases.assert_parity(w, got, exp, f"shift {shift} {c.info['kernel_name']}")
-        c.close()
-    assert len(seen) >= 2
+    probe = wl.Contraction(gpu_handle, w)
+    cls, full = probe.info["kernel_class"], probe.info["x_vec"]
+    assert full > 1 and probe.info["cd_vec"] == full, probe.info
+    probe.close()
+    ran = 0
+    try:
+        for tile in range(lib.hiptk_tile_count(cls)):
+            for split in (1, 2):
+                os.environ["HIPTENSOR_AMD_FORCE_KERNEL"] = f"{tile},{split}"
+                for alias in (True, False):
+                    try:
+                        got, info = gpu_util.run_gpu(gpu_handle, w, inp, pref=api.HIPTENSOR_WORKSPACE_MAX, d_alias_c=alias, return_info=True)
+                    except api.HiptensorError as e:
+                        assert e.status == api.HIPTENSOR_STATUS_EXECUTION_FAILED, e
+                        continue
+                    print(f"[case] {w['name']} tile={tile} split={split} alias={alias} {info['kernel_name']}", flush=True)
+                    cases.assert_parity(w, got, exp, f"{info['kernel_name']} split {split} alias {alias}")
+                    ran += 1
+    finally:
+        os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
+    assert ran >= 4

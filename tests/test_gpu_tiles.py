@@ -49,6 +49,13 @@ def layouts(dtype, compute, big):
                                         name=f"tiles_{tag}_kfast_{dtype}"))
             out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], ev, a, b,
                                         name=f"tiles_{tag}_mixed_{dtype}"))
+    # odd extents of 256 and more, each index one contiguous run: vectors stay, tiles that would
+    # overhang are moved back (2 row tiles of 256, 3 of 128, 5 of 64; columns likewise)
+    rg = {0: 15, 1: 19, 10: 17, 11: 21, 20: 16, 21: 9 if big else 5}
+    out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], rg, a, b,
+                                name=f"tiles_ragged_rowfast_{dtype}"))
+    out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], rg, a, None,
+                                name=f"tiles_ragged_mixed_{dtype}"))
     # odd extents: scalar gathers on every operand
     odd = {0: 7, 1: 23, 10: 5, 11: 29, 20: 3, 21: 37 if big else 21}
     out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], odd, a, b,

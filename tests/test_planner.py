@@ -95,13 +95,15 @@ def test_operand_pairing_is_consistent(host_handle):
     assert np.allclose(acc, ref[np.add.outer(dp, dq)], rtol=0, atol=1e-11)
 
 
-def test_vector_width_follows_runs_and_alignment(host_handle):
+def test_vector_width_follows_runs_not_alignment(host_handle):
     ext = {0: 16, 1: 6, 10: 8, 11: 10, 20: 16, 21: 5}
     w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
     info, _ = plan(host_handle, w)
     assert (info["x_vec"], info["y_vec"], info["cd_vec"]) == (8, 8, 8)
-    info, _ = plan(host_handle, w, align=2)  # pointers only element-aligned: scalar gathers
-    assert (info["x_vec"], info["y_vec"], info["cd_vec"]) == (1, 1, 1)
+    # pointers that are only element-aligned keep the vectors: global memory takes vector loads
+    # and stores at any element-aligned address
+    info, _ = plan(host_handle, w, align=2)
+    assert (info["x_vec"], info["y_vec"], info["cd_vec"]) == (8, 8, 8)
     ext[0], ext[1] = 12, 5  # the fused M run has 60 elements: not a multiple of 8
     w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
     info, _ = plan(host_handle, w)
@@ -124,6 +126,36 @@ def test_vector_width_follows_runs_and_alignment(host_handle):
     w = wl.make_workload("f32", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
     info, _ = plan(host_handle, w)
     assert (info["x_vec"], info["y_vec"]) == (4, 1)
+    # an odd row pitch (leading dimension padded by one element) does not narrow anything either
+    ext = {0: 16, 1: 6, 10: 8, 11: 10, 20: 16, 21: 5}
+    w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None,
+                         strideA=[1, 16, 97, 97 * 16], strideB=[1, 8, 81, 81 * 16])
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"], info["x_kfast"], info["y_kfast"]) == (8, 8, 0, 0)
+
+
+def test_ragged_contiguous_rows_and_columns_keep_their_vectors(host_handle):
+    """A row (column) index that is one contiguous run of at least 256 elements carries vectors
+    even when its extent is odd: the last tile is moved back to end at the extent.  Shorter or
+    multi-dim ragged indices fall to scalars as before."""
+    ext = {0: 15, 1: 19, 10: 17, 11: 21, 20: 16, 21: 4}  # M = 285, N = 357, packed: each fuses to one run
+    w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, 0.5)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"], info["cd_vec"], info["x_kfast"], info["y_kfast"]) == (8, 8, 8, 0, 0)
+    assert info["n_pdims"] == 1 and info["n_qdims"] == 1
+    w32 = wl.make_workload("f32", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
+    info, _ = plan(host_handle, w32)
+    assert (info["x_vec"], info["y_vec"], info["cd_vec"]) == (4, 4, 4)
+    ext = {0: 15, 1: 13, 10: 17, 11: 11, 20: 16, 21: 4}  # M = 195, N = 187: too short to move a 256-wide tile back
+    w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"], info["cd_vec"]) == (1, 1, 1)
+    # padded leading dimension: M stays two dims (15 | 19), vectors cannot straddle the gap
+    ext = {0: 15, 1: 19, 10: 17, 11: 21, 20: 16, 21: 4}
+    w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None,
+                         strideA=[1, 16, 16 * 19, 16 * 19 * 16])
+    info, _ = plan(host_handle, w)
+    assert info["n_pdims"] + info["n_qdims"] >= 3 and 1 in (info["x_vec"], info["y_vec"])
 
 
 def test_extent_one_modes_and_missing_groups(host_handle):
