@@ -126,7 +126,7 @@ namespace hipta
         // Neither the base address nor the other strides need to be multiples of the vector:
         // global memory takes vector loads and stores at any element-aligned address on this
         // target (the compiler itself emits them for under-aligned types).
-        int vector_width(int64_t lead_len, bool sole, int maxv, bool* ragged)
+        int vector_width(int64_t lead_len, bool sole, int maxv, bool* ragged, int64_t ragged_min = RAGGED_MIN)
         {
             if(ragged)
                 *ragged = false;
@@ -134,7 +134,7 @@ namespace hipta
             {
                 if(lead_len % v == 0)
                     return v;
-                if(ragged && sole && lead_len >= RAGGED_MIN)
+                if(ragged && sole && lead_len >= ragged_min)
                 {
                     *ragged = true;
                     return v;
@@ -374,8 +374,10 @@ namespace hipta
         auto pick = [&](bool use_x, const std::vector<Dim>& rows, int& kfast, int& vec, bool& ragged) {
             int  vk = 1, vr = 1;
             bool rr = false;
+            // (a ragged K needs no flag: the kernels' last K tile handles a straddling vector)
+            bool kr = false;
             if(!v.kdims.empty() && (use_x ? v.kdims[0].sx : v.kdims[0].sy) == 1)
-                vk = vector_width(v.kdims[0].len, false, maxv, nullptr);
+                vk = vector_width(v.kdims[0].len, v.kdims.size() == 1, maxv, &kr, 2 * maxv);
             if(!rows.empty() && (use_x ? rows[0].sx : rows[0].sy) == 1)
                 vr = vector_width(rows[0].len, rows.size() == 1, maxv, &rr);
             // the wide classes are instantiated for full-width vectors and for scalars; the

@@ -236,23 +236,86 @@ namespace hiptk
                 d[0] = (uint32_t)*p & mask;
         }
 
+        // d holds V staged 16-bit elements, element e in bits 16 * (e % 2) of word e / 2.  Moves
+        // element e + s to element e (s = 1 .. V - 1, the same for the whole wave) and clears the
+        // top s elements.
+        __device__ static inline void shift_down(uint32_t (&d)[W], int s)
+        {
+            if constexpr(V >= 2)
+            {
+                uint32_t t[2 * W];
+#pragma unroll
+                for(int i = 0; i < W; i++)
+                {
+                    t[i]     = d[i];
+                    t[W + i] = 0u;
+                }
+                const int ws = s >> 1;
+                // s is uniform: a switch over the word shift keeps every register index static
+                switch(ws)
+                {
+#define HIPTK_SHIFT_CASE(WS)                                                                        \
+    case WS:                                                                                        \
+        _Pragma("unroll") for(int i = 0; i < W; i++)                                                \
+        {                                                                                           \
+            const uint32_t lo = (i + WS < 2 * W) ? t[(i + WS) % (2 * W)] : 0u;                      \
+            const uint32_t hi = (i + WS + 1 < 2 * W) ? t[(i + WS + 1) % (2 * W)] : 0u;              \
+            d[i]              = (s & 1) ? __builtin_amdgcn_alignbit(hi, lo, 16) : lo;               \
+        }                                                                                           \
+        break;
+                    HIPTK_SHIFT_CASE(0)
+                    HIPTK_SHIFT_CASE(1)
+                    HIPTK_SHIFT_CASE(2)
+                    HIPTK_SHIFT_CASE(3)
+#undef HIPTK_SHIFT_CASE
+                default: break;
+                }
+            }
+        }
+
         // Fetch the tile whose first k is k0.  TAIL: the tile may reach beyond K.
+        //
+        // k-fast vectors and a K that is not a multiple of the vector (the planner allows that
+        // when k is one contiguous run): the vector that straddles K is loaded V elements back
+        // from the end of the run - inside the tensor - and moved down in registers, which also
+        // clears the slots from K on.
         template <bool TAIL>
         __device__ inline void fetch(const void* base, int k0, int K, int kstride)
         {
             const src_t* bp = (const src_t*)base;
             if constexpr(KF)
             {
-                const int      k    = k0 + a * V;
-                const uint32_t mask = (!TAIL || k < K) ? 0xFFFFFFFFu : 0u;
+                const int      k       = k0 + a * V;
+                const bool     partial = TAIL && V > 1 && k < K && k + V > K;
+                const int      over    = k + V - K; // elements of a straddling vector beyond K
+                const uint32_t mask    = (!TAIL || k < K) ? 0xFFFFFFFFu : 0u;
                 uint32_t       ko;
                 if constexpr(KAFF)
-                    ko = (uint32_t)((TAIL && k >= K) ? 0 : k) * (uint32_t)kstride;
+                    ko = (uint32_t)((TAIL && k >= K) ? 0 : (partial ? k - over : k)) * (uint32_t)kstride;
                 else
-                    ko = (uint32_t)koff[0];
+                    ko = (uint32_t)koff[0] - (partial ? (uint32_t)over : 0u); // (k is this operand's unit-stride index)
 #pragma unroll
                 for(int i = 0; i < N; i++)
                     fetch_one(bp + ((uint32_t)roff[i] + ko), mask, data[i]);
+                if constexpr(TAIL && V > 1)
+                {
+                    const int r = K % V; // uniform; 0 when no vector straddles K
+                    if(r != 0)
+                    {
+#pragma unroll
+                        for(int i = 0; i < N; i++)
+                        {
+                            uint32_t sh[W];
+#pragma unroll
+                            for(int w = 0; w < W; w++)
+                                sh[w] = data[i][w];
+                            shift_down(sh, V - r);
+#pragma unroll
+                            for(int w = 0; w < W; w++)
+                                data[i][w] = partial ? sh[w] : data[i][w];
+                        }
+                    }
+                }
             }
             else
             {

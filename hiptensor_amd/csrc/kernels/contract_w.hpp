@@ -319,14 +319,47 @@ namespace hiptk
             {
                 const int  k  = MODE == GATHER_MN_VEC ? k0 + b + i * STEP : k0 + a * V;
                 const bool ok = !TAIL || k < K;
+                // A k-fast vector that straddles K (K is then one contiguous run, not a multiple
+                // of the vector) is loaded V elements back from the end of the run, inside the
+                // tensor, and moved down in registers; that also clears the slots from K on.
+                const bool partial = MODE == GATHER_K_VEC && TAIL && V > 1 && k < K && k + V > K;
                 const uint32_t off = MODE == GATHER_MN_VEC ? (uint32_t)roff[0] + (uint32_t)koff[i]
-                                                            : (uint32_t)roff[i] + (uint32_t)koff[0];
+                                                            : (uint32_t)roff[i] + (uint32_t)koff[0] - (partial ? (uint32_t)(k + V - K) : 0u);
                 PackE v = *(const PackE*)(bp + off);
                 if(TAIL && !ok)
                 {
 #pragma unroll
                     for(int j = 0; j < V; j++)
                         v.e[j] = E{};
+                }
+                if constexpr(MODE == GATHER_K_VEC && TAIL && V > 1)
+                {
+                    const int r = K % V; // uniform; 0 when no vector straddles K
+                    if(r != 0)
+                    {
+                        PackE sh = v;
+                        switch(V - r) // uniform: every register index below is static
+                        {
+                        case 1:
+#pragma unroll
+                            for(int j = 0; j < V; j++)
+                                sh.e[j] = j + 1 < V ? v.e[(j + 1) % V] : E{};
+                            break;
+                        case 2:
+#pragma unroll
+                            for(int j = 0; j < V; j++)
+                                sh.e[j] = j + 2 < V ? v.e[(j + 2) % V] : E{};
+                            break;
+                        case 3:
+#pragma unroll
+                            for(int j = 0; j < V; j++)
+                                sh.e[j] = j + 3 < V ? v.e[(j + 3) % V] : E{};
+                            break;
+                        default: break;
+                        }
+                        if(partial)
+                            v = sh;
+                    }
                 }
                 data[i] = v;
             }

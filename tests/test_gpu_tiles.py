@@ -56,6 +56,14 @@ def layouts(dtype, compute, big):
                                 name=f"tiles_ragged_rowfast_{dtype}"))
     out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], rg, a, None,
                                 name=f"tiles_ragged_mixed_{dtype}"))
+    # a contiguous reduction index of odd extent under k-fast vectors: the vector that straddles
+    # K is loaded from inside the run and moved down in registers (K = 105 and K = 17)
+    for tag, k0, k1 in (("k105", 15, 7), ("k17", 17, 1)):
+        rk = {0: 40, 1: 5, 10: 24, 11: 7, 20: k0, 21: k1}
+        out.append(wl.make_workload(dtype, compute, [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], rk, a, b,
+                                    name=f"tiles_ragged_{tag}_kfast_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], rk, a, None,
+                                    name=f"tiles_ragged_{tag}_mixed_{dtype}"))
     # odd extents: scalar gathers on every operand
     odd = {0: 7, 1: 23, 10: 5, 11: 29, 20: 3, 21: 37 if big else 21}
     out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], odd, a, b,

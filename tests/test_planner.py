@@ -150,6 +150,14 @@ def test_ragged_contiguous_rows_and_columns_keep_their_vectors(host_handle):
     w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
     info, _ = plan(host_handle, w)
     assert (info["x_vec"], info["y_vec"], info["cd_vec"]) == (1, 1, 1)
+    # a contiguous K of odd extent keeps k-fast vectors (the straddling vector is handled in the last K tile)
+    ext = {0: 16, 1: 6, 10: 8, 11: 10, 20: 15, 21: 7}
+    w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"], info["x_kfast"], info["y_kfast"], info["n_kdims"]) == (8, 8, 1, 1, 1)
+    w = wl.make_workload("f64", api.HIPTENSOR_COMPUTE_64F, [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"], info["x_kfast"], info["y_kfast"]) == (2, 2, 1, 1)
     # padded leading dimension: M stays two dims (15 | 19), vectors cannot straddle the gap
     ext = {0: 15, 1: 19, 10: 17, 11: 21, 20: 16, 21: 4}
     w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None,
