@@ -116,8 +116,9 @@ namespace hipta
         }
 
         // Extent from which a sole row / column dim may carry vectors although it is not a multiple
-        // of them: every tile (at most 256 rows or columns) then fits and can be moved back.
-        constexpr int64_t RAGGED_MIN = 256;
+        // of them: the smallest tile of every class with vector kernels (64 x 64) then fits and can
+        // be moved back; larger tiles are offered only where they fit (hiptk_kernel_available).
+        constexpr int64_t RAGGED_MIN = 64;
 
         // Widest power-of-two vector (<= maxv elements) along a contiguous leading dim.  Vectors
         // must not straddle the end of that dim's run: its length is a multiple of the vector, or

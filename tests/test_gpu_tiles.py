@@ -56,6 +56,10 @@ def layouts(dtype, compute, big):
                                 name=f"tiles_ragged_rowfast_{dtype}"))
     out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], rg, a, None,
                                 name=f"tiles_ragged_mixed_{dtype}"))
+    # ... and with extents between the tile sizes: only the tiles that fit are offered
+    rs = {0: 15, 1: 7, 10: 13, 11: 15, 20: 16, 21: 3}
+    out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], rs, a, b,
+                                name=f"tiles_ragged_small_rowfast_{dtype}"))
     # a contiguous reduction index of odd extent under k-fast vectors: the vector that straddles
     # K is loaded from inside the run and moved down in registers (K = 105 and K = 17)
     for tag, k0, k1 in (("k105", 15, 7), ("k17", 17, 1)):
@@ -64,9 +68,10 @@ def layouts(dtype, compute, big):
                                     name=f"tiles_ragged_{tag}_kfast_{dtype}"))
         out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], rk, a, None,
                                     name=f"tiles_ragged_{tag}_mixed_{dtype}"))
-    # odd extents: scalar gathers on every operand
+    # odd extents with the modes interleaved, so that no index is one contiguous run: scalar
+    # gathers on every operand
     odd = {0: 7, 1: 23, 10: 5, 11: 29, 20: 3, 21: 37 if big else 21}
-    out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], odd, a, b,
+    out.append(wl.make_workload(dtype, compute, [0, 20, 1, 21], [10, 20, 11, 21], [0, 10, 1, 11], odd, a, b,
                                 name=f"tiles_scalar_{dtype}"))
     return out
 

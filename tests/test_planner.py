@@ -146,7 +146,11 @@ def test_ragged_contiguous_rows_and_columns_keep_their_vectors(host_handle):
     w32 = wl.make_workload("f32", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
     info, _ = plan(host_handle, w32)
     assert (info["x_vec"], info["y_vec"], info["cd_vec"]) == (4, 4, 4)
-    ext = {0: 15, 1: 13, 10: 17, 11: 11, 20: 16, 21: 4}  # M = 195, N = 187: too short to move a 256-wide tile back
+    ext = {0: 15, 1: 13, 10: 17, 11: 11, 20: 16, 21: 4}  # M = 195, N = 187: only tiles of at most 128 can be moved back
+    w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"], info["cd_vec"]) == (8, 8, 8) and max(info["tile_p"], info["tile_q"]) <= 128
+    ext = {0: 15, 1: 3, 10: 17, 11: 3, 20: 16, 21: 4}  # M = 45, N = 51: shorter than the smallest tile
     w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
     info, _ = plan(host_handle, w)
     assert (info["x_vec"], info["y_vec"], info["cd_vec"]) == (1, 1, 1)
