@@ -93,11 +93,12 @@ def measure_permutation(handle, w, steps, warmup, settle_s=0.25):
     for l in w["lensA"]:
         n *= l
     nbytes = n * wl.ELEM_BYTES[w["dtype"]]
-    A = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    padded = (nbytes + 3) // 4 * 4  # the fill writes whole 32-bit words
+    A = torch.empty(padded, dtype=torch.uint8, device="cuda")
     from hiptensor_amd._lib import lib as _native
     stream = torch.cuda.current_stream()
     # finite pseudo-random elements (class ids of the fill: 0 f16, 2 f32)
-    assert _native.hiptk_fill_pattern(A.data_ptr(), nbytes, 0 if w["dtype"] == "f16" else 2, stream.cuda_stream) == 0
+    assert _native.hiptk_fill_pattern(A.data_ptr(), padded, 0 if w["dtype"] == "f16" else 2, stream.cuda_stream) == 0
     B = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     p = wl.Permutation(handle, w)
     info = p.info(A.data_ptr(), B.data_ptr())

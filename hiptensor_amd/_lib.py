@@ -42,6 +42,8 @@ class PlanInfo(C.Structure):
         ("n_pdims", C.c_int32), ("n_qdims", C.c_int32), ("n_kdims", C.c_int32),
         ("workspace_bytes", C.c_uint64), ("kernel_uid", C.c_uint64),
         ("estimate_us", C.c_double), ("kernel_name", C.c_char * 96),
+        ("pack_a", C.c_int32), ("pack_b", C.c_int32), ("pack_bytes", C.c_uint64),
+        ("pack_a_kernel", C.c_char * 96), ("pack_b_kernel", C.c_char * 96),
     ]
 
 

@@ -240,7 +240,8 @@ def planInfo(plan):
     if st != 0:
         raise HiptensorError(st, "hiptensorAmdPlanInfo")
     out = {name: getattr(info, name) for name, _ in _lib.PlanInfo._fields_}
-    out["kernel_name"] = info.kernel_name.decode()
+    for name in ("kernel_name", "pack_a_kernel", "pack_b_kernel"):
+        out[name] = getattr(info, name).decode()
     return out
 
 

@@ -200,6 +200,7 @@ namespace
     }
 
     constexpr uint64_t WS_CAP = 512ull << 20; // most workspace split-K is ever allowed to ask for
+    constexpr uint64_t PACK_CAP = 8ull << 30; // most workspace packed copies of A and B may take
 
     // Uploads the eight offset tables as one device block and points prob at them.
     hiptensorStatus_t uploadTables(PlanState& st)
@@ -604,18 +605,22 @@ hiptensorStatus_t hiptensorContractionGetWorkspaceSize(const hiptensorHandle_t* 
         return HIPTENSOR_STATUS_NOT_INITIALIZED;
     if(pref == HIPTENSOR_WORKSPACE_MIN)
         return HIPTENSOR_STATUS_SUCCESS; // the single-pass kernels need none
-    hipta::GemmView view;
-    std::string     why;
-    if(hipta::build_view(problemFromDesc(*desc), view, why) != hipta::PlanStatus::OK)
+    // the most a plan can use: packed copies of both operands plus split-K partials
+    hipta::ContractionPlanChoice pc;
+    std::string                  why;
+    const hipta::ProblemIn       in = problemFromDesc(*desc);
+    if(hipta::plan_contraction(in, candidatesOf(find), PACK_CAP + WS_CAP, WS_CAP, h->model(), hipta::repack_mode_from_env(), pc, why)
+       != hipta::PlanStatus::OK)
         return HIPTENSOR_STATUS_SUCCESS; // nothing can run it: 0 bytes, like the reference
-    auto ranked = hipta::rank_choices(candidatesOf(find), view, WS_CAP, h->model());
-    if(ranked.empty())
+    if(pc.ranked.empty())
         return HIPTENSOR_STATUS_SUCCESS;
     if(pref == HIPTENSOR_WORKSPACE_RECOMMENDED)
-        *workspaceSize = ranked.front().ws_bytes;
+        *workspaceSize = pc.pack_bytes + pc.ranked.front().ws_bytes;
     else
-        for(const hipta::Choice& c : ranked)
-            *workspaceSize = std::max<uint64_t>(*workspaceSize, c.ws_bytes);
+    {
+        for(const hipta::Choice& c : pc.ranked)
+            *workspaceSize = std::max<uint64_t>(*workspaceSize, pc.pack_bytes + c.ws_bytes);
+    }
     return HIPTENSOR_STATUS_SUCCESS;
 }
 
@@ -660,13 +665,16 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
     const hipta::ProblemIn in = problemFromDesc(*desc);
     // HIPTENSOR_AMD_FORCE_KERNEL="tile[,splitK]" pins the kernel choice (testing / tuning aid)
     const char*            force = std::getenv("HIPTENSOR_AMD_FORCE_KERNEL");
-    const std::string      key = planKey(in, (int)find->mSelectionAlgorithm, workspaceSize) + (force ? std::string("|force=") + force : std::string());
+    const hipta::RepackMode repack = hipta::repack_mode_from_env();
+    const std::string       key    = planKey(in, (int)find->mSelectionAlgorithm, workspaceSize) + (force ? std::string("|force=") + force : std::string())
+                            + "|repack=" + std::to_string((int)repack);
     PlanState*             st  = h->lookup(key);
     if(!st)
     {
-        auto        fresh = std::make_unique<PlanState>();
-        std::string why;
-        switch(hipta::build_view(in, fresh->view, why))
+        auto                         fresh = std::make_unique<PlanState>();
+        std::string                  why;
+        hipta::ContractionPlanChoice pc;
+        switch(hipta::plan_contraction(in, candidatesOf(find), std::min<uint64_t>(workspaceSize, PACK_CAP + WS_CAP), WS_CAP, h->model(), repack, pc, why))
         {
         case hipta::PlanStatus::OK: break;
         case hipta::PlanStatus::INVALID:
@@ -681,12 +689,31 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
             log.errorf(fn, "Init contraction plan not successful: %s (%s)", why.c_str(), hiptensorGetErrorString(HIPTENSOR_STATUS_EXECUTION_FAILED));
             return HIPTENSOR_STATUS_EXECUTION_FAILED;
         }
-        const hipta::GemmView& v      = fresh->view;
-        auto                   ranked = hipta::rank_choices(candidatesOf(find), v, std::min<uint64_t>(workspaceSize, WS_CAP), h->model());
+        fresh->view                        = std::move(pc.view);
+        fresh->pack_a                      = pc.a;
+        fresh->pack_b                      = pc.b;
+        fresh->pack_bytes                  = pc.pack_bytes;
+        const hipta::GemmView&     v      = fresh->view;
+        std::vector<hipta::Choice> ranked = std::move(pc.ranked);
         if(ranked.empty())
         {
             log.errorf(fn, "Init contraction plan not successful: no kernel candidate (%s)", hiptensorGetErrorString(HIPTENSOR_STATUS_EXECUTION_FAILED));
             return HIPTENSOR_STATUS_EXECUTION_FAILED;
+        }
+        if((log.mask() & HIPTENSOR_LOG_LEVEL_HEURISTICS_TRACE) && (pc.a.on || pc.b.on))
+        {
+            char msg[256];
+            snprintf(msg,
+                     sizeof(msg),
+                     "packed copies: A %s (%s, %0.1f us), B %s (%s, %0.1f us), %lu bytes of workspace",
+                     pc.a.on ? "yes" : "no",
+                     pc.a.on ? hiptk_permute_kernel_name(&pc.a.perm) : "-",
+                     pc.a.est_us,
+                     pc.b.on ? "yes" : "no",
+                     pc.b.on ? hiptk_permute_kernel_name(&pc.b.perm) : "-",
+                     pc.b.est_us,
+                     (unsigned long)pc.pack_bytes);
+            log.heuristics(fn, msg);
         }
         if(log.mask() & HIPTENSOR_LOG_LEVEL_HEURISTICS_TRACE)
         {
@@ -741,7 +768,7 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         const hipta::Choice& c = ranked[pick];
         fresh->magic           = PlanState::MAGIC;
         fresh->sol             = c.sol;
-        fresh->ws_bytes        = c.ws_bytes;
+        fresh->ws_bytes        = fresh->pack_bytes + c.ws_bytes;
         fresh->est_us          = c.est_us;
         fresh->device          = h->device();
         fresh->compute         = (int)desc->mComputeType;
@@ -894,9 +921,6 @@ hiptensorStatus_t hiptensorContraction(const hiptensorHandle_t*          handle,
     packScalar(st->prob.cls, av, ab);
     packScalar(st->prob.cls, bv, bb);
 
-    const void* X = st->view.swapped ? B : A;
-    const void* Y = st->view.swapped ? A : B;
-
     const bool timed = (log.mask() & HIPTENSOR_LOG_LEVEL_PERF_TRACE) != 0;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if(timed)
@@ -905,8 +929,35 @@ hiptensorStatus_t hiptensorContraction(const hiptensorHandle_t*          handle,
             return HIPTENSOR_STATUS_HIP_ERROR;
         (void)hipEventRecord(e0, stream);
     }
-    int hipErr = 0;
-    int rc     = hiptk_contract(&st->prob, ab, bilinear ? bb : nullptr, X, Y, bilinear ? C : nullptr, D, workspace, workspaceSize, (void*)stream, &hipErr);
+    int  hipErr     = 0;
+    int  rc         = HIPTK_OK;
+    bool misaligned = false;
+    if(st->pack_bytes)
+    {
+        // the copies start at the first 256-byte boundary of the workspace; what follows them is
+        // left to the kernel (split-K partials)
+        const uintptr_t base = (reinterpret_cast<uintptr_t>(workspace) + hipta::PACK_ALIGN - 1) / hipta::PACK_ALIGN * hipta::PACK_ALIGN;
+        const uint64_t  lead = (uint64_t)(base - reinterpret_cast<uintptr_t>(workspace));
+        char*           wsb  = reinterpret_cast<char*>(base);
+        if(st->pack_a.on && rc == HIPTK_OK)
+        {
+            rc = hiptk_permute(&st->pack_a.perm, A, wsb + st->pack_a.offset, (void*)stream, &hipErr);
+            A  = wsb + st->pack_a.offset;
+        }
+        if(st->pack_b.on && rc == HIPTK_OK)
+        {
+            rc = hiptk_permute(&st->pack_b.perm, B, wsb + st->pack_b.offset, (void*)stream, &hipErr);
+            B  = wsb + st->pack_b.offset;
+        }
+        misaligned = rc == HIPTK_ERR_ARG; // the only argument a plan's own move can get wrong
+        const uint64_t used = st->pack_bytes - hipta::PACK_ALIGN + lead;
+        workspace           = wsb + (st->pack_bytes - hipta::PACK_ALIGN);
+        workspaceSize       = workspaceSize - used;
+    }
+    const void* X = st->view.swapped ? B : A;
+    const void* Y = st->view.swapped ? A : B;
+    if(rc == HIPTK_OK)
+        rc = hiptk_contract(&st->prob, ab, bilinear ? bb : nullptr, X, Y, bilinear ? C : nullptr, D, workspace, workspaceSize, (void*)stream, &hipErr);
     if(timed)
     {
         (void)hipEventRecord(e1, stream);
@@ -933,6 +984,13 @@ hiptensorStatus_t hiptensorContraction(const hiptensorHandle_t*          handle,
                      bytes / 1e6 / ms);
             log.perf(fn, msg);
         }
+    }
+    if(misaligned)
+    {
+        log.errorf(fn,
+                   "An operand is not aligned as its contraction descriptor declared (%s)",
+                   hiptensorGetErrorString(HIPTENSOR_STATUS_INVALID_VALUE));
+        return HIPTENSOR_STATUS_INVALID_VALUE;
     }
     switch(rc)
     {

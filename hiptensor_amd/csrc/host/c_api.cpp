@@ -310,6 +310,13 @@ extern "C" int hiptensorAmdPlanInfo(const void* plan, hiptensorAmdPlanInfo_t* ou
     out->kernel_uid          = st->sol->uid;
     out->estimate_us         = st->est_us;
     std::strncpy(out->kernel_name, st->kernel_name.c_str(), sizeof(out->kernel_name) - 1);
+    out->pack_a     = st->pack_a.on ? 1 : 0;
+    out->pack_b     = st->pack_b.on ? 1 : 0;
+    out->pack_bytes = st->pack_bytes;
+    if(st->pack_a.on)
+        std::strncpy(out->pack_a_kernel, hiptk_permute_kernel_name(&st->pack_a.perm), sizeof(out->pack_a_kernel) - 1);
+    if(st->pack_b.on)
+        std::strncpy(out->pack_b_kernel, hiptk_permute_kernel_name(&st->pack_b.perm), sizeof(out->pack_b_kernel) - 1);
     return 0;
 }
 

@@ -16,6 +16,7 @@
 
 #include "hiptk_kernels.h"
 #include "planner.hpp"
+#include "repack.hpp"
 #include "solution.hpp"
 
 namespace hipta
@@ -26,7 +27,9 @@ namespace hipta
         GemmView        view; // host copy of the folded problem (tables kept for inspection)
         hiptk_problem_t prob{}; // table pointers are device addresses (null on a host-only handle)
         const Solution* sol       = nullptr;
-        uint64_t        ws_bytes  = 0; // workspace the chosen split-K needs
+        uint64_t        ws_bytes  = 0; // workspace the plan needs: packed copies, then split-K partials
+        PackedOperand   pack_a, pack_b; // operands moved into a packed copy before the kernel runs
+        uint64_t        pack_bytes = 0; // leading part of the workspace that holds those copies
         void*           dev_block = nullptr; // one allocation holding all eight tables
         int             device    = -1;
         int             compute   = 0; // hiptensorComputeType_t (how alpha / beta are read)

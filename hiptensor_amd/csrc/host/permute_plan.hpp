@@ -26,7 +26,7 @@ namespace hipta
     {
         OK,
         EMPTY, // an extent is zero: nothing to do
-        BAD_RANK, // ranks differ
+        BAD_RANK, // ranks differ, or more than HIPTK_PERM_MAX_RANK modes are left after fusion
         BAD_MODES, // modeB is not a reordering of modeA, or a length disagrees
         TOO_LARGE // 2^31 elements or more
     };

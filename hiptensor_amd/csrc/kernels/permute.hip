@@ -116,6 +116,8 @@ namespace hiptk
         template <typename T>
         __device__ inline T element_op(T x, T alpha, int op_a, int op_b)
         {
+            if(op_a == HIPTK_PERM_OP_RAW)
+                return x; // a plain move: every bit pattern, NaN payloads included, arrives unchanged
             T y = x;
             if(op_a)
                 y = y * y;
@@ -840,7 +842,7 @@ namespace hiptk
         {
             if(!p || (p->elem_bytes != 2 && p->elem_bytes != 4) || p->rank < 1 || p->rank > HIPTK_PERM_MAX_RANK)
                 return false;
-            if((p->op_a | p->op_b) & ~1)
+            if(((p->op_a | p->op_b) & ~1) && !(p->op_a == HIPTK_PERM_OP_RAW && p->op_b == 0))
                 return false;
             int64_t n = 1;
             for(int d = 0; d < p->rank; ++d)

@@ -151,6 +151,11 @@ typedef struct hiptensorAmdPlanInfo
     uint64_t kernel_uid;
     double   estimate_us;
     char     kernel_name[96];
+    /* operands the plan first moves into a packed copy in the workspace (interleaved layouts
+     * that would otherwise be gathered element by element); the view above is that of the copies */
+    int32_t  pack_a, pack_b;
+    uint64_t pack_bytes;     /* leading part of workspace_bytes that holds the copies  */
+    char     pack_a_kernel[96], pack_b_kernel[96];
 } hiptensorAmdPlanInfo_t;
 int hiptensorAmdPlanInfo(const void* plan, hiptensorAmdPlanInfo_t* out);
 /* Copies offset table `which` (0 xp, 1 xk, 2 yq, 3 yk, 4 cp, 5 cq, 6 dp, 7 dq; logical

@@ -175,6 +175,7 @@ enum
 };
 
 #define HIPTK_PERM_MAX_RANK 6
+#define HIPTK_PERM_OP_RAW 2
 
 typedef struct hiptk_permute
 {
@@ -183,7 +184,8 @@ typedef struct hiptk_permute
     int32_t extent[HIPTK_PERM_MAX_RANK];
     int32_t a_stride[HIPTK_PERM_MAX_RANK]; /* elements                                            */
     int32_t b_stride[HIPTK_PERM_MAX_RANK];
-    int32_t op_a, op_b; /* 0: identity, 1: square                                                 */
+    int32_t op_a, op_b; /* 0: identity, 1: square; op_a = HIPTK_PERM_OP_RAW (with op_b = 0): the bits
+                         * are moved as they are, alpha is not applied                           */
     float   alpha;      /* multiplies in float for f32, rounded to half first for f16             */
     int32_t kernel;     /* HIPTK_PERM_*                                                           */
     int32_t mode_i, mode_j; /* TILED / ROWS: positions (in this struct's order) of the two tile modes */
