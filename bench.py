@@ -246,7 +246,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--settle", type=float, default=0.25,
                     help="seconds of untimed load before the warm-up steps (clock ramp of the device)")
-    ap.add_argument("--workload", default="cfg2_f16_scale")
+    ap.add_argument("--workload", default="cfg2_f16_scale",
+                    help="a baseline configuration (cfg1 ... cfg5), or interleaved_f16 / interleaved_f16_d_too / "
+                         "interleaved_f32: operands with interleaved modes, contracted from packed copies")
     ap.add_argument("--all", action="store_true", help="also time every other configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--permutation", action="store_true",
@@ -280,7 +282,7 @@ def main():
         print(json.dumps(out))
         return
     cfgs = wl.baseline_configs()
-    w = cfgs[a.workload]
+    w = cfgs[a.workload] if a.workload in cfgs else wl.interleaved_configs()[a.workload]
     r = measure(handle, w, a.steps, a.warmup, a.settle)
     fl = wl.flops(w)
     tflops = fl / (r["kernel_ms"] * 1e-3) / 1e12
@@ -295,7 +297,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": w["name"], "M": M, "N": N, "K": K, "op": "bilinear" if w["beta"] is not None else "scale",
-                   "kernel": r["info"]["kernel_name"], "split_k": r["info"]["split_k"]},
+                   "kernel": r["info"]["kernel_name"], "split_k": r["info"]["split_k"],
+                   "packed_copy_kernels": [k for k in (r["info"]["pack_a_kernel"], r["info"]["pack_b_kernel"]) if k]},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak,
                      "traffic": MEASURED_TRAFFIC_BYTES.get((w["name"], r["info"]["kernel_name"])),
                      "kernel_ms": r["kernel_ms"],

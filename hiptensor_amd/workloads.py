@@ -257,6 +257,21 @@ def baseline_configs():
     }
 
 
+def interleaved_configs():
+    """Layouts outside the baseline set: A and B stored with free and contracted modes
+    interleaved (A[m0,k0,m1,k1], runs of 15 elements), 4845 x 4845 x 1001.  In place they can only
+    be gathered element by element; with workspace the plan contracts packed copies."""
+    ext = {0: 15, 1: 323, 10: 15, 11: 323, 20: 7, 21: 143}
+    mA, mB = [0, 20, 1, 21], [10, 20, 11, 21]
+    c32 = api.HIPTENSOR_COMPUTE_32F
+    return {
+        "interleaved_f16": make_workload("f16", c32, mA, mB, [0, 1, 10, 11], ext, 1.0, None, name="interleaved_f16_scale_4845x4845x1001"),
+        "interleaved_f16_d_too": make_workload("f16", c32, mA, mB, [0, 10, 1, 11], ext, 1.0, 1.0,
+                                               name="interleaved_f16_bilinear_d_interleaved_4845x4845x1001"),
+        "interleaved_f32": make_workload("f32", c32, mA, mB, [0, 1, 10, 11], ext, 1.0, None, name="interleaved_f32_scale_4845x4845x1001"),
+    }
+
+
 def host_inputs(w, nan_gaps=True):
     """Seeded host buffers {"A", "B", "C" (or None)} plus spans."""
     A = fill_tensor(w["dtype"], w["lens"]["A"], w["strides"]["A"], SEED_A, nan_gaps)
