@@ -140,3 +140,46 @@ def test_large_interleaved_problem_is_packed_by_itself(gpu_handle, oracle_mod, m
     got0, info0 = gpu_util.run_gpu(gpu_handle, w, inp, return_info=True)
     assert info0["pack_a"] == 0 and info0["x_vec"] == 1
     cases.assert_parity(w, gl, cases.logical_view(w, got0), "packed against in place")
+
+
+def _random_problem(rng, k):
+    """Random storage orders for A, B and D (each dense, or padded after its fastest mode),
+    random small extents including 1, one to three modes per group."""
+    dtype = str(rng.choice(["f16", "bf16", "f32", "f64", "c32"]))
+    nm, nn, nk = (int(rng.integers(1, 4)) for _ in range(3))
+    pool = [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 24]
+    ext = {}
+    M, N, K = list(range(0, nm)), list(range(10, 10 + nn)), list(range(20, 20 + nk))
+    for m in M + N + K:
+        ext[m] = int(rng.choice(pool))
+    order = lambda modes: [int(x) for x in rng.permutation(modes)]
+    mA, mB, mD = order(M + K), order(N + K), order(M + N)
+    beta = None if rng.random() < 0.4 else 0.5
+    a, b = (1.1 + 1.2j, None if beta is None else 2.2 + 2.3j) if dtype == "c32" else (1.5, beta)
+    strides = {}
+    for t, modes in (("A", mA), ("B", mB), ("D", mD)):
+        lens = [ext[m] for m in modes]
+        pad = int(rng.choice([0, 0, 0, 1, 3]))
+        strides[t] = wl.storage_order_strides(modes, ext, modes, pad_after_first=pad)
+    return wl.make_workload(dtype, cases.COMPUTE[dtype], mA, mB, mD, ext, a, b, strideA=strides["A"], strideB=strides["B"],
+                            strideD=strides["D"], name=f"repack_random_{k}_{dtype}")
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_random_layouts_in_place_and_from_copies(gpu_handle, oracle_mod, monkeypatch, seed):
+    rng = np.random.default_rng(seed)
+    monkeypatch.delenv("HIPTENSOR_AMD_FORCE_KERNEL", raising=False)
+    packed = 0
+    for k in range(60):
+        w = _random_problem(rng, k)
+        inp = wl.host_inputs(w)
+        exp = cases.logical_view(w, oracle_mod.contract(w, inp["A"], inp["B"], inp["C"]))
+        for mode in ("0", "1"):
+            monkeypatch.setenv("HIPTENSOR_AMD_REPACK", mode)
+            print(f"[case] seed {seed} {w['name']} A{w['modes']['A']} B{w['modes']['B']} D{w['modes']['D']} "
+                  f"{w['extent']} strides {w['strides']} repack={mode}", flush=True)
+            got, info = gpu_util.run_gpu(gpu_handle, w, inp, return_info=True)
+            cases.assert_parity(w, cases.logical_view(w, got), exp, info["kernel_name"])
+            packed += info["pack_a"] + info["pack_b"]
+    print(f"[case] seed {seed}: {packed} operand copies", flush=True)
+    assert packed >= 20
