@@ -960,29 +960,58 @@ namespace hiptk
             return;
         }
         {
+            // Element by element through the offset tables.  D may alias C (and, for all the
+            // compiler knows, the tables), so it would fetch one offset, one C element and store
+            // one D element at a time; the offsets of a slab's 16 rows are therefore fetched once,
+            // ahead of the columns, and the 16 C elements of a column before the first store.
             const int pw = p0 + wp * WTP + 4 * (lane >> 5);
             const int qw = q0 + wq * WTQ + (lane & 31);
+            const bool bil = a.bilinear != 0;
+            uint32_t   dqo[TQ], cqo[TQ];
+            bool       qok[TQ];
 #pragma unroll
             for(int j = 0; j < TQ; j++)
             {
                 const int q = qw + j * 32;
-                if(!q_in(q))
-                    continue;
-                const uint32_t dqo = (uint32_t)a.dq[q];
-                const uint32_t cqo = a.bilinear ? (uint32_t)a.cq[q] : 0u;
+                qok[j]      = q_in(q);
+                // (the tables are padded beyond every index a tile can reach, with the offset of
+                // index 0: loads need no guard, only the stores do)
+                dqo[j] = (uint32_t)a.dq[q];
+                cqo[j] = bil ? (uint32_t)a.cq[q] : 0u;
+            }
 #pragma unroll
-                for(int i = 0; i < TP; i++)
+            for(int i = 0; i < TP; i++)
+            {
+                uint32_t dpo[16], cpo[16];
+                bool     pok[16];
+#pragma unroll
+                for(int r = 0; r < 16; r++)
+                {
+                    const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
+                    pok[r]      = p_in(p);
+                    dpo[r]      = (uint32_t)a.dp[p];
+                    cpo[r]      = bil ? (uint32_t)a.cp[p] : 0u;
+                }
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+                {
+                    if(!qok[j])
+                        continue;
+                    float c[16];
 #pragma unroll
                     for(int r = 0; r < 16; r++)
+                        c[r] = 0.f;
+                    if(bil)
                     {
-                        const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
-                        if(p_in(p))
-                        {
-                            const float c = a.bilinear ? Tr::out_to_f32(Cp[(uint32_t)a.cp[p] + cqo]) : 0.f;
-                            Dp[(uint32_t)a.dp[p] + dqo]
-                                = Tr::out_from_f32(Tr::axpby(alpha, acc[i][j][r], beta, c, a.bilinear != 0));
-                        }
+#pragma unroll
+                        for(int r = 0; r < 16; r++)
+                            c[r] = Tr::out_to_f32(Cp[cpo[r] + cqo[j]]);
                     }
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                        if(pok[r])
+                            Dp[dpo[r] + dqo[j]] = Tr::out_from_f32(Tr::axpby(alpha, acc[i][j][r], beta, c[r], bil));
+                }
             }
         }
     }

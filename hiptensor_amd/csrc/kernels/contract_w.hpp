@@ -593,38 +593,63 @@ namespace hiptk
         const E*   Cp  = (const E*)a.C;
         const bool bil = a.bilinear != 0;
         const bool aff = a.cd_affine != 0; // C / D offsets are index * stride: no table lookups
-        uint32_t   dqo[TQ], cqo[TQ];
+        // D may alias C (and, for all the compiler knows, the offset tables), so written naively
+        // every element is one dependent round trip: offset, C element, D store.  The offsets and C
+        // elements of four accumulator rows are therefore fetched together, ahead of their stores.
+        // A lane outside the extents fetches element (0, 0) instead, a valid address, and stores
+        // nothing.
+        uint32_t dqo[TQ], cqo[TQ];
+        bool     qok[TQ];
 #pragma unroll
         for(int j = 0; j < TQ; j++)
         {
-            // the q tables are padded with valid entries, so the lookup is safe beyond Q
-            const int q = qw + j * TILE;
-            dqo[j]      = aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
-            cqo[j]      = !bil ? 0u : aff ? (uint32_t)q * (uint32_t)a.cq_stride : (uint32_t)a.cq[q];
+            const int q  = qw + j * TILE;
+            qok[j]       = q_in(q);
+            const int qv = qok[j] ? q : 0;
+            dqo[j]       = aff ? (uint32_t)qv * (uint32_t)a.dq_stride : (uint32_t)a.dq[qv];
+            cqo[j]       = !bil ? 0u : aff ? (uint32_t)qv * (uint32_t)a.cq_stride : (uint32_t)a.cq[qv];
         }
+        constexpr int RB = 4;
+        static_assert(Tr::NREG % RB == 0, "accumulator rows are fetched four at a time");
 #pragma unroll
         for(int i = 0; i < TP; i++)
 #pragma unroll
-            for(int r = 0; r < Tr::NREG; r++)
+            for(int rb = 0; rb < Tr::NREG; rb += RB)
             {
-                const int p = pw + i * TILE + Tr::p_of(r, lane);
-                if(!p_in(p))
-                    continue;
-                const uint32_t dpo = aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p];
-                const uint32_t cpo = !bil ? 0u : aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p];
+                uint32_t dpo[RB], cpo[RB];
+                bool     pok[RB];
 #pragma unroll
-                for(int j = 0; j < TQ; j++)
+                for(int t = 0; t < RB; t++)
                 {
-                    if(q_in(qw + j * TILE))
-                    {
-                        const E* cptr = bil ? Cp + (cpo + cqo[j]) : nullptr;
-                        const E val = Tr::finish(Tr::get(acc[i][j], r), a.alpha, a.beta, bil, cptr);
-                        if constexpr(std::is_arithmetic<E>::value)
-                            __builtin_nontemporal_store(val, Dp + (dpo + dqo[j]));
-                        else
-                            Dp[dpo + dqo[j]] = val;
-                    }
+                    const int p  = pw + i * TILE + Tr::p_of(rb + t, lane);
+                    pok[t]       = p_in(p);
+                    const int pv = pok[t] ? p : 0;
+                    dpo[t]       = aff ? (uint32_t)pv * (uint32_t)a.dp_stride : (uint32_t)a.dp[pv];
+                    cpo[t]       = !bil ? 0u : aff ? (uint32_t)pv * (uint32_t)a.cp_stride : (uint32_t)a.cp[pv];
                 }
+                E cv[RB][TQ];
+                if(bil)
+                {
+#pragma unroll
+                    for(int t = 0; t < RB; t++)
+#pragma unroll
+                        for(int j = 0; j < TQ; j++)
+                            cv[t][j] = Cp[cpo[t] + cqo[j]];
+                }
+#pragma unroll
+                for(int t = 0; t < RB; t++)
+#pragma unroll
+                    for(int j = 0; j < TQ; j++)
+                    {
+                        if(pok[t] && qok[j])
+                        {
+                            const E val = Tr::finish(Tr::get(acc[i][j], rb + t), a.alpha, a.beta, bil, &cv[t][j]);
+                            if constexpr(std::is_arithmetic<E>::value)
+                                __builtin_nontemporal_store(val, Dp + (dpo[t] + dqo[j]));
+                            else
+                                Dp[dpo[t] + dqo[j]] = val;
+                        }
+                    }
             }
     }
 
