@@ -44,3 +44,17 @@ def test_permutation_validation_document(gpu_handle, oracle_mod, rank):
     run = run_permutation_cases(gpu_handle, oracle_mod, expanded, f"permutation_rank{rank}", thin)
     print(f"[case] permutation rank {rank}: {len(expanded)} expanded, {run} run", flush=True)
     assert run == (len(expanded) + thin - 1) // thin
+
+
+@pytest.mark.parametrize("name", ["bilinear_rank3", "scale_rank6", "complex_bilinear_rank4", "mode_permutations"])
+def test_validation_document_from_packed_copies(gpu_handle, oracle_mod, monkeypatch, name):
+    """The same documents with every eligible operand first moved into a packed copy inside the
+    workspace (HIPTENSOR_AMD_REPACK=1): the step the plan takes by itself for large operands with
+    interleaved modes, here forced onto the reference's own small shapes."""
+    monkeypatch.setenv("HIPTENSOR_AMD_REPACK", "1")
+    _, kind, text = next(d for d in DOCS if d[0] == name)
+    cfg = tc.loads(text, name)
+    expanded = tc.expand_combined(cfg) if kind == "combined" else tc.expand_sequence(cfg)
+    print(f"[case] {name} from packed copies: {len(expanded)} expanded cases", flush=True)
+    run, skipped = run_cases(gpu_handle, oracle_mod, expanded, name)
+    assert skipped == 0 and run > 0
