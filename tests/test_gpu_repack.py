@@ -183,3 +183,32 @@ def test_random_layouts_in_place_and_from_copies(gpu_handle, oracle_mod, monkeyp
             packed += info["pack_a"] + info["pack_b"]
     print(f"[case] seed {seed}: {packed} operand copies", flush=True)
     assert packed >= 20
+
+
+def test_declared_alignment_sizes_the_move(gpu_handle, oracle_mod, forced):
+    """The move into the copy uses vectors as wide as the alignment declared for the operand
+    allows: an operand declared 2-byte aligned may sit at any even address; one that sits below
+    its declared alignment is refused before anything is launched."""
+    import torch
+
+    w = layouts("f16", cases.COMPUTE["f16"])[4]  # A transposed: the tiled move kernels, 16-byte vectors
+    inp = wl.host_inputs(w)
+    exp = cases.logical_view(w, oracle_mod.contract(w, inp["A"], inp["B"], inp["C"]))
+    shifted = torch.empty(inp["A"].nbytes + 16, dtype=torch.uint8, device="cuda")
+    shifted[2:2 + inp["A"].nbytes].copy_(gpu_util.to_device(inp["A"]))
+    B = gpu_util.to_device(inp["B"])
+    stream = torch.cuda.current_stream().cuda_stream
+    for align_a, status in ((2, api.HIPTENSOR_STATUS_SUCCESS), (16, api.HIPTENSOR_STATUS_INVALID_VALUE)):
+        print(f"[case] A declared {align_a}-byte aligned, placed at +2 bytes", flush=True)
+        c = wl.Contraction(gpu_handle, w, align={"A": align_a, "B": 16, "C": 16, "D": 16})
+        assert c.info["pack_a"] == 1
+        D = gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"]))
+        ws = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+        st = c.run(shifted.data_ptr() + 2, B.data_ptr(), None, D.data_ptr(), ws.data_ptr(), stream)
+        torch.cuda.synchronize()
+        assert st == status
+        if st == api.HIPTENSOR_STATUS_SUCCESS:
+            got = D.cpu().numpy().view(wl.NP_STORE[w["dtype"]])
+            cases.assert_parity(w, cases.logical_view(w, got), exp, c.info["pack_a_kernel"])
+            assert "_r1_" in c.info["pack_a_kernel"], c.info["pack_a_kernel"]  # element-wise reads, vector writes
+        c.close()
