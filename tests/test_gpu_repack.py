@@ -212,3 +212,45 @@ def test_declared_alignment_sizes_the_move(gpu_handle, oracle_mod, forced):
             cases.assert_parity(w, cases.logical_view(w, got), exp, c.info["pack_a_kernel"])
             assert "_r1_" in c.info["pack_a_kernel"], c.info["pack_a_kernel"]  # element-wise reads, vector writes
         c.close()
+
+
+def test_packed_contraction_under_graph_capture(gpu_handle, oracle_mod, forced):
+    """Two moves and the contraction kernel are ordinary launches on the caller's stream: the
+    whole call is captured into one HIP graph and every replay, with fresh operands, matches
+    both the eager call and the oracle."""
+    import torch
+
+    w = layouts("f16", cases.COMPUTE["f16"])[0]
+    inp = wl.host_inputs(w)
+    A, B, Cd = (gpu_util.to_device(inp[k]) for k in "ABC")
+    D = gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"]))
+    De = torch.empty_like(D)
+    c = wl.Contraction(gpu_handle, w)
+    assert c.info["pack_a"] and c.info["pack_b"]
+    ws = torch.empty(int(c.workspace_bytes), dtype=torch.uint8, device="cuda")
+    assert c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(), ws.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.graph(g, stream=side):
+        st = c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(), ws.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert st == 0
+    rng = np.random.default_rng(5)
+    for rep in range(3):
+        print(f"[case] graph replay {rep}", flush=True)
+        newA = inp["A"].copy()
+        rng.shuffle(newA)
+        A.copy_(gpu_util.to_device(newA))
+        D.copy_(gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"])))
+        ws.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), De.data_ptr(), ws.data_ptr(), torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        got = D.cpu().numpy().view(wl.NP_STORE[w["dtype"]])
+        eager = De.cpu().numpy().view(wl.NP_STORE[w["dtype"]])
+        assert np.array_equal(got.view(np.uint8), eager.view(np.uint8)), f"replay {rep} differs from the eager call"
+        exp = oracle_mod.contract(w, newA, inp["B"], inp["C"])
+        cases.assert_parity(w, got, exp, f"graph replay {rep}")
+    c.close()
