@@ -99,7 +99,7 @@ namespace hipta
             // 15 elements: the element-wise fallback moves 1.2 (2-byte) to 2.0 TB/s (4-byte), the
             // tile kernels 1.6-3.2 TB/s (5-6 TB/s on large tensors with long runs)
             const double rate = po.perm.kernel == HIPTK_PERM_GATHER ? (pin.elem_bytes == 2 ? 1.2e6 : 2.0e6) : 2.5e6; // bytes / us
-            po.est_us         = 2.0 * raw / rate + 5.0;
+            po.est_us         = 2.0 * raw / rate + 3.0;
 
             packed       = t;
             packed.align = (uint32_t)PACK_ALIGN;

@@ -174,11 +174,11 @@ namespace hipta
         {
             // narrower gathers are issue bound: measured on 2040^3 f16 problems whose runs
             // admit 16 / 8 / 4 / 2 bytes per load: 456 / 395 / 209 / 114 TFLOP/s
-            // (16-bit classes); the f32 kernels with 4-byte gathers reach 0.79 of their 16-byte
-            // form (4845 x 4845 x 1001: 86 against 108 TFLOP/s)
+            // (16-bit classes); the f32 kernels with 4-byte gathers reach 0.75-0.79 of their 16-byte
+            // form (4845 x 4845 x 1001: 86 against 108 TFLOP/s; 1965 x 1965 x 1001: 115 against 86 us)
             const int    bytes = std::min(v.x_vec, v.y_vec) * v.elem_bytes;
             const bool   wide  = class_max_vec(v.cls) != 8;
-            const double f     = bytes >= 16 ? 1.0 : bytes >= 8 ? 0.87 : wide ? 0.79 : bytes >= 4 ? 0.45 : 0.25;
+            const double f     = bytes >= 16 ? 1.0 : bytes >= 8 ? 0.87 : wide ? 0.77 : bytes >= 4 ? 0.45 : 0.25;
             r.alone *= f;
             r.full *= f;
         }
