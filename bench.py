@@ -247,7 +247,8 @@ def main():
     ap.add_argument("--settle", type=float, default=0.25,
                     help="seconds of untimed load before the warm-up steps (clock ramp of the device)")
     ap.add_argument("--workload", default="cfg2_f16_scale",
-                    help="a baseline configuration (cfg1 ... cfg5), or interleaved_f16 / interleaved_f16_d_too / "
+                    help="a baseline configuration (cfg1 ... cfg5); rowmajor_{f16,bf16}_{scale,bilinear}: 4096^3 in "
+                         "the reference's default (NULL-stride) layout; interleaved_f16 / interleaved_f16_d_too / "
                          "interleaved_f32: operands with interleaved modes, contracted from packed copies")
     ap.add_argument("--all", action="store_true", help="also time every other configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -282,7 +283,7 @@ def main():
         print(json.dumps(out))
         return
     cfgs = wl.baseline_configs()
-    w = cfgs[a.workload] if a.workload in cfgs else wl.interleaved_configs()[a.workload]
+    w = cfgs[a.workload] if a.workload in cfgs else {**wl.interleaved_configs(), **wl.row_major_configs()}[a.workload]
     r = measure(handle, w, a.steps, a.warmup, a.settle)
     fl = wl.flops(w)
     tflops = fl / (r["kernel_ms"] * 1e-3) / 1e12

@@ -257,6 +257,23 @@ def baseline_configs():
     }
 
 
+def row_major_configs():
+    """Config 2's problem (4096^3 from six modes of extent 64) in the layout the reference gives a
+    descriptor created with NULL strides: packed with the last listed mode fastest
+    (library/src/hiptensor.cpp:106-214), so A and B are contiguous along k and D along n."""
+    ext = {0: 64, 1: 64, 10: 64, 11: 64, 20: 64, 21: 64}
+    mA, mB, mD = [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11]
+    rm = lambda modes: [64 ** (len(modes) - 1 - i) for i in range(len(modes))]
+    out = {}
+    for dtype in ("f16", "bf16"):
+        for beta in (None, 1.0):
+            op = "scale" if beta is None else "bilinear"
+            out[f"rowmajor_{dtype}_{op}"] = make_workload(
+                dtype, api.HIPTENSOR_COMPUTE_32F, mA, mB, mD, ext, 1.0, beta, strideA=rm(mA), strideB=rm(mB), strideD=rm(mD),
+                name=f"rowmajor_{dtype}_{op}_4096")
+    return out
+
+
 def interleaved_configs():
     """Layouts outside the baseline set: A and B stored with free and contracted modes
     interleaved (A[m0,k0,m1,k1], runs of 15 elements), 4845 x 4845 x 1001.  In place they can only
