@@ -829,6 +829,9 @@ namespace hiptk
             static_assert(32 * EP * 4 * WP * WQ <= 2 * STAGE * 2, "epilogue staging must fit the operand buffers");
             const int pw = p0 + wp * WTP;
             const int qw = q0 + wq * WTQ;
+            // One slab of C in flight, requested (after the look-ups behind its addresses) while the
+            // slab before it is staged.
+            auto one_in_flight = [&]() {
             const bool bil = a.bilinear != 0;
             const bool aff = a.cd_affine != 0;
             // Offsets and C values of a slab are fetched while the slab before it is being
@@ -953,6 +956,175 @@ namespace hiptk
                     if(cur.ok[v])
                         HIPTK_STORE_D((u32x4_t*)(Dp + cur.doff[v]), o[v]);
                 wave_lds_fence();
+            }
+            };
+            // Two slabs in flight.  One copy of the code per case (C read or not; offsets computed):
+            // where the choice is made at run time inside the loop, the compiler has to wait for
+            // every outstanding load wherever the paths join, and the overlap below is lost.
+            auto run = [&](auto aff_c, auto bil_c) {
+            constexpr bool aff = decltype(aff_c)::value;
+            constexpr bool bil = decltype(bil_c)::value;
+            // The C vectors of a slab are requested two slabs ahead of their use, and the table
+            // look-ups behind their addresses one slab before that.  (The compiler cannot move any
+            // of this itself: D may alias C and, for all it knows, the offset tables.)  Loads and
+            // stores complete in issue order, so a wait for a load also waits for every store issued
+            // before it: with this lead the youngest stores such a wait can catch are a slab old,
+            // and C loads, LDS staging and D stores of neighbouring slabs overlap.  A lane reads
+            // each C element before it writes the D element at the same place, and no lane reads an
+            // element another lane writes, so exact aliasing stays valid.
+            uint32_t dqo[NVEC], cqo[NVEC];
+            bool     qok[NVEC];
+#pragma unroll
+            for(int v = 0; v < NVEC; v++)
+            {
+                const int q = qw + ((v * 64 + lane) % VPR) * 8;
+                qok[v]      = q_in8(q);
+                // affine C / D (every benchmark-style packed layout): offsets are computed; else
+                // looked up (the tables are padded beyond every index a tile reaches, with the
+                // offset of index 0, so the look-ups need no guard)
+                dqo[v] = aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
+                cqo[v] = !bil ? 0u : aff ? (uint32_t)q * (uint32_t)a.cq_stride : (uint32_t)a.cq[q];
+            }
+            struct Offsets
+            {
+                uint32_t d[NVEC], c[NVEC];
+                bool     ok[NVEC];
+            };
+            auto prepare = [&](int i, Offsets& o) {
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    const int p        = pw + i * 32 + (v * 64 + lane) / VPR;
+                    o.ok[v]            = qok[v] && p_in(p);
+                    const uint32_t dpo = aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p];
+                    const uint32_t cpo = !bil ? 0u : aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p];
+                    // a vector outside the extents reads element 0 of C, a valid address, and is not stored
+                    o.d[v] = o.ok[v] ? dpo + dqo[v] : 0u;
+                    o.c[v] = o.ok[v] ? cpo + cqo[v] : 0u;
+                }
+            };
+            // two slabs in flight, and the offsets of the slab that is requested next
+            constexpr int NB = 2;
+            Offsets       off[NB], nxt;
+            u32x4_t       cbuf[NB][NVEC];
+            auto          request = [&](int b) {
+                if(bil)
+                {
+#pragma unroll
+                    for(int v = 0; v < NVEC; v++)
+                        cbuf[b][v] = *(const u32x4_t*)(Cp + off[b].c[v]);
+                }
+            };
+            // Two staging buffers per wave when the operand buffers have room for them: slab
+            // i+1 is written to LDS while slab i is read back, converted and stored.
+            constexpr bool DB = 2 * 32 * EP * 4 * WP * WQ <= 2 * STAGE * 2;
+            float* const   st0 = (float*)lds + wave * ((DB ? 2 : 1) * 32 * EP);
+            auto write_slab = [&](int i, float* dst) {
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                        dst[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
+            };
+            // (all look-ups of the first two slabs before their first C load: one wait, not two)
+            prepare(0, off[0]);
+            if constexpr(TP > 1)
+                prepare(1, off[1]);
+            request(0);
+            if constexpr(TP > 1)
+                request(1);
+            if constexpr(TP > NB)
+                prepare(NB, nxt);
+            if constexpr(DB)
+            {
+                write_slab(0, st0);
+                wave_lds_fence();
+            }
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+            {
+                const float* cur_st = st0 + (DB ? (i & 1) * 32 * EP : 0);
+                if constexpr(DB)
+                {
+                    if(i + 1 < TP)
+                        write_slab(i + 1, st0 + ((i + 1) & 1) * 32 * EP);
+                }
+                else
+                {
+                    write_slab(i, st0);
+                    wave_lds_fence();
+                }
+                // up to four of the slab's vectors are read from LDS together, then converted and stored
+                constexpr int HV = NVEC > 4 ? 4 : NVEC;
+#pragma unroll
+                for(int h = 0; h < NVEC; h += HV)
+                {
+                    f32x4_t lo[HV], hi[HV];
+#pragma unroll
+                    for(int w = 0; w < HV; w++)
+                    {
+                        const int    slot = (h + w) * 64 + lane;
+                        const float* src  = cur_st + (slot / VPR) * EP + (slot % VPR) * 8;
+                        lo[w]             = *(const f32x4_t*)src;
+                        hi[w]             = *(const f32x4_t*)(src + 4);
+                    }
+                    u32x4_t o[HV];
+#pragma unroll
+                    for(int w = 0; w < HV; w++)
+                    {
+                        float v8[8] = {lo[w][0], lo[w][1], lo[w][2], lo[w][3], hi[w][0], hi[w][1], hi[w][2], hi[w][3]};
+                        if(bil)
+                        {
+                            const u32x4_t c4 = cbuf[i % NB][h + w];
+#pragma unroll
+                            for(int e = 0; e < 8; e++)
+                            {
+                                const uint16_t cb = (uint16_t)(c4[e >> 1] >> ((e & 1) * 16));
+                                v8[e]             = alpha * v8[e] + beta * Tr::to_f32(cb);
+                            }
+                        }
+                        else
+                        {
+#pragma unroll
+                            for(int e = 0; e < 8; e++)
+                                v8[e] = alpha * v8[e];
+                        }
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                            o[w][e] = (uint32_t)Tr::from_f32(v8[2 * e]) | ((uint32_t)Tr::from_f32(v8[2 * e + 1]) << 16);
+                    }
+#pragma unroll
+                    for(int w = 0; w < HV; w++)
+                        if(off[i % NB].ok[h + w])
+                            HIPTK_STORE_D((u32x4_t*)(Dp + off[i % NB].d[h + w]), o[w]);
+                }
+                // this slab's registers are free: request the slab NB ahead, then look up the
+                // offsets of the one after that
+                if(i + NB < TP)
+                {
+                    off[i % NB] = nxt;
+                    request(i % NB);
+                }
+                if(i + NB + 1 < TP)
+                    prepare(i + NB + 1, nxt);
+                wave_lds_fence();
+            }
+            };
+            typedef std::integral_constant<bool, true>  Yes;
+            typedef std::integral_constant<bool, false> No;
+            // The 128-wide wave tiles of the four-wave kernels hold 8 vectors per lane and slab and
+            // have no registers to spare for a second slab.  With offsets from the tables the
+            // deeper lead did not pay either (rank-6 benchmark layout: 366-372 us against 374).
+            if constexpr(NVEC * TP > 16)
+                one_in_flight();
+            else
+            {
+                if(a.cd_affine == 0)
+                    one_in_flight();
+                else if(a.bilinear != 0)
+                    run(Yes{}, Yes{});
+                else
+                    run(Yes{}, No{});
             }
 #ifdef HIPTK_CLOCK_PROBE
             probe_out();
