@@ -60,8 +60,9 @@ namespace hiptk
             void*       B;
             uint32_t    n;
             int32_t     rank;
-            uint32_t    ext[HIPTK_PERM_MAX_RANK]; // in B's order, fastest first
+            uint32_t    ext[HIPTK_PERM_MAX_RANK]; // in B's order, fastest first; extents of 1 left out
             uint32_t    astr[HIPTK_PERM_MAX_RANK];
+            uint32_t    magic[HIPTK_PERM_MAX_RANK]; // floor(2^32 / ext) + 1
             float       alpha;
             int32_t     op_a, op_b;
         };
@@ -639,11 +640,20 @@ namespace hiptk
             const uint32_t idx = blockIdx.x * PERM_THREADS + threadIdx.x;
             if(idx >= g.n)
                 return;
+            // index -> coordinates by multiplication: with m = floor(2^32 / e) + 1 the high word of
+            // rem * m is the quotient or one more, for every 32-bit rem; one compare corrects it
             uint32_t rem = idx, aoff = 0;
             for(int d = 0; d < g.rank; ++d)
             {
-                const uint32_t c = rem % g.ext[d];
-                rem /= g.ext[d];
+                const uint32_t e = g.ext[d];
+                uint32_t       q = __umulhi(rem, g.magic[d]);
+                uint32_t       c = rem - q * e;
+                if((int32_t)c < 0)
+                {
+                    q -= 1;
+                    c += e;
+                }
+                rem = q;
                 aoff += c * g.astr[d];
             }
             const T alpha               = static_cast<T>(g.alpha);
@@ -999,11 +1009,18 @@ extern "C" int hiptk_permute(const hiptk_permute_t* p, const void* A, void* B, v
         std::sort(order, order + p->rank, [p](int x, int y) {
             return p->b_stride[x] != p->b_stride[y] ? p->b_stride[x] < p->b_stride[y] : x < y;
         });
+        int kept = 0;
         for(int d = 0; d < p->rank; ++d)
         {
-            g.ext[d]  = (uint32_t)p->extent[order[d]];
-            g.astr[d] = (uint32_t)p->a_stride[order[d]];
+            const uint32_t e = (uint32_t)p->extent[order[d]];
+            if(e == 1)
+                continue; // its coordinate is always 0
+            g.ext[kept]   = e;
+            g.astr[kept]  = (uint32_t)p->a_stride[order[d]];
+            g.magic[kept] = magic_of(e);
+            ++kept;
         }
+        g.rank = kept;
         const uint32_t grid = (uint32_t)((n + PERM_THREADS - 1) / PERM_THREADS);
         if(p->elem_bytes == 4)
             hipLaunchKernelGGL((permute_gather_kernel<float>), dim3(grid), dim3(PERM_THREADS), 0, s, g);
