@@ -976,12 +976,17 @@ hiptensorStatus_t hiptensorContraction(const hiptensorHandle_t*          handle,
             char                   msg[512];
             snprintf(msg,
                      sizeof(msg),
-                     "KernelId: %lu KernelName: %s, %0.3f ms, %0.3f TFlops, %0.3f GB/s",
+                     "KernelId: %lu KernelName: %s, %0.3f ms, %0.3f TFlops, %0.3f GB/s%s",
                      (unsigned long)st->sol->uid,
                      st->kernel_name.c_str(),
                      ms,
                      flops / 1e9 / ms,
-                     bytes / 1e6 / ms);
+                     bytes / 1e6 / ms,
+                     // (the time then covers the moves into the packed copies as well)
+                     st->pack_a.on && st->pack_b.on ? ", A and B from packed copies"
+                     : st->pack_a.on               ? ", A from a packed copy"
+                     : st->pack_b.on               ? ", B from a packed copy"
+                                                   : "");
             log.perf(fn, msg);
         }
     }
