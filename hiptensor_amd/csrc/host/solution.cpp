@@ -77,6 +77,7 @@ namespace hipta
         p.k_affine = v.k_affine;
         p.P        = v.P;
         p.Q        = v.Q;
+        p.K        = v.K;
         p.shift_p  = v.shift_p;
         p.shift_q  = v.shift_q;
         return hiptk_kernel_available(&p) != 0;

@@ -395,6 +395,519 @@ namespace hiptk
         }
     }
 
+    // Epilogue of the 16-bit kernels: D = alpha * acc (+ beta * C) for the wave tiles of one
+    // workgroup tile.  `lds` is the workgroup's whole LDS allocation of LDSCAP bytes, free by
+    // now (every wave has passed the main loop's last barrier); p0 / q0 are the first row / column
+    // the tile computed, p_own / q_own the first it stores (they differ for a tile that was moved
+    // back to end at P / Q).
+    // DEEP: two slabs of C in flight also for the 128-wide wave tiles (for kernels whose main loop
+    // leaves the registers for it).
+    template <typename Tr, int WP, int WQ, int TP, int TQ, int LDSCAP, bool DEEP = false>
+    __device__ __forceinline__ void epilogue_h(const KArgs& a, f32x16_t (&acc)[TP][TQ], uint16_t* lds, int p0, int q0, int p_own, int q_own)
+    {
+        constexpr int WTP = TP * 32, WTQ = TQ * 32;
+        const int     tid  = threadIdx.x;
+        const int     lane = tid & 63;
+        const int     wave = tid >> 6;
+        const int     wp   = wave / WQ;
+        const int     wq   = wave % WQ;
+        auto          p_in = [&](int p) { return p >= p_own && p < a.P; };
+        auto          q_in = [&](int q) { return q >= q_own && q < a.Q; };
+        // a vector of 8 columns is stored when any of it is this tile's (the others are the
+        // neighbour's, recomputed here to the same values)
+        auto q_in8 = [&](int q) { return q + 8 > q_own && q < a.Q; };
+        const float alpha = (float)a.alpha[0];
+        const float beta  = (float)a.beta[0];
+        if(a.split_k > 1)
+        {
+            const int pw = p0 + wp * WTP + 4 * (lane >> 5);
+            const int qw = q0 + wq * WTQ + (lane & 31);
+            float*    ws = (float*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+            {
+                const int q = qw + j * 32;
+                if(!q_in(q))
+                    continue;
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                    {
+                        const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
+                        if(p_in(p))
+                            ws[(size_t)p * a.Q + q] = acc[i][j][r];
+                    }
+            }
+            return;
+        }
+        typedef typename Tr::out_t out_t;
+        out_t*       Dp = (out_t*)a.D;
+        const out_t* Cp = (const out_t*)a.C;
+        // (measured: a gain only for the wide wave tiles; and the staging has to fit)
+        if constexpr(sizeof(out_t) == 2 && WTQ >= 128 && 2 * WTQ * 36 * 2 * WP * WQ <= LDSCAP)
+        if(a.cd_vec == 8 && !a.bilinear)
+        {
+            // Scale with D contiguous along q in runs of 8.  The results are converted to their
+            // 16-bit type in the accumulator layout (lane = column q, 4 consecutive registers =
+            // 4 consecutive rows p) and transposed through LDS at half the f32 volume: a slab is
+            // staged as [q][32 rows + 4] halves with one ds_write_b64 per 4 registers, and read
+            // back with the transposing ds_read_b64_tr_b16, which hands every lane 4 consecutive
+            // q of one row; two of them make the 16-byte store.  A 16-lane group covers 4 rows x
+            // 32 q, a store instruction 4 rows x 256 contiguous bytes (8 x 128 for 64-wide wave
+            // tiles).  The 72-byte column pitch keeps both the writes and the reads conflict free.
+            constexpr int PH   = 36; // halves per staged column: 32 rows + pad
+            constexpr int NVEC = (32 * WTQ / 8) / 64; // 16-byte stores per lane and slab
+            constexpr int QB   = WTQ / 32; // 32-column blocks per wave tile
+            static_assert(2 * WTQ * PH * 2 * WP * WQ <= LDSCAP, "epilogue staging must fit the operand buffers");
+            typedef short4_t __attribute__((address_space(3))) * lds_s4_ptr;
+            uint16_t* const st0 = lds + wave * (2 * WTQ * PH);
+            const int       pw  = p0 + wp * WTP;
+            const int       qw  = q0 + wq * WTQ;
+            const bool      aff = a.cd_affine != 0;
+            const int       L   = lane & 15;
+            const int       G   = lane >> 4;
+            // this lane's row within a slab and first column, per store vector
+            int      prow[NVEC], qcol[NVEC];
+            uint32_t dqo[NVEC];
+            bool     qok[NVEC];
+#pragma unroll
+            for(int v = 0; v < NVEC; v++)
+            {
+                const int u = v * 4 + G; // (row quad, column block) unit of this 16-lane group
+                prow[v]     = 4 * (u / QB) + (L & 3);
+                qcol[v]     = 32 * (u % QB) + 8 * (L >> 2);
+                const int q = qw + qcol[v];
+                qok[v]      = q_in8(q);
+                dqo[v]      = !qok[v] ? 0u : aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
+            }
+            uint32_t doff[2][NVEC];
+            auto     offsets = [&](int i, uint32_t (&d)[NVEC]) {
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    const int p = pw + i * 32 + prow[v];
+                    d[v] = !(qok[v] && p_in(p)) ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
+                }
+            };
+            auto write_slab = [&](int i, uint16_t* dst) {
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+#pragma unroll
+                    for(int g = 0; g < 4; g++)
+                    {
+                        u32x2_t w;
+                        w[0] = (uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g]) | ((uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 1]) << 16);
+                        w[1] = (uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 2]) | ((uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 3]) << 16);
+                        *(u32x2_t*)(dst + (j * 32 + (lane & 31)) * PH + 8 * g + 4 * (lane >> 5)) = w;
+                    }
+            };
+            offsets(0, doff[0]);
+            write_slab(0, st0);
+            wave_lds_fence();
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+            {
+                const uint16_t* cur = st0 + (i & 1) * (WTQ * PH);
+                if(i + 1 < TP)
+                {
+                    offsets(i + 1, doff[(i + 1) & 1]);
+                    write_slab(i + 1, st0 + ((i + 1) & 1) * (WTQ * PH));
+                }
+                u32x4_t o[NVEC];
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    // the word this lane supplies: column qcol-block + 8 * (L % 4) + L / 4, the group's 4 rows
+                    const int       u   = v * 4 + G;
+                    const uint16_t* src = cur + (32 * (u % QB) + 8 * (L & 3) + (L >> 2)) * PH + 4 * (u / QB);
+                    const short4_t  lo  = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(src));
+                    const short4_t  hi  = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(src + 4 * PH));
+                    const u32x2_t   l2  = __builtin_bit_cast(u32x2_t, lo);
+                    const u32x2_t   h2  = __builtin_bit_cast(u32x2_t, hi);
+                    o[v]                = u32x4_t{l2[0], l2[1], h2[0], h2[1]};
+                }
+                // table-driven offsets are loads: await the next slab's before this slab's stores
+                // go out (loads and stores share one in-order counter)
+                if(!aff)
+                    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                    if(qok[v] && p_in(pw + i * 32 + prow[v]))
+                        HIPTK_STORE_D((u32x4_t*)(Dp + doff[i & 1][v]), o[v]);
+                wave_lds_fence();
+            }
+            return;
+        }
+        if constexpr(sizeof(out_t) == 2)
+        if(a.cd_vec == 8)
+        {
+            // C and D are contiguous along q in runs of 8: route each 32-row slab of the
+            // wave's accumulators through LDS (the operand buffers are free now) so that a
+            // lane ends up with 8 consecutive q of one row and moves them as one 16-byte
+            // access; 16 lanes cover 256 contiguous bytes of a row.
+            constexpr int EP   = WTQ + 4; // floats per staged row
+            constexpr int VPR  = WTQ / 8; // 8-element vectors per staged row
+            constexpr int NVEC = (32 * WTQ / 8) / 64; // vectors per lane and slab
+            static_assert(32 * EP * 4 * WP * WQ <= LDSCAP, "epilogue staging must fit the operand buffers");
+            const int pw = p0 + wp * WTP;
+            const int qw = q0 + wq * WTQ;
+            // One slab of C in flight, requested (after the look-ups behind its addresses) while the
+            // slab before it is staged.
+            auto one_in_flight = [&]() {
+            const bool bil = a.bilinear != 0;
+            const bool aff = a.cd_affine != 0;
+            // Offsets and C values of a slab are fetched while the slab before it is being
+            // written, so that table look-ups, C loads and D stores of different vectors are
+            // all in flight together instead of one dependent round trip per vector.  (The
+            // compiler cannot hoist them itself: D may alias C.)  A lane reads every C element
+            // before it writes the D element at the same place, so exact aliasing stays valid.
+            uint32_t dqo[NVEC], cqo[NVEC];
+            bool     qok[NVEC];
+#pragma unroll
+            for(int v = 0; v < NVEC; v++)
+            {
+                const int q = qw + ((v * 64 + lane) % VPR) * 8;
+                qok[v]      = q_in8(q);
+                // affine C / D (every benchmark-style packed layout): offsets are computed, so the
+                // epilogue starts without a round trip to the offset tables
+                dqo[v] = !qok[v] ? 0u : aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
+                cqo[v] = !(qok[v] && bil) ? 0u : aff ? (uint32_t)q * (uint32_t)a.cq_stride : (uint32_t)a.cq[q];
+            }
+            struct Slab
+            {
+                u32x4_t  c[NVEC];
+                uint32_t doff[NVEC];
+                bool     ok[NVEC];
+            };
+            Slab sl[2];
+            auto prefetch = [&](int i, Slab& s) {
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    const int p = pw + i * 32 + (v * 64 + lane) / VPR;
+                    s.ok[v]     = qok[v] && p_in(p);
+                    s.doff[v]   = !s.ok[v] ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
+                    u32x4_t c4  = {0u, 0u, 0u, 0u};
+                    if(s.ok[v] && bil)
+                        c4 = *(const u32x4_t*)(Cp + ((aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p]) + cqo[v]));
+                    s.c[v] = c4;
+                }
+            };
+            // Two staging buffers per wave when the operand buffers have room for them: slab
+            // i+1 is written to LDS while slab i is read back, converted and stored.
+            constexpr bool DB = 2 * 32 * EP * 4 * WP * WQ <= LDSCAP;
+            float* const   st0 = (float*)lds + wave * ((DB ? 2 : 1) * 32 * EP);
+            auto write_slab = [&](int i, float* dst) {
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                        dst[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
+            };
+            prefetch(0, sl[0]);
+            if constexpr(DB)
+            {
+                write_slab(0, st0);
+                wave_lds_fence();
+            }
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+            {
+                const float* cur_st = st0 + (DB ? (i & 1) * 32 * EP : 0);
+                if constexpr(DB)
+                {
+                    if(i + 1 < TP)
+                    {
+                        prefetch(i + 1, sl[(i + 1) & 1]);
+                        write_slab(i + 1, st0 + ((i + 1) & 1) * 32 * EP);
+                    }
+                }
+                else
+                {
+                    write_slab(i, st0);
+                    if(i + 1 < TP)
+                        prefetch(i + 1, sl[(i + 1) & 1]);
+                    wave_lds_fence();
+                }
+                const Slab& cur = sl[i & 1];
+                // all of the slab's vectors are read from LDS before any is converted and stored
+                f32x4_t lo[NVEC], hi[NVEC];
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    const int    slot = v * 64 + lane;
+                    const float* src  = cur_st + (slot / VPR) * EP + (slot % VPR) * 8;
+                    lo[v]             = *(const f32x4_t*)src;
+                    hi[v]             = *(const f32x4_t*)(src + 4);
+                }
+                u32x4_t o[NVEC];
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    float v8[8] = {lo[v][0], lo[v][1], lo[v][2], lo[v][3], hi[v][0], hi[v][1], hi[v][2], hi[v][3]};
+                    if(bil)
+                    {
+                        const u32x4_t c4 = cur.c[v];
+#pragma unroll
+                        for(int e = 0; e < 8; e++)
+                        {
+                            const uint16_t cb = (uint16_t)(c4[e >> 1] >> ((e & 1) * 16));
+                            v8[e]             = alpha * v8[e] + beta * Tr::to_f32(cb);
+                        }
+                    }
+                    else
+                    {
+#pragma unroll
+                        for(int e = 0; e < 8; e++)
+                            v8[e] = alpha * v8[e];
+                    }
+#pragma unroll
+                    for(int e = 0; e < 4; e++)
+                        o[v][e] = (uint32_t)Tr::from_f32(v8[2 * e]) | ((uint32_t)Tr::from_f32(v8[2 * e + 1]) << 16);
+                }
+                // Loads and stores share one in-order counter, so waiting for a load also waits
+                // for every store issued before it.  The next slab's prefetch is therefore
+                // awaited here, before this slab's stores are issued: the only stores it can
+                // wait for are the previous slab's, a whole slab old, and this slab's stores
+                // then drain while the next slab is converted.
+                // (With computed offsets and no C there are no loads, and nothing to wait for.)
+                if(bil || !aff)
+                    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                    if(cur.ok[v])
+                        HIPTK_STORE_D((u32x4_t*)(Dp + cur.doff[v]), o[v]);
+                wave_lds_fence();
+            }
+            };
+            // Two slabs in flight.  One copy of the code per case (C read or not; offsets computed):
+            // where the choice is made at run time inside the loop, the compiler has to wait for
+            // every outstanding load wherever the paths join, and the overlap below is lost.
+            auto run = [&](auto aff_c, auto bil_c) {
+            constexpr bool aff = decltype(aff_c)::value;
+            constexpr bool bil = decltype(bil_c)::value;
+            // The C vectors of a slab are requested two slabs ahead of their use, and the table
+            // look-ups behind their addresses one slab before that.  (The compiler cannot move any
+            // of this itself: D may alias C and, for all it knows, the offset tables.)  Loads and
+            // stores complete in issue order, so a wait for a load also waits for every store issued
+            // before it: with this lead the youngest stores such a wait can catch are a slab old,
+            // and C loads, LDS staging and D stores of neighbouring slabs overlap.  A lane reads
+            // each C element before it writes the D element at the same place, and no lane reads an
+            // element another lane writes, so exact aliasing stays valid.
+            uint32_t dqo[NVEC], cqo[NVEC];
+            bool     qok[NVEC];
+#pragma unroll
+            for(int v = 0; v < NVEC; v++)
+            {
+                const int q = qw + ((v * 64 + lane) % VPR) * 8;
+                qok[v]      = q_in8(q);
+                // affine C / D (every benchmark-style packed layout): offsets are computed; else
+                // looked up (the tables are padded beyond every index a tile reaches, with the
+                // offset of index 0, so the look-ups need no guard)
+                dqo[v] = aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
+                cqo[v] = !bil ? 0u : aff ? (uint32_t)q * (uint32_t)a.cq_stride : (uint32_t)a.cq[q];
+            }
+            struct Offsets
+            {
+                uint32_t d[NVEC], c[NVEC];
+                bool     ok[NVEC];
+            };
+            auto prepare = [&](int i, Offsets& o) {
+#pragma unroll
+                for(int v = 0; v < NVEC; v++)
+                {
+                    const int p        = pw + i * 32 + (v * 64 + lane) / VPR;
+                    o.ok[v]            = qok[v] && p_in(p);
+                    const uint32_t dpo = aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p];
+                    const uint32_t cpo = !bil ? 0u : aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p];
+                    // a vector outside the extents reads element 0 of C, a valid address, and is not stored
+                    o.d[v] = o.ok[v] ? dpo + dqo[v] : 0u;
+                    o.c[v] = o.ok[v] ? cpo + cqo[v] : 0u;
+                }
+            };
+            // two slabs in flight, and the offsets of the slab that is requested next
+            constexpr int NB = 2;
+            Offsets       off[NB], nxt;
+            u32x4_t       cbuf[NB][NVEC];
+            auto          request = [&](int b) {
+                if(bil)
+                {
+#pragma unroll
+                    for(int v = 0; v < NVEC; v++)
+                        cbuf[b][v] = *(const u32x4_t*)(Cp + off[b].c[v]);
+                }
+            };
+            // Two staging buffers per wave when the operand buffers have room for them: slab
+            // i+1 is written to LDS while slab i is read back, converted and stored.
+            constexpr bool DB = 2 * 32 * EP * 4 * WP * WQ <= LDSCAP;
+            float* const   st0 = (float*)lds + wave * ((DB ? 2 : 1) * 32 * EP);
+            auto write_slab = [&](int i, float* dst) {
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                        dst[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
+            };
+            // (all look-ups of the first two slabs before their first C load: one wait, not two)
+            prepare(0, off[0]);
+            if constexpr(TP > 1)
+                prepare(1, off[1]);
+            request(0);
+            if constexpr(TP > 1)
+                request(1);
+            if constexpr(TP > NB)
+                prepare(NB, nxt);
+            if constexpr(DB)
+            {
+                write_slab(0, st0);
+                wave_lds_fence();
+            }
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+            {
+                const float* cur_st = st0 + (DB ? (i & 1) * 32 * EP : 0);
+                if constexpr(DB)
+                {
+                    if(i + 1 < TP)
+                        write_slab(i + 1, st0 + ((i + 1) & 1) * 32 * EP);
+                }
+                else
+                {
+                    write_slab(i, st0);
+                    wave_lds_fence();
+                }
+                // up to four of the slab's vectors are read from LDS together, then converted and stored
+                constexpr int HV = NVEC > 4 ? 4 : NVEC;
+#pragma unroll
+                for(int h = 0; h < NVEC; h += HV)
+                {
+                    f32x4_t lo[HV], hi[HV];
+#pragma unroll
+                    for(int w = 0; w < HV; w++)
+                    {
+                        const int    slot = (h + w) * 64 + lane;
+                        const float* src  = cur_st + (slot / VPR) * EP + (slot % VPR) * 8;
+                        lo[w]             = *(const f32x4_t*)src;
+                        hi[w]             = *(const f32x4_t*)(src + 4);
+                    }
+                    u32x4_t o[HV];
+#pragma unroll
+                    for(int w = 0; w < HV; w++)
+                    {
+                        float v8[8] = {lo[w][0], lo[w][1], lo[w][2], lo[w][3], hi[w][0], hi[w][1], hi[w][2], hi[w][3]};
+                        if(bil)
+                        {
+                            const u32x4_t c4 = cbuf[i % NB][h + w];
+#pragma unroll
+                            for(int e = 0; e < 8; e++)
+                            {
+                                const uint16_t cb = (uint16_t)(c4[e >> 1] >> ((e & 1) * 16));
+                                v8[e]             = alpha * v8[e] + beta * Tr::to_f32(cb);
+                            }
+                        }
+                        else
+                        {
+#pragma unroll
+                            for(int e = 0; e < 8; e++)
+                                v8[e] = alpha * v8[e];
+                        }
+#pragma unroll
+                        for(int e = 0; e < 4; e++)
+                            o[w][e] = (uint32_t)Tr::from_f32(v8[2 * e]) | ((uint32_t)Tr::from_f32(v8[2 * e + 1]) << 16);
+                    }
+#pragma unroll
+                    for(int w = 0; w < HV; w++)
+                        if(off[i % NB].ok[h + w])
+                            HIPTK_STORE_D((u32x4_t*)(Dp + off[i % NB].d[h + w]), o[w]);
+                }
+                // this slab's registers are free: request the slab NB ahead, then look up the
+                // offsets of the one after that
+                if(i + NB < TP)
+                {
+                    off[i % NB] = nxt;
+                    request(i % NB);
+                }
+                if(i + NB + 1 < TP)
+                    prepare(i + NB + 1, nxt);
+                wave_lds_fence();
+            }
+            };
+            typedef std::integral_constant<bool, true>  Yes;
+            typedef std::integral_constant<bool, false> No;
+            // The 128-wide wave tiles of the four-wave kernels hold 8 vectors per lane and slab and
+            // have no registers to spare for a second slab.  With offsets from the tables the
+            // deeper lead did not pay either (rank-6 benchmark layout: 366-372 us against 374).
+            if constexpr(NVEC * TP > 16 && !DEEP)
+                one_in_flight();
+            else
+            {
+                if(a.cd_affine == 0)
+                    one_in_flight();
+                else if(a.bilinear != 0)
+                    run(Yes{}, Yes{});
+                else
+                    run(Yes{}, No{});
+            }
+            return;
+        }
+        {
+            // Element by element through the offset tables.  D may alias C (and, for all the
+            // compiler knows, the tables), so it would fetch one offset, one C element and store
+            // one D element at a time; the offsets of a slab's 16 rows are therefore fetched once,
+            // ahead of the columns, and the 16 C elements of a column before the first store.
+            const int pw = p0 + wp * WTP + 4 * (lane >> 5);
+            const int qw = q0 + wq * WTQ + (lane & 31);
+            const bool bil = a.bilinear != 0;
+            uint32_t   dqo[TQ], cqo[TQ];
+            bool       qok[TQ];
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+            {
+                const int q = qw + j * 32;
+                qok[j]      = q_in(q);
+                // (the tables are padded beyond every index a tile can reach, with the offset of
+                // index 0: loads need no guard, only the stores do)
+                dqo[j] = (uint32_t)a.dq[q];
+                cqo[j] = bil ? (uint32_t)a.cq[q] : 0u;
+            }
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+            {
+                uint32_t dpo[16], cpo[16];
+                bool     pok[16];
+#pragma unroll
+                for(int r = 0; r < 16; r++)
+                {
+                    const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
+                    pok[r]      = p_in(p);
+                    dpo[r]      = (uint32_t)a.dp[p];
+                    cpo[r]      = bil ? (uint32_t)a.cp[p] : 0u;
+                }
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+                {
+                    if(!qok[j])
+                        continue;
+                    float c[16];
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                        c[r] = 0.f;
+                    if(bil)
+                    {
+#pragma unroll
+                        for(int r = 0; r < 16; r++)
+                            c[r] = Tr::out_to_f32(Cp[cpo[r] + cqo[j]]);
+                    }
+#pragma unroll
+                    for(int r = 0; r < 16; r++)
+                        if(pok[r])
+                            Dp[dpo[r] + dqo[j]] = Tr::out_from_f32(Tr::axpby(alpha, acc[i][j][r], beta, c[r], bil));
+                }
+            }
+        }
+    }
+
     template <typename Tr,
               int  BP,
               int  BQ,
@@ -424,11 +937,6 @@ namespace hiptk
         const int wave = tid >> 6;
         const int wp   = wave / WQ;
         const int wq   = wave % WQ;
-#ifdef HIPTK_CLOCK_PROBE
-        // diagnostic build: shader-clock cycles of the main loop and 100 MHz wall-clock stamps
-        // of the kernel's stages go to the workspace (8 x int64 per workgroup, first 256)
-        const long long cp_c0 = clock64(), cp_w0 = wall_clock64();
-#endif
 
         int tp, tq;
         tile_coords(blockIdx.x, a.tiles_p, a.tiles_q, tp, tq);
@@ -437,11 +945,6 @@ namespace hiptk
         const int p_own = tp * BP, q_own = tq * BQ;
         const int p0    = (a.shift_p && p_own + BP > a.P) ? a.P - BP : p_own;
         const int q0    = (a.shift_q && q_own + BQ > a.Q) ? a.Q - BQ : q_own;
-        auto      p_in  = [&](int p) { return p >= p_own && p < a.P; };
-        auto      q_in  = [&](int q) { return q >= q_own && q < a.Q; };
-        // a vector of 8 columns is stored when any of it is this tile's (the others are the
-        // neighbour's, recomputed here to the same values)
-        auto q_in8 = [&](int q) { return q + 8 > q_own && q < a.Q; };
 
         const int kt_begin = blockIdx.z * a.ktiles_per_split;
         int       kt_end   = kt_begin + a.ktiles_per_split;
@@ -518,9 +1021,6 @@ namespace hiptk
             lds_barrier();
         }
 
-#ifdef HIPTK_CLOCK_PROBE
-        const long long cp_c1 = clock64(), cp_w1 = wall_clock64();
-#endif
         int buf = 0;
         int kt  = kt_begin;
         // steady state: tile kt+2 exists and is a full tile
@@ -672,520 +1172,7 @@ namespace hiptk
             buf ^= 1;
         }
 
-        // ---- epilogue ----
-#ifdef HIPTK_CLOCK_PROBE
-        const long long cp_c2 = clock64(), cp_w2 = wall_clock64();
-        auto            probe_out = [&]() {
-            __builtin_amdgcn_s_waitcnt(0);
-            if(a.ws && a.split_k == 1 && tid == 0 && blockIdx.x < 256)
-            {
-                long long* o = (long long*)a.ws + 8 * blockIdx.x;
-                o[0]         = cp_c2 - cp_c1; // main loop, shader cycles
-                o[1]         = cp_w2 - cp_w1; // main loop, wall ticks
-                o[2]         = cp_w0;
-                o[3]         = cp_w1;
-                o[4]         = cp_w2;
-                o[5]         = wall_clock64();
-                o[6]         = cp_c1 - cp_c0;
-            }
-        };
-#endif
-        const float alpha = (float)a.alpha[0];
-        const float beta  = (float)a.beta[0];
-        if(a.split_k > 1)
-        {
-            const int pw = p0 + wp * WTP + 4 * (lane >> 5);
-            const int qw = q0 + wq * WTQ + (lane & 31);
-            float*    ws = (float*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
-#pragma unroll
-            for(int j = 0; j < TQ; j++)
-            {
-                const int q = qw + j * 32;
-                if(!q_in(q))
-                    continue;
-#pragma unroll
-                for(int i = 0; i < TP; i++)
-#pragma unroll
-                    for(int r = 0; r < 16; r++)
-                    {
-                        const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
-                        if(p_in(p))
-                            ws[(size_t)p * a.Q + q] = acc[i][j][r];
-                    }
-            }
-            return;
-        }
-        typedef typename Tr::out_t out_t;
-        out_t*       Dp = (out_t*)a.D;
-        const out_t* Cp = (const out_t*)a.C;
-        // (measured: a gain only for the wide wave tiles; and the staging has to fit)
-        if constexpr(sizeof(out_t) == 2 && WTQ >= 128 && 2 * WTQ * 36 * 2 * WP * WQ <= 2 * STAGE * 2)
-        if(a.cd_vec == 8 && !a.bilinear)
-        {
-            // Scale with D contiguous along q in runs of 8.  The results are converted to their
-            // 16-bit type in the accumulator layout (lane = column q, 4 consecutive registers =
-            // 4 consecutive rows p) and transposed through LDS at half the f32 volume: a slab is
-            // staged as [q][32 rows + 4] halves with one ds_write_b64 per 4 registers, and read
-            // back with the transposing ds_read_b64_tr_b16, which hands every lane 4 consecutive
-            // q of one row; two of them make the 16-byte store.  A 16-lane group covers 4 rows x
-            // 32 q, a store instruction 4 rows x 256 contiguous bytes (8 x 128 for 64-wide wave
-            // tiles).  The 72-byte column pitch keeps both the writes and the reads conflict free.
-            constexpr int PH   = 36; // halves per staged column: 32 rows + pad
-            constexpr int NVEC = (32 * WTQ / 8) / 64; // 16-byte stores per lane and slab
-            constexpr int QB   = WTQ / 32; // 32-column blocks per wave tile
-            static_assert(2 * WTQ * PH * 2 * WP * WQ <= 2 * STAGE * 2, "epilogue staging must fit the operand buffers");
-            typedef short4_t __attribute__((address_space(3))) * lds_s4_ptr;
-            uint16_t* const st0 = lds + wave * (2 * WTQ * PH);
-            const int       pw  = p0 + wp * WTP;
-            const int       qw  = q0 + wq * WTQ;
-            const bool      aff = a.cd_affine != 0;
-            const int       L   = lane & 15;
-            const int       G   = lane >> 4;
-            // this lane's row within a slab and first column, per store vector
-            int      prow[NVEC], qcol[NVEC];
-            uint32_t dqo[NVEC];
-            bool     qok[NVEC];
-#pragma unroll
-            for(int v = 0; v < NVEC; v++)
-            {
-                const int u = v * 4 + G; // (row quad, column block) unit of this 16-lane group
-                prow[v]     = 4 * (u / QB) + (L & 3);
-                qcol[v]     = 32 * (u % QB) + 8 * (L >> 2);
-                const int q = qw + qcol[v];
-                qok[v]      = q_in8(q);
-                dqo[v]      = !qok[v] ? 0u : aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
-            }
-            uint32_t doff[2][NVEC];
-            auto     offsets = [&](int i, uint32_t (&d)[NVEC]) {
-#pragma unroll
-                for(int v = 0; v < NVEC; v++)
-                {
-                    const int p = pw + i * 32 + prow[v];
-                    d[v] = !(qok[v] && p_in(p)) ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
-                }
-            };
-            auto write_slab = [&](int i, uint16_t* dst) {
-#pragma unroll
-                for(int j = 0; j < TQ; j++)
-#pragma unroll
-                    for(int g = 0; g < 4; g++)
-                    {
-                        u32x2_t w;
-                        w[0] = (uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g]) | ((uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 1]) << 16);
-                        w[1] = (uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 2]) | ((uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 3]) << 16);
-                        *(u32x2_t*)(dst + (j * 32 + (lane & 31)) * PH + 8 * g + 4 * (lane >> 5)) = w;
-                    }
-            };
-            offsets(0, doff[0]);
-            write_slab(0, st0);
-            wave_lds_fence();
-#pragma unroll
-            for(int i = 0; i < TP; i++)
-            {
-                const uint16_t* cur = st0 + (i & 1) * (WTQ * PH);
-                if(i + 1 < TP)
-                {
-                    offsets(i + 1, doff[(i + 1) & 1]);
-                    write_slab(i + 1, st0 + ((i + 1) & 1) * (WTQ * PH));
-                }
-                u32x4_t o[NVEC];
-#pragma unroll
-                for(int v = 0; v < NVEC; v++)
-                {
-                    // the word this lane supplies: column qcol-block + 8 * (L % 4) + L / 4, the group's 4 rows
-                    const int       u   = v * 4 + G;
-                    const uint16_t* src = cur + (32 * (u % QB) + 8 * (L & 3) + (L >> 2)) * PH + 4 * (u / QB);
-                    const short4_t  lo  = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(src));
-                    const short4_t  hi  = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s4_ptr)(src + 4 * PH));
-                    const u32x2_t   l2  = __builtin_bit_cast(u32x2_t, lo);
-                    const u32x2_t   h2  = __builtin_bit_cast(u32x2_t, hi);
-                    o[v]                = u32x4_t{l2[0], l2[1], h2[0], h2[1]};
-                }
-                // table-driven offsets are loads: await the next slab's before this slab's stores
-                // go out (loads and stores share one in-order counter)
-                if(!aff)
-                    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-#pragma unroll
-                for(int v = 0; v < NVEC; v++)
-                    if(qok[v] && p_in(pw + i * 32 + prow[v]))
-                        HIPTK_STORE_D((u32x4_t*)(Dp + doff[i & 1][v]), o[v]);
-                wave_lds_fence();
-            }
-#ifdef HIPTK_CLOCK_PROBE
-            probe_out();
-#endif
-            return;
-        }
-        if constexpr(sizeof(out_t) == 2)
-        if(a.cd_vec == 8)
-        {
-            // C and D are contiguous along q in runs of 8: route each 32-row slab of the
-            // wave's accumulators through LDS (the operand buffers are free now) so that a
-            // lane ends up with 8 consecutive q of one row and moves them as one 16-byte
-            // access; 16 lanes cover 256 contiguous bytes of a row.
-            constexpr int EP   = WTQ + 4; // floats per staged row
-            constexpr int VPR  = WTQ / 8; // 8-element vectors per staged row
-            constexpr int NVEC = (32 * WTQ / 8) / 64; // vectors per lane and slab
-            static_assert(32 * EP * 4 * WP * WQ <= 2 * STAGE * 2, "epilogue staging must fit the operand buffers");
-            const int pw = p0 + wp * WTP;
-            const int qw = q0 + wq * WTQ;
-            // One slab of C in flight, requested (after the look-ups behind its addresses) while the
-            // slab before it is staged.
-            auto one_in_flight = [&]() {
-            const bool bil = a.bilinear != 0;
-            const bool aff = a.cd_affine != 0;
-            // Offsets and C values of a slab are fetched while the slab before it is being
-            // written, so that table look-ups, C loads and D stores of different vectors are
-            // all in flight together instead of one dependent round trip per vector.  (The
-            // compiler cannot hoist them itself: D may alias C.)  A lane reads every C element
-            // before it writes the D element at the same place, so exact aliasing stays valid.
-            uint32_t dqo[NVEC], cqo[NVEC];
-            bool     qok[NVEC];
-#pragma unroll
-            for(int v = 0; v < NVEC; v++)
-            {
-                const int q = qw + ((v * 64 + lane) % VPR) * 8;
-                qok[v]      = q_in8(q);
-                // affine C / D (every benchmark-style packed layout): offsets are computed, so the
-                // epilogue starts without a round trip to the offset tables
-                dqo[v] = !qok[v] ? 0u : aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
-                cqo[v] = !(qok[v] && bil) ? 0u : aff ? (uint32_t)q * (uint32_t)a.cq_stride : (uint32_t)a.cq[q];
-            }
-            struct Slab
-            {
-                u32x4_t  c[NVEC];
-                uint32_t doff[NVEC];
-                bool     ok[NVEC];
-            };
-            Slab sl[2];
-            auto prefetch = [&](int i, Slab& s) {
-#pragma unroll
-                for(int v = 0; v < NVEC; v++)
-                {
-                    const int p = pw + i * 32 + (v * 64 + lane) / VPR;
-                    s.ok[v]     = qok[v] && p_in(p);
-                    s.doff[v]   = !s.ok[v] ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
-                    u32x4_t c4  = {0u, 0u, 0u, 0u};
-                    if(s.ok[v] && bil)
-                        c4 = *(const u32x4_t*)(Cp + ((aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p]) + cqo[v]));
-                    s.c[v] = c4;
-                }
-            };
-            // Two staging buffers per wave when the operand buffers have room for them: slab
-            // i+1 is written to LDS while slab i is read back, converted and stored.
-            constexpr bool DB = 2 * 32 * EP * 4 * WP * WQ <= 2 * STAGE * 2;
-            float* const   st0 = (float*)lds + wave * ((DB ? 2 : 1) * 32 * EP);
-            auto write_slab = [&](int i, float* dst) {
-#pragma unroll
-                for(int j = 0; j < TQ; j++)
-#pragma unroll
-                    for(int r = 0; r < 16; r++)
-                        dst[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
-            };
-            prefetch(0, sl[0]);
-            if constexpr(DB)
-            {
-                write_slab(0, st0);
-                wave_lds_fence();
-            }
-#pragma unroll
-            for(int i = 0; i < TP; i++)
-            {
-                const float* cur_st = st0 + (DB ? (i & 1) * 32 * EP : 0);
-                if constexpr(DB)
-                {
-                    if(i + 1 < TP)
-                    {
-                        prefetch(i + 1, sl[(i + 1) & 1]);
-                        write_slab(i + 1, st0 + ((i + 1) & 1) * 32 * EP);
-                    }
-                }
-                else
-                {
-                    write_slab(i, st0);
-                    if(i + 1 < TP)
-                        prefetch(i + 1, sl[(i + 1) & 1]);
-                    wave_lds_fence();
-                }
-                const Slab& cur = sl[i & 1];
-                // all of the slab's vectors are read from LDS before any is converted and stored
-                f32x4_t lo[NVEC], hi[NVEC];
-#pragma unroll
-                for(int v = 0; v < NVEC; v++)
-                {
-                    const int    slot = v * 64 + lane;
-                    const float* src  = cur_st + (slot / VPR) * EP + (slot % VPR) * 8;
-                    lo[v]             = *(const f32x4_t*)src;
-                    hi[v]             = *(const f32x4_t*)(src + 4);
-                }
-                u32x4_t o[NVEC];
-#pragma unroll
-                for(int v = 0; v < NVEC; v++)
-                {
-                    float v8[8] = {lo[v][0], lo[v][1], lo[v][2], lo[v][3], hi[v][0], hi[v][1], hi[v][2], hi[v][3]};
-                    if(bil)
-                    {
-                        const u32x4_t c4 = cur.c[v];
-#pragma unroll
-                        for(int e = 0; e < 8; e++)
-                        {
-                            const uint16_t cb = (uint16_t)(c4[e >> 1] >> ((e & 1) * 16));
-                            v8[e]             = alpha * v8[e] + beta * Tr::to_f32(cb);
-                        }
-                    }
-                    else
-                    {
-#pragma unroll
-                        for(int e = 0; e < 8; e++)
-                            v8[e] = alpha * v8[e];
-                    }
-#pragma unroll
-                    for(int e = 0; e < 4; e++)
-                        o[v][e] = (uint32_t)Tr::from_f32(v8[2 * e]) | ((uint32_t)Tr::from_f32(v8[2 * e + 1]) << 16);
-                }
-                // Loads and stores share one in-order counter, so waiting for a load also waits
-                // for every store issued before it.  The next slab's prefetch is therefore
-                // awaited here, before this slab's stores are issued: the only stores it can
-                // wait for are the previous slab's, a whole slab old, and this slab's stores
-                // then drain while the next slab is converted.
-                // (With computed offsets and no C there are no loads, and nothing to wait for.)
-                if(bil || !aff)
-                    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-#pragma unroll
-                for(int v = 0; v < NVEC; v++)
-                    if(cur.ok[v])
-                        HIPTK_STORE_D((u32x4_t*)(Dp + cur.doff[v]), o[v]);
-                wave_lds_fence();
-            }
-            };
-            // Two slabs in flight.  One copy of the code per case (C read or not; offsets computed):
-            // where the choice is made at run time inside the loop, the compiler has to wait for
-            // every outstanding load wherever the paths join, and the overlap below is lost.
-            auto run = [&](auto aff_c, auto bil_c) {
-            constexpr bool aff = decltype(aff_c)::value;
-            constexpr bool bil = decltype(bil_c)::value;
-            // The C vectors of a slab are requested two slabs ahead of their use, and the table
-            // look-ups behind their addresses one slab before that.  (The compiler cannot move any
-            // of this itself: D may alias C and, for all it knows, the offset tables.)  Loads and
-            // stores complete in issue order, so a wait for a load also waits for every store issued
-            // before it: with this lead the youngest stores such a wait can catch are a slab old,
-            // and C loads, LDS staging and D stores of neighbouring slabs overlap.  A lane reads
-            // each C element before it writes the D element at the same place, and no lane reads an
-            // element another lane writes, so exact aliasing stays valid.
-            uint32_t dqo[NVEC], cqo[NVEC];
-            bool     qok[NVEC];
-#pragma unroll
-            for(int v = 0; v < NVEC; v++)
-            {
-                const int q = qw + ((v * 64 + lane) % VPR) * 8;
-                qok[v]      = q_in8(q);
-                // affine C / D (every benchmark-style packed layout): offsets are computed; else
-                // looked up (the tables are padded beyond every index a tile reaches, with the
-                // offset of index 0, so the look-ups need no guard)
-                dqo[v] = aff ? (uint32_t)q * (uint32_t)a.dq_stride : (uint32_t)a.dq[q];
-                cqo[v] = !bil ? 0u : aff ? (uint32_t)q * (uint32_t)a.cq_stride : (uint32_t)a.cq[q];
-            }
-            struct Offsets
-            {
-                uint32_t d[NVEC], c[NVEC];
-                bool     ok[NVEC];
-            };
-            auto prepare = [&](int i, Offsets& o) {
-#pragma unroll
-                for(int v = 0; v < NVEC; v++)
-                {
-                    const int p        = pw + i * 32 + (v * 64 + lane) / VPR;
-                    o.ok[v]            = qok[v] && p_in(p);
-                    const uint32_t dpo = aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p];
-                    const uint32_t cpo = !bil ? 0u : aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p];
-                    // a vector outside the extents reads element 0 of C, a valid address, and is not stored
-                    o.d[v] = o.ok[v] ? dpo + dqo[v] : 0u;
-                    o.c[v] = o.ok[v] ? cpo + cqo[v] : 0u;
-                }
-            };
-            // two slabs in flight, and the offsets of the slab that is requested next
-            constexpr int NB = 2;
-            Offsets       off[NB], nxt;
-            u32x4_t       cbuf[NB][NVEC];
-            auto          request = [&](int b) {
-                if(bil)
-                {
-#pragma unroll
-                    for(int v = 0; v < NVEC; v++)
-                        cbuf[b][v] = *(const u32x4_t*)(Cp + off[b].c[v]);
-                }
-            };
-            // Two staging buffers per wave when the operand buffers have room for them: slab
-            // i+1 is written to LDS while slab i is read back, converted and stored.
-            constexpr bool DB = 2 * 32 * EP * 4 * WP * WQ <= 2 * STAGE * 2;
-            float* const   st0 = (float*)lds + wave * ((DB ? 2 : 1) * 32 * EP);
-            auto write_slab = [&](int i, float* dst) {
-#pragma unroll
-                for(int j = 0; j < TQ; j++)
-#pragma unroll
-                    for(int r = 0; r < 16; r++)
-                        dst[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
-            };
-            // (all look-ups of the first two slabs before their first C load: one wait, not two)
-            prepare(0, off[0]);
-            if constexpr(TP > 1)
-                prepare(1, off[1]);
-            request(0);
-            if constexpr(TP > 1)
-                request(1);
-            if constexpr(TP > NB)
-                prepare(NB, nxt);
-            if constexpr(DB)
-            {
-                write_slab(0, st0);
-                wave_lds_fence();
-            }
-#pragma unroll
-            for(int i = 0; i < TP; i++)
-            {
-                const float* cur_st = st0 + (DB ? (i & 1) * 32 * EP : 0);
-                if constexpr(DB)
-                {
-                    if(i + 1 < TP)
-                        write_slab(i + 1, st0 + ((i + 1) & 1) * 32 * EP);
-                }
-                else
-                {
-                    write_slab(i, st0);
-                    wave_lds_fence();
-                }
-                // up to four of the slab's vectors are read from LDS together, then converted and stored
-                constexpr int HV = NVEC > 4 ? 4 : NVEC;
-#pragma unroll
-                for(int h = 0; h < NVEC; h += HV)
-                {
-                    f32x4_t lo[HV], hi[HV];
-#pragma unroll
-                    for(int w = 0; w < HV; w++)
-                    {
-                        const int    slot = (h + w) * 64 + lane;
-                        const float* src  = cur_st + (slot / VPR) * EP + (slot % VPR) * 8;
-                        lo[w]             = *(const f32x4_t*)src;
-                        hi[w]             = *(const f32x4_t*)(src + 4);
-                    }
-                    u32x4_t o[HV];
-#pragma unroll
-                    for(int w = 0; w < HV; w++)
-                    {
-                        float v8[8] = {lo[w][0], lo[w][1], lo[w][2], lo[w][3], hi[w][0], hi[w][1], hi[w][2], hi[w][3]};
-                        if(bil)
-                        {
-                            const u32x4_t c4 = cbuf[i % NB][h + w];
-#pragma unroll
-                            for(int e = 0; e < 8; e++)
-                            {
-                                const uint16_t cb = (uint16_t)(c4[e >> 1] >> ((e & 1) * 16));
-                                v8[e]             = alpha * v8[e] + beta * Tr::to_f32(cb);
-                            }
-                        }
-                        else
-                        {
-#pragma unroll
-                            for(int e = 0; e < 8; e++)
-                                v8[e] = alpha * v8[e];
-                        }
-#pragma unroll
-                        for(int e = 0; e < 4; e++)
-                            o[w][e] = (uint32_t)Tr::from_f32(v8[2 * e]) | ((uint32_t)Tr::from_f32(v8[2 * e + 1]) << 16);
-                    }
-#pragma unroll
-                    for(int w = 0; w < HV; w++)
-                        if(off[i % NB].ok[h + w])
-                            HIPTK_STORE_D((u32x4_t*)(Dp + off[i % NB].d[h + w]), o[w]);
-                }
-                // this slab's registers are free: request the slab NB ahead, then look up the
-                // offsets of the one after that
-                if(i + NB < TP)
-                {
-                    off[i % NB] = nxt;
-                    request(i % NB);
-                }
-                if(i + NB + 1 < TP)
-                    prepare(i + NB + 1, nxt);
-                wave_lds_fence();
-            }
-            };
-            typedef std::integral_constant<bool, true>  Yes;
-            typedef std::integral_constant<bool, false> No;
-            // The 128-wide wave tiles of the four-wave kernels hold 8 vectors per lane and slab and
-            // have no registers to spare for a second slab.  With offsets from the tables the
-            // deeper lead did not pay either (rank-6 benchmark layout: 366-372 us against 374).
-            if constexpr(NVEC * TP > 16)
-                one_in_flight();
-            else
-            {
-                if(a.cd_affine == 0)
-                    one_in_flight();
-                else if(a.bilinear != 0)
-                    run(Yes{}, Yes{});
-                else
-                    run(Yes{}, No{});
-            }
-#ifdef HIPTK_CLOCK_PROBE
-            probe_out();
-#endif
-            return;
-        }
-        {
-            // Element by element through the offset tables.  D may alias C (and, for all the
-            // compiler knows, the tables), so it would fetch one offset, one C element and store
-            // one D element at a time; the offsets of a slab's 16 rows are therefore fetched once,
-            // ahead of the columns, and the 16 C elements of a column before the first store.
-            const int pw = p0 + wp * WTP + 4 * (lane >> 5);
-            const int qw = q0 + wq * WTQ + (lane & 31);
-            const bool bil = a.bilinear != 0;
-            uint32_t   dqo[TQ], cqo[TQ];
-            bool       qok[TQ];
-#pragma unroll
-            for(int j = 0; j < TQ; j++)
-            {
-                const int q = qw + j * 32;
-                qok[j]      = q_in(q);
-                // (the tables are padded beyond every index a tile can reach, with the offset of
-                // index 0: loads need no guard, only the stores do)
-                dqo[j] = (uint32_t)a.dq[q];
-                cqo[j] = bil ? (uint32_t)a.cq[q] : 0u;
-            }
-#pragma unroll
-            for(int i = 0; i < TP; i++)
-            {
-                uint32_t dpo[16], cpo[16];
-                bool     pok[16];
-#pragma unroll
-                for(int r = 0; r < 16; r++)
-                {
-                    const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
-                    pok[r]      = p_in(p);
-                    dpo[r]      = (uint32_t)a.dp[p];
-                    cpo[r]      = bil ? (uint32_t)a.cp[p] : 0u;
-                }
-#pragma unroll
-                for(int j = 0; j < TQ; j++)
-                {
-                    if(!qok[j])
-                        continue;
-                    float c[16];
-#pragma unroll
-                    for(int r = 0; r < 16; r++)
-                        c[r] = 0.f;
-                    if(bil)
-                    {
-#pragma unroll
-                        for(int r = 0; r < 16; r++)
-                            c[r] = Tr::out_to_f32(Cp[cpo[r] + cqo[j]]);
-                    }
-#pragma unroll
-                    for(int r = 0; r < 16; r++)
-                        if(pok[r])
-                            Dp[dpo[r] + dqo[j]] = Tr::out_from_f32(Tr::axpby(alpha, acc[i][j][r], beta, c[r], bil));
-                }
-            }
-        }
+        epilogue_h<Tr, WP, WQ, TP, TQ, 2 * STAGE * 2>(a, acc, lds, p0, q0, p_own, q_own);
     }
 
     template <typename Tr,

@@ -17,7 +17,9 @@ namespace hiptk
             Registry()
             {
                 typedef const KernelEntry* (*src_fn)(int*);
-                const src_fn sources[] = {entries_f16_aff,
+                const src_fn sources[] = {entries_f16_hd,
+                                          entries_bf16_hd,
+                                          entries_f16_aff,
                                           entries_bf16_aff,
                                           entries_f16_vec,
                                           entries_f16_gen,
@@ -166,6 +168,9 @@ namespace hiptk
                 {
                     // a tile can only be moved back to end at P / Q if it fits into P / Q
                     if((p->shift_p && p->P < e.bp) || (p->shift_q && p->Q < e.bq))
+                        continue;
+                    // kernels without a K tail
+                    if(e.k_multiple > 0 && p->K % e.k_multiple != 0)
                         continue;
                     if(e.k_affine && p->k_affine)
                         return &e;

@@ -68,6 +68,21 @@ def layouts(dtype, compute, big):
                                     name=f"tiles_ragged_{tag}_kfast_{dtype}"))
         out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], rk, a, None,
                                     name=f"tiles_ragged_{tag}_mixed_{dtype}"))
+    if big:
+        # K a multiple of 32 with one stride per operand: the kernels that load their operand tiles
+        # straight into LDS have no K tail and take only these; 1, 4, 5 and 11 K tiles, row-fast,
+        # k-fast and mixed operands, whole and partial 256 x 256 output tiles
+        for kk in ((32, 1), (32, 4), (32, 5), (32, 11)):
+            dk = {0: 40, 1: 9, 10: 24, 11: 13, 20: kk[0], 21: kk[1]}
+            tag = f"k{kk[0] * kk[1]}"
+            out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, b,
+                                        name=f"tiles_{tag}_rowfast_{dtype}"))
+            out.append(wl.make_workload(dtype, compute, [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], dk, a, None,
+                                        name=f"tiles_{tag}_kfast_{dtype}"))
+            out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], dk, a, b,
+                                        name=f"tiles_{tag}_mixed_{dtype}"))
+            out.append(wl.make_workload(dtype, compute, [20, 21, 0, 1], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, None,
+                                        name=f"tiles_{tag}_mixed2_{dtype}"))
     # odd extents with the modes interleaved, so that no index is one contiguous run: scalar
     # gathers on every operand
     odd = {0: 7, 1: 23, 10: 5, 11: 29, 20: 3, 21: 37 if big else 21}
