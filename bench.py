@@ -12,7 +12,9 @@ f16 scale contraction at M = N = K = 4096 (extents 64^6, packed column-major).  
 prints ONE JSON line: metric / value (TFLOP/s of the headline workload), a `roofline` object
 for its kernel (average launch duration measured with HIP events on the launch stream), a
 `cpu_baseline` object (the reference's own CPU contraction, or the oracle port, timed on a
-bounded slab of the same workload on this host), a short `permutation` object (GB/s of one
+bounded slab of the same workload on this host), a `target` object (the same problem as a
+bilinear contraction in f16 and in bf16: kernel time, TFLOP/s, fraction of the nominal peak and
+of the MFMA-only sustained rate), a short `permutation` object (GB/s of one
 hiptensorPermutation workload; --permutation gives that operation its own full line) and, with
 --all, the other configurations.
 """
@@ -30,15 +32,37 @@ PEAK_TFLOPS = {"f16": 2516.6, "bf16": 2516.6, "f32": 157.3, "c32": 157.3, "f64":
 FLOP_PER_CLK_CU = {"f16": 4096, "bf16": 4096, "f32": 256, "c32": 256, "f64": 128, "c64": 128}
 HBM_PEAK_GBS = 8000.0
 
-# Bytes per launch crossing the L2 <-> memory boundary, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of this script (profiles/contract_h_kernel_f16_4096cubed_scale.md gives the commands, the
-# raw readings and the copy-kernel scale factors).  Keyed by (workload, kernel); null otherwise.
-MEASURED_TRAFFIC_BYTES = {
-    ("cfg2_f16_scale_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue"): (2.0 * 98533.9 + 1.0 * 32768.0) * 1024,
-    ("cfg2_f16_scale_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue_pipe2x2"): (2.0 * 98563.0 + 1.0 * 32768.0) * 1024,
+# Bytes per launch crossing the L2 <-> memory boundary: constants taken from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs of this script (the files under profiles/ give the commands, the raw
+# readings per dispatch and the copy-kernel scale factors: FETCH_SIZE x 2.0, WRITE_SIZE x 1.0, KiB).
+# They are properties of (workload, kernel) and are not re-measured by a run of this script: a kernel
+# that has no profile reports null.
+MEASURED_TRAFFIC_KIB = {
     # profiles/permute_kernels_1GiB_tensors.md
-    ("perm_f32_512x64x128x64_2031", "permute_tiled_f32_128x128_r4_w4"): (2.0 * 524329.9 + 1.0 * 1049097.7) * 1024,
+    ("perm_f32_512x64x128x64_2031", "permute_tiled_f32_128x128_r4_w4"): (524329.9, 1049097.7),
 }
+
+
+def measured_traffic(workload, kernel):
+    kib = MEASURED_TRAFFIC_KIB.get((workload, kernel))
+    return None if kib is None else (2.0 * kib[0] + 1.0 * kib[1]) * 1024
+
+
+_CALIB = None
+
+
+def mfma_ceiling(dtype, random_operands):
+    """TFLOP/s of a loop of nothing but this type's MFMA instruction (bench-only calibration library)."""
+    import ctypes
+
+    global _CALIB
+    if _CALIB is None:
+        _CALIB = ctypes.CDLL(os.path.join(ROOT, "hiptensor_amd", "lib", "libhiptk_calib.so"))
+        _CALIB.hiptk_mfma_ceiling.restype = ctypes.c_int
+        _CALIB.hiptk_mfma_ceiling.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)]
+    kcls = {"f16": 0, "bf16": 1, "f32": 2, "f64": 3, "c32": 4, "c64": 5}
+    tf = ctypes.c_double(0)
+    return tf.value if _CALIB.hiptk_mfma_ceiling(kcls[dtype], 1 if random_operands else 0, ctypes.byref(tf)) == 0 else None
 
 
 def measure(handle, w, steps, warmup, settle_s=0.25):
@@ -167,7 +191,7 @@ def permutation_line(a, handle, prop):
         "config": {"workload": w["name"], "lengths": w["lensA"], "permuted_dims": w["perm"], "alpha": w["alpha"],
                    "kernel": r["info"]["kernel_name"]},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((w["name"], r["info"]["kernel_name"])),
+                     "traffic": measured_traffic(w["name"], r["info"]["kernel_name"]),
                      "kernel_ms": r["kernel_ms"], "algorithmic_bytes": nbytes},
         "device": {"name": prop.name, "cus": prop.multi_processor_count},
     }
@@ -252,6 +276,7 @@ def main():
                          "interleaved_f32: operands with interleaved modes, contracted from packed copies")
     ap.add_argument("--all", action="store_true", help="also time every other configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-target", action="store_true", help="skip the bilinear f16 / bf16 rows of the default line")
     ap.add_argument("--permutation", action="store_true",
                     help="time hiptensorPermutation instead (workload: a name of workloads.permutation_configs(), "
                          "default perm_f32_rank4); the JSON line then carries GB/s against the HBM roofline")
@@ -301,25 +326,40 @@ def main():
                    "kernel": r["info"]["kernel_name"], "split_k": r["info"]["split_k"],
                    "packed_copy_kernels": [k for k in (r["info"]["pack_a_kernel"], r["info"]["pack_b_kernel"]) if k]},
         "roofline": {"bound": "mfma", "achieved": tflops, "peak": peak, "unit": "TFLOP/s", "frac": tflops / peak,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((w["name"], r["info"]["kernel_name"])),
+                     "traffic": measured_traffic(w["name"], r["info"]["kernel_name"]),
+                     "traffic_source": "profile constant (rocprofv3 FETCH_SIZE / WRITE_SIZE of this workload and kernel), null if not profiled",
                      "kernel_ms": r["kernel_ms"],
                      "peak_from_device_clock": cus * clock_ghz * FLOP_PER_CLK_CU[w["dtype"]] / 1e3,
                      "hbm_GBs_algorithmic": wl.algorithmic_bytes(w) / (r["kernel_ms"] * 1e-3) / 1e9},
         "device": {"name": prop.name, "cus": cus, "clock_ghz": clock_ghz},
     }
     # what a loop of nothing but this type's MFMA instruction sustains on this device
-    import ctypes
-
-    from hiptensor_amd._lib import lib as _native
-    kcls = {"f16": 0, "bf16": 1, "f32": 2, "f64": 3, "c32": 4, "c64": 5}
     ceil = {}
     for label, rnd in (("constant_operands", 0), ("random_operands", 1)):
-        tf = ctypes.c_double(0)
-        if _native.hiptk_mfma_ceiling(kcls[w["dtype"]], rnd, ctypes.byref(tf)) == 0:
-            ceil[label] = tf.value
+        tf = mfma_ceiling(w["dtype"], rnd)
+        if tf:
+            ceil[label] = tf
     out["roofline"]["mfma_only_sustained_tflops"] = ceil
     if ceil.get("random_operands"):
         out["roofline"]["frac_of_sustained"] = tflops / ceil["random_operands"]
+    out["parity"] = {"oracle": "CPU restatement of the reference's contraction, pinned bit-for-bit to the reference's compiled CPU path",
+                     "tolerance": {"f16": 1e-2, "bf16": 1e-2, "f32": 1e-5, "c32": 1e-5, "f64": 1e-12, "c64": 1e-12}[w["dtype"]],
+                     "tolerance_metric": "max|d - r| / max|r| over the checked outputs (tests/cases.py); the reference "
+                                         "harness's element-wise |d - r| / (|d| + |r| + 1) is held to its own bound 2 K eps beside it"}
+    # The same 4096^3 problem as a bilinear contraction (beta = 1, C read), f16 and bf16: the
+    # operation and types the throughput target is stated on.
+    if a.workload == "cfg2_f16_scale" and not a.no_target:
+        target = {}
+        for tname in ("cfg2_f16_bilinear", "cfg2_bf16_bilinear"):
+            tw = cfgs[tname]
+            tr = measure(handle, tw, a.steps, a.warmup, a.settle)
+            ttf = wl.flops(tw) / (tr["kernel_ms"] * 1e-3) / 1e12
+            sustained = mfma_ceiling(tw["dtype"], 1)
+            target[tname] = {"kernel_ms": tr["kernel_ms"], "tflops": ttf, "frac": ttf / PEAK_TFLOPS[tw["dtype"]],
+                             "mfma_only_sustained_tflops": sustained,
+                             "frac_of_sustained": ttf / sustained if sustained else None,
+                             "kernel": tr["info"]["kernel_name"], "op": "bilinear", "dtype": tw["dtype"]}
+        out["target"] = target
     if a.all:
         others = {}
         for name, cw in cfgs.items():
@@ -328,8 +368,7 @@ def main():
             steps = max(5, a.steps // 2)
             rr = measure(handle, cw, steps, a.warmup, a.settle)
             tf = wl.flops(cw) / (rr["kernel_ms"] * 1e-3) / 1e12
-            tfc = ctypes.c_double(0)
-            sustained = tfc.value if _native.hiptk_mfma_ceiling(kcls[cw["dtype"]], 1, ctypes.byref(tfc)) == 0 else None
+            sustained = mfma_ceiling(cw["dtype"], 1)
             others[name] = {"kernel_ms": rr["kernel_ms"], "tflops": tf, "frac_peak": tf / PEAK_TFLOPS[cw["dtype"]],
                             "mfma_only_sustained_tflops": sustained,
                             "hbm_GBs_algorithmic": wl.algorithmic_bytes(cw) / (rr["kernel_ms"] * 1e-3) / 1e9,

@@ -1,4 +1,5 @@
-// Device calibration: the rate a loop of nothing but MFMA instructions sustains on every CU,
+// Bench-only calibration library (libhiptk_calib.so, not part of the product library):
+// the rate a loop of nothing but MFMA instructions sustains on every CU,
 // with constant operands and with pseudo-random operands in [-1, 1).  Under a full MFMA load
 // the clock this part holds depends on how much the operand bits toggle, so this is the
 // practical ceiling the contraction kernels are measured against (next to the nominal peak).
@@ -8,6 +9,7 @@
 #include <algorithm>
 #include <chrono>
 
+#include "hiptk_calib.h"
 #include "hiptk_kernels.h"
 
 namespace
@@ -129,43 +131,6 @@ namespace
         if(sum == 1.2345)
             sink[threadIdx.x] = (float)sum;
     }
-}
-
-namespace
-{
-    // Pseudo-random finite values of magnitude [0.5, 1) with random signs, written as 32-bit
-    // words laid out for the class's element type.
-    __global__ void __launch_bounds__(256) fill_pattern(uint32_t* out, size_t words, int cls)
-    {
-        const size_t stride = (size_t)gridDim.x * 256;
-        for(size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < words; i += stride)
-        {
-            const uint32_t r = hash32((uint32_t)i * 2654435761u + (uint32_t)(i >> 32));
-            uint32_t       w;
-            switch(cls)
-            {
-            case HIPTK_F16: w = 0x38003800u | (r & 0x83FF83FFu); break;
-            case HIPTK_BF16: w = 0x3F003F00u | (r & 0x807F807Fu); break;
-            case HIPTK_F64:
-            case HIPTK_C64:
-            case HIPTK_F64_AS_F32: w = (i & 1) ? (0x3FE00000u | (r & 0x800FFFFFu)) : r; break;
-            default: w = 0x3F000000u | (r & 0x807FFFFFu); break;
-            }
-            out[i] = w;
-        }
-    }
-}
-
-extern "C" int hiptk_fill_pattern(void* dst, uint64_t bytes, int cls, void* stream)
-{
-    if(!dst || (bytes & 3))
-        return HIPTK_ERR_ARG;
-    const size_t words = (size_t)(bytes / 4);
-    if(words == 0)
-        return HIPTK_OK;
-    const unsigned blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
-    hipLaunchKernelGGL(fill_pattern, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (uint32_t*)dst, words, cls);
-    return hipGetLastError() == hipSuccess ? HIPTK_OK : HIPTK_ERR_LAUNCH;
 }
 
 extern "C" int hiptk_mfma_ceiling(int cls, int random_operands, double* tflops)

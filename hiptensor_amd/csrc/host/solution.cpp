@@ -162,7 +162,18 @@ namespace hipta
         const double per_cu  = std::ceil(wgs / dev.cus); // workgroups the busiest CU runs
         const double sharing = std::min<double>(resident, per_cu);
         TileRate     r       = tile_rate(v.cls, s.bp * s.bq);
-        if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152)
+        if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152 && s.bk == 32)
+        {
+            // the 256 x 256 tile whose operand tiles are loaded straight into LDS (four waves, K in
+            // steps of 32).  4096^3, both operands contiguous along their row index: 117.2 us against
+            // 126.0 on eight waves (f16 scale), 115.5 against 125.9 (f16 bilinear), 108.5 against 118.4
+            // (bf16 bilinear); both contiguous along k (64-byte runs per row and K step): 125.8 against
+            // 120.3
+            const double f = kper / s.bk < 16 ? 0.9 : (v.x_kfast || v.y_kfast) ? 0.95 : 1.08;
+            r.alone *= f;
+            r.full *= f;
+        }
+        else if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152)
         {
             // the four-wave form of the 256 x 256 tile (one wave per SIMD): level with the
             // eight-wave form over a long K without C, behind it in the epilogue that reads C

@@ -125,15 +125,6 @@ int hiptk_contract(const hiptk_problem_t* prob,
                    void*                  stream,
                    int*                   hip_error);
 
-/* Calibration, no counterpart in the reference: the TFLOP/s a loop of nothing but the class's
- * MFMA instruction sustains on the current device (one 4-wave workgroup per CU), with
- * constant operands (random_operands = 0) or pseudo-random operands in [-1, 1) (1).  The
- * clock the part holds under a full matrix-core load depends on the operand data, so the
- * second figure is the practical ceiling for a contraction of random data.  Synchronous:
- * loads the device for about 150 ms first so that its clock has settled, then times 20
- * launches; allocates 4 KiB. */
-int hiptk_mfma_ceiling(int cls, int random_operands, double* tflops);
-
 /* Fills `bytes` (a multiple of 4) of device memory with pseudo-random finite elements of the
  * class's storage type, magnitudes in [0.5, 1) and random signs, on `stream`.  No counterpart
  * in the reference: the measured kernel selection times its candidates on such data, since
