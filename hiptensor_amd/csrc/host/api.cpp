@@ -304,6 +304,11 @@ hiptensorStatus_t hiptensorCreate(hiptensorHandle_t** handle)
     if(arch.compare(0, 6, "gfx950") != 0)
         return fail(HIPTENSOR_STATUS_ARCH_MISMATCH, "this library runs on gfx950 only");
     Handle::create((*handle)->fields, dev, arch, prop.multiProcessorCount, prop.clockRate * 1e-6);
+    // look up, once per device, the address of the workspace the library itself holds (used by
+    // hiptensorAmdContractionNoAlloc); a failure here is reported when that entry point is called
+    void*    ws       = nullptr;
+    uint64_t ws_bytes = 0;
+    (void)hiptk_static_workspace(&ws, &ws_bytes, nullptr);
     return HIPTENSOR_STATUS_SUCCESS;
 }
 
@@ -822,6 +827,26 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
     return HIPTENSOR_STATUS_SUCCESS;
 }
 
+namespace
+{
+    // hiptensorContraction, and its variant that takes the workspace from the library's own device
+    // array instead of the caller (static_ws: `workspace` / `workspaceSize` are ignored, nothing is
+    // allocated and no event is created, so PERF_TRACE timing is left out).
+    hiptensorStatus_t contractionImpl(const char*                       fn,
+                                      bool                              static_ws,
+                                      const hiptensorHandle_t*          handle,
+                                      const hiptensorContractionPlan_t* plan,
+                                      const void*                       alpha,
+                                      const void*                       A,
+                                      const void*                       B,
+                                      const void*                       beta,
+                                      const void*                       C,
+                                      void*                             D,
+                                      void*                             workspace,
+                                      uint64_t                          workspaceSize,
+                                      hipStream_t                       stream);
+}
+
 hiptensorStatus_t hiptensorContraction(const hiptensorHandle_t*          handle,
                                        const hiptensorContractionPlan_t* plan,
                                        const void*                       alpha,
@@ -834,8 +859,42 @@ hiptensorStatus_t hiptensorContraction(const hiptensorHandle_t*          handle,
                                        uint64_t                          workspaceSize,
                                        hipStream_t                       stream)
 {
+    return contractionImpl("hiptensorContraction", false, handle, plan, alpha, A, B, beta, C, D, workspace, workspaceSize, stream);
+}
+
+namespace hipta
+{
+    hiptensorStatus_t contractionNoAlloc(const hiptensorHandle_t*          handle,
+                                         const hiptensorContractionPlan_t* plan,
+                                         const void*                       alpha,
+                                         const void*                       A,
+                                         const void*                       B,
+                                         const void*                       beta,
+                                         const void*                       C,
+                                         void*                             D,
+                                         hipStream_t                       stream)
+    {
+        return contractionImpl("hiptensorAmdContractionNoAlloc", true, handle, plan, alpha, A, B, beta, C, D, nullptr, 0, stream);
+    }
+}
+
+namespace
+{
+hiptensorStatus_t contractionImpl(const char*                       fn,
+                                  bool                              static_ws,
+                                  const hiptensorHandle_t*          handle,
+                                  const hiptensorContractionPlan_t* plan,
+                                  const void*                       alpha,
+                                  const void*                       A,
+                                  const void*                       B,
+                                  const void*                       beta,
+                                  const void*                       C,
+                                  void*                             D,
+                                  void*                             workspace,
+                                  uint64_t                          workspaceSize,
+                                  hipStream_t                       stream)
+{
     Logger&     log = Logger::get();
-    const char* fn  = "hiptensorContraction";
     if(log.mask() & HIPTENSOR_LOG_LEVEL_API_TRACE)
     {
         char   am[64] = "alpha=NULL", bm[64] = "beta=NULL";
@@ -903,6 +962,32 @@ hiptensorStatus_t hiptensorContraction(const hiptensorHandle_t*          handle,
         log.errorf(fn, "Input Parameter Error : beta/C = nullptr (%s)", hiptensorGetErrorString(HIPTENSOR_STATUS_INVALID_VALUE));
         return HIPTENSOR_STATUS_INVALID_VALUE;
     }
+    if(static_ws)
+    {
+        // the workspace is the library's own device array: a fixed size, shared by every call on
+        // this device
+        workspace     = nullptr;
+        workspaceSize = 0;
+        if(st->ws_bytes > 0)
+        {
+            int hipErr = 0;
+            if(hiptk_static_workspace(&workspace, &workspaceSize, &hipErr) != HIPTK_OK)
+            {
+                log.errorf(fn, "The library's workspace is not available on this device: hip error %d (%s)", hipErr, hiptensorGetErrorString(HIPTENSOR_STATUS_HIP_ERROR));
+                return HIPTENSOR_STATUS_HIP_ERROR;
+            }
+            if(st->ws_bytes > workspaceSize)
+            {
+                log.errorf(fn,
+                           "This plan needs %lu bytes of workspace; the library's own holds %lu: plan with a smaller workspaceSize, "
+                           "or call hiptensorContraction with a workspace of the caller's (%s)",
+                           (unsigned long)st->ws_bytes,
+                           (unsigned long)workspaceSize,
+                           hiptensorGetErrorString(HIPTENSOR_STATUS_INSUFFICIENT_WORKSPACE));
+                return HIPTENSOR_STATUS_INSUFFICIENT_WORKSPACE;
+            }
+        }
+    }
     if(st->ws_bytes > 0 && (!workspace || workspaceSize < st->ws_bytes))
     {
         log.errorf(fn,
@@ -921,7 +1006,7 @@ hiptensorStatus_t hiptensorContraction(const hiptensorHandle_t*          handle,
     packScalar(st->prob.cls, av, ab);
     packScalar(st->prob.cls, bv, bb);
 
-    const bool timed = (log.mask() & HIPTENSOR_LOG_LEVEL_PERF_TRACE) != 0;
+    const bool timed = !static_ws && (log.mask() & HIPTENSOR_LOG_LEVEL_PERF_TRACE) != 0;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if(timed)
     {
@@ -1015,6 +1100,7 @@ hiptensorStatus_t hiptensorContraction(const hiptensorHandle_t*          handle,
         return HIPTENSOR_STATUS_INTERNAL_ERROR;
     }
 }
+} // namespace
 
 // ---- logger control (reference: library/src/hiptensor.cpp:323-458) ----
 

@@ -11,6 +11,15 @@ namespace hipta
 {
     hiptensorStatus_t createHostOnlyHandle(hiptensorHandle_t** handle);
     const PlanState*  planState(const hiptensorContractionPlan_t* plan);
+    hiptensorStatus_t contractionNoAlloc(const hiptensorHandle_t*          handle,
+                                         const hiptensorContractionPlan_t* plan,
+                                         const void*                       alpha,
+                                         const void*                       A,
+                                         const void*                       B,
+                                         const void*                       beta,
+                                         const void*                       C,
+                                         void*                             D,
+                                         hipStream_t                       stream);
     hiptensorStatus_t planPermutation(const hiptensorTensorDescriptor_t* descA,
                                       const int32_t                      modeA[],
                                       const hiptensorTensorDescriptor_t* descB,
@@ -208,6 +217,27 @@ extern "C" int hiptensorAmdContraction(const void* handle,
                                      workspace,
                                      workspaceSize,
                                      (hipStream_t)stream);
+}
+
+extern "C" int hiptensorAmdContractionNoAlloc(const void* handle,
+                                              const void* plan,
+                                              const void* alpha,
+                                              const void* A,
+                                              const void* B,
+                                              const void* beta,
+                                              const void* C,
+                                              void*       D,
+                                              void*       stream)
+{
+    return (int)hipta::contractionNoAlloc((const hiptensorHandle_t*)handle,
+                                          (const hiptensorContractionPlan_t*)plan,
+                                          alpha,
+                                          A,
+                                          B,
+                                          beta,
+                                          C,
+                                          D,
+                                          (hipStream_t)stream);
 }
 
 extern "C" int hiptensorAmdPermutation(const void*    handle,

@@ -2,6 +2,7 @@
 // split-K reduction kernels.
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "contract_h.hpp"
@@ -358,5 +359,54 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
             *hip_error = rc;
         return HIPTK_ERR_LAUNCH;
     }
+    return HIPTK_OK;
+}
+
+// ---- a workspace that lives in the library, for callers that cannot allocate ----
+//
+// Device memory of a fixed, modest size that every device the library runs on holds until the
+// process ends.  In host code the array's name is only a stand-in (passing it to a kernel would
+// hand the kernel a host-side address); its device address is looked up once per device with
+// hipGetSymbolAddress, with that device current, and from then on only that address is used.
+static __device__ __align__(256) unsigned char scratch[HIPTK_STATIC_WORKSPACE_BYTES];
+
+namespace
+{
+    constexpr int MAX_DEVICES = 64;
+    std::mutex    g_scratch_lock;
+    void*         g_scratch_ptr[MAX_DEVICES] = {};
+}
+
+extern "C" int hiptk_static_workspace(void** ptr, uint64_t* bytes, int* hip_error)
+{
+    if(hip_error)
+        *hip_error = 0;
+    if(!ptr || !bytes)
+        return HIPTK_ERR_ARG;
+    *ptr   = nullptr;
+    *bytes = 0;
+    int        dev = -1;
+    hipError_t e   = hipGetDevice(&dev);
+    if(e != hipSuccess || dev < 0 || dev >= MAX_DEVICES)
+    {
+        if(hip_error)
+            *hip_error = (int)e;
+        return HIPTK_ERR_LAUNCH;
+    }
+    std::lock_guard<std::mutex> guard(g_scratch_lock);
+    if(!g_scratch_ptr[dev])
+    {
+        void* p = nullptr;
+        e       = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+        if(e != hipSuccess || !p)
+        {
+            if(hip_error)
+                *hip_error = (int)e;
+            return HIPTK_ERR_LAUNCH;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr   = g_scratch_ptr[dev];
+    *bytes = HIPTK_STATIC_WORKSPACE_BYTES;
     return HIPTK_OK;
 }

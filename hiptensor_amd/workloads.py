@@ -332,6 +332,10 @@ class Contraction:
             self.handle, self.plan, self.alpha, A, B, self.beta, Cb, D, workspace,
             self.workspace_bytes if workspace_bytes is None else workspace_bytes, stream or None)
 
+    def run_no_alloc(self, A, B, Cb, D, stream=0):
+        """The same contraction through the entry point that takes its workspace from the library."""
+        return api.hiptensorContractionNoAlloc(self.handle, self.plan, self.alpha, A, B, self.beta, Cb, D, stream or None)
+
     def close(self):
         api.destroy("plan", self.plan)
         api.destroy("find", self.find)

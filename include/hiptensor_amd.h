@@ -93,6 +93,26 @@ int hiptensorAmdContraction(const void* handle,
                             uint64_t    workspaceSize,
                             void*       stream);
 
+/* hiptensorAmdContraction for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results as hiptensorAmdContraction, minus the workspace: whatever
+ * workspace the plan needs (split-K partials, packed operand copies) is taken from a device array
+ * of HIPTK_STATIC_WORKSPACE_BYTES (32 MiB) that the library itself holds on every device until the
+ * process ends.  The call allocates nothing and frees nothing (and skips the PERF_TRACE timing,
+ * which would create events).  A plan that needs more than the array holds is refused with
+ * HIPTENSOR_STATUS_INSUFFICIENT_WORKSPACE: plan with a smaller workspaceSize.  Every call on one
+ * device uses the same array: calls that overlap in time on one device (different streams, or
+ * threads) race on it and must be serialised by the caller; calls in one stream are safe. */
+int hiptensorAmdContractionNoAlloc(const void* handle,
+                                   const void* plan,
+                                   const void* alpha,
+                                   const void* A,
+                                   const void* B,
+                                   const void* beta,
+                                   const void* C,
+                                   void*       D,
+                                   void*       stream);
+
 /* hiptensorPermutation; typeScalar is a hipDataType, stream a hipStream_t  (hiptensor.hpp:89-98) */
 int hiptensorAmdPermutation(const void*    handle,
                             const void*    alpha,

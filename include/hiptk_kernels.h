@@ -125,6 +125,15 @@ int hiptk_contract(const hiptk_problem_t* prob,
                    void*                  stream,
                    int*                   hip_error);
 
+/* Device address and size of the workspace the library itself holds on the current device: a
+ * file-scope device array of HIPTK_STATIC_WORKSPACE_BYTES, present on every device from the moment
+ * the library is loaded until the process ends.  The first call on a device looks the address up
+ * (hipGetSymbolAddress; nothing is allocated), later calls return the stored address.  No
+ * counterpart in the reference; it serves hiptensorAmdContractionNoAlloc, the entry point for
+ * callers that cannot allocate.  Every user of the address on one device shares the same bytes. */
+#define HIPTK_STATIC_WORKSPACE_BYTES (32u << 20)
+int hiptk_static_workspace(void** ptr, uint64_t* bytes, int* hip_error);
+
 /* Fills `bytes` (a multiple of 4) of device memory with pseudo-random finite elements of the
  * class's storage type, magnitudes in [0.5, 1) and random signs, on `stream`.  No counterpart
  * in the reference: the measured kernel selection times its candidates on such data, since
