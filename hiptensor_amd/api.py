@@ -252,6 +252,13 @@ def planInfo(plan):
     return out
 
 
+def planCacheInfo(handle):
+    """(plan states, planning requests) the handle's cache holds."""
+    a, b = C.c_int64(0), C.c_int64(0)
+    check(lib.hiptensorAmdPlanCacheInfo(handle, C.byref(a), C.byref(b)), "hiptensorAmdPlanCacheInfo")
+    return a.value, b.value
+
+
 def planTable(plan, which):
     n = lib.hiptensorAmdPlanTable(plan, which, None, 0)
     if n < 0:

@@ -169,6 +169,8 @@ namespace
         return d->mTensorDesc.size() == 4 && d->mAlignmentReq.size() == 4 && d->mTensorMode.size() >= 3;
     }
 
+    // Key of a planning request.  `ws` is the workspace size as it bounds the plan: sizes beyond
+    // what planning can ever use are one request.
     std::string planKey(const hipta::ProblemIn& in, int algo, uint64_t ws)
     {
         std::ostringstream os;
@@ -620,7 +622,26 @@ hiptensorStatus_t hiptensorContractionGetWorkspaceSize(const hiptensorHandle_t* 
     if(pc.ranked.empty())
         return HIPTENSOR_STATUS_SUCCESS;
     if(pref == HIPTENSOR_WORKSPACE_RECOMMENDED)
-        *workspaceSize = pc.pack_bytes + pc.ranked.front().ws_bytes;
+    {
+        // RECOMMENDED never asks for more than the problem's own tensors occupy (at least 64 MiB,
+        // at most 1 GiB): a caller that allocates what is recommended at most doubles its footprint.
+        // Plans that want more (packed copies of large operands) are left to MAX.
+        const hipta::GemmView& v         = pc.view;
+        const uint64_t         footprint = (uint64_t)(v.spanA + v.spanB + v.spanC + v.spanD) * (uint64_t)v.elem_bytes;
+        const uint64_t         budget    = std::min<uint64_t>(1ull << 30, std::max<uint64_t>(64ull << 20, footprint));
+        uint64_t               need      = pc.pack_bytes + pc.ranked.front().ws_bytes;
+        if(need > budget)
+        {
+            hipta::ContractionPlanChoice bounded;
+            if(hipta::plan_contraction(in, candidatesOf(find), budget, std::min<uint64_t>(WS_CAP, budget), h->model(), hipta::repack_mode_from_env(), bounded, why)
+                   == hipta::PlanStatus::OK
+               && !bounded.ranked.empty())
+                need = bounded.pack_bytes + bounded.ranked.front().ws_bytes;
+            else
+                need = 0;
+        }
+        *workspaceSize = need;
+    }
     else
     {
         for(const hipta::Choice& c : pc.ranked)
@@ -671,15 +692,17 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
     // HIPTENSOR_AMD_FORCE_KERNEL="tile[,splitK]" pins the kernel choice (testing / tuning aid)
     const char*            force = std::getenv("HIPTENSOR_AMD_FORCE_KERNEL");
     const hipta::RepackMode repack = hipta::repack_mode_from_env();
-    const std::string       key    = planKey(in, (int)find->mSelectionAlgorithm, workspaceSize) + (force ? std::string("|force=") + force : std::string())
-                            + "|repack=" + std::to_string((int)repack);
+    const uint64_t          ws_eff = std::min<uint64_t>(workspaceSize, PACK_CAP + WS_CAP);
+    const std::string       problem = planKey(in, (int)find->mSelectionAlgorithm, 0) + (force ? std::string("|force=") + force : std::string())
+                                + "|repack=" + std::to_string((int)repack);
+    const std::string       key = problem + "|ws=" + std::to_string(ws_eff);
     PlanState*             st  = h->lookup(key);
     if(!st)
     {
         auto                         fresh = std::make_unique<PlanState>();
         std::string                  why;
         hipta::ContractionPlanChoice pc;
-        switch(hipta::plan_contraction(in, candidatesOf(find), std::min<uint64_t>(workspaceSize, PACK_CAP + WS_CAP), WS_CAP, h->model(), repack, pc, why))
+        switch(hipta::plan_contraction(in, candidatesOf(find), ws_eff, WS_CAP, h->model(), repack, pc, why))
         {
         case hipta::PlanStatus::OK: break;
         case hipta::PlanStatus::INVALID:
@@ -771,6 +794,15 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
             pick = hit;
         }
         const hipta::Choice& c = ranked[pick];
+        // what planning decided: requests that differ only in a workspace size that did not change
+        // the decision share one state (and one set of device tables)
+        const std::string decision = problem + "|tile=" + std::to_string(c.sol->tile_id) + ",split=" + std::to_string(c.split_k) + ",pack="
+                                     + std::to_string((int)pc.a.on) + std::to_string((int)pc.b.on) + "," + std::to_string((unsigned long long)pc.pack_bytes);
+        if(PlanState* known = h->findDecision(key, decision))
+        {
+            st = known;
+            goto planned;
+        }
         fresh->magic           = PlanState::MAGIC;
         fresh->sol             = c.sol;
         fresh->ws_bytes        = fresh->pack_bytes + c.ws_bytes;
@@ -807,8 +839,9 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
                 log.errorf(fn, "Could not place the offset tables on the device (%s)", hiptensorGetErrorString(e));
                 return e;
             }
-        st = h->intern(key, std::move(fresh));
+        st = h->intern(key, decision, std::move(fresh));
     }
+planned:
     const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     if(log.mask() & HIPTENSOR_LOG_LEVEL_PERF_TRACE)
     {
@@ -950,7 +983,18 @@ hiptensorStatus_t contractionImpl(const char*                       fn,
     }
     if(auto st = checkDevice(h, fn); st != HIPTENSOR_STATUS_SUCCESS)
         return st;
+    if(plan->mSolution && ((const PlanState*)plan->mSolution)->magic == PlanState::RETIRED)
+    {
+        // (retired states stay allocated for the life of the process, so this read is safe)
+        log.errorf(fn,
+                   "This plan is no longer valid: its handle was destroyed, or the handle's plan cache retired it; "
+                   "create the plan again (%s)",
+                   hiptensorGetErrorString(HIPTENSOR_STATUS_INTERNAL_ERROR));
+        return HIPTENSOR_STATUS_INTERNAL_ERROR;
+    }
     const PlanState* st = hipta::planState(plan);
+    if(st)
+        st->last_use.store(hipta::next_use_tick(), std::memory_order_relaxed);
     if(!st || st->device != h->device() || !st->dev_block)
     {
         log.errorf(fn, "Selected kernel is unable to solve the problem (%s)", hiptensorGetErrorString(HIPTENSOR_STATUS_INTERNAL_ERROR));
@@ -1006,12 +1050,25 @@ hiptensorStatus_t contractionImpl(const char*                       fn,
     packScalar(st->prob.cls, av, ab);
     packScalar(st->prob.cls, bv, bb);
 
-    const bool timed = !static_ws && (log.mask() & HIPTENSOR_LOG_LEVEL_PERF_TRACE) != 0;
+    bool timed = !static_ws && (log.mask() & HIPTENSOR_LOG_LEVEL_PERF_TRACE) != 0;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if(timed)
     {
-        if(hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
+        // timing synchronises with the stream, which would invalidate a capture in progress: the
+        // call is then enqueued untimed (no PERF_TRACE line)
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if(hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone)
+            timed = false;
+    }
+    if(timed)
+    {
+        if(hipEventCreate(&e0) != hipSuccess)
             return HIPTENSOR_STATUS_HIP_ERROR;
+        if(hipEventCreate(&e1) != hipSuccess)
+        {
+            (void)hipEventDestroy(e0);
+            return HIPTENSOR_STATUS_HIP_ERROR;
+        }
         (void)hipEventRecord(e0, stream);
     }
     int  hipErr     = 0;

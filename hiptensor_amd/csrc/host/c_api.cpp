@@ -350,6 +350,20 @@ extern "C" int hiptensorAmdPlanInfo(const void* plan, hiptensorAmdPlanInfo_t* ou
     return 0;
 }
 
+extern "C" int hiptensorAmdPlanCacheInfo(const void* handle, int64_t* states, int64_t* requests)
+{
+    if(!handle)
+        return (int)HIPTENSOR_STATUS_NOT_INITIALIZED;
+    hipta::Handle* h = hipta::Handle::from(((const hiptensorHandle_t*)handle)->fields);
+    if(!h)
+        return (int)HIPTENSOR_STATUS_NOT_INITIALIZED;
+    if(states)
+        *states = (int64_t)h->planCount();
+    if(requests)
+        *requests = (int64_t)h->aliasCount();
+    return 0;
+}
+
 extern "C" int64_t hiptensorAmdPlanTable(const void* plan, int which, int32_t* out, int64_t cap)
 {
     const hipta::PlanState* st = hipta::planState((const hiptensorContractionPlan_t*)plan);

@@ -2,6 +2,10 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
+#include <cstdlib>
+#include <iterator>
+
 namespace hipta
 {
     namespace
@@ -22,6 +26,8 @@ namespace hipta
             h->mModel.cus = cus;
         if(clock_ghz > 0)
             h->mModel.clock_ghz = clock_ghz;
+        if(const char* e = std::getenv("HIPTENSOR_AMD_PLAN_CACHE"))
+            h->mMaxPlans = (size_t)std::max(1, std::atoi(e));
         Slot* s  = reinterpret_cast<Slot*>(fields);
         s->magic = MAGIC;
         s->impl  = h;
@@ -45,46 +51,116 @@ namespace hipta
         }
     }
 
+    namespace
+    {
+        std::atomic<uint64_t> g_tick{1};
+        // retired plan states: kept (a few hundred bytes each) so that a stale plan reads RETIRED
+        std::mutex                              g_graveyard_lock;
+        std::vector<std::unique_ptr<PlanState>> g_graveyard;
+    }
+
+    uint64_t next_use_tick()
+    {
+        return g_tick.fetch_add(1, std::memory_order_relaxed);
+    }
+
+    void Handle::retire(std::unique_ptr<PlanState> p)
+    {
+        if(!p)
+            return;
+        if(p->dev_block)
+        {
+            (void)hipFree(p->dev_block);
+            p->dev_block = nullptr;
+        }
+        p->prob  = hiptk_problem_t{};
+        p->magic = PlanState::RETIRED;
+        for(std::vector<int32_t>* t : {&p->view.xp, &p->view.xk, &p->view.yq, &p->view.yk, &p->view.cp, &p->view.cq, &p->view.dp, &p->view.dq})
+            std::vector<int32_t>().swap(*t);
+        std::lock_guard<std::mutex> g(g_graveyard_lock);
+        g_graveyard.push_back(std::move(p));
+    }
+
     Handle::~Handle()
     {
         for(auto& kv : mPlans)
+            retire(std::move(kv.second));
+        mPlans.clear();
+        mAlias.clear();
+    }
+
+    void Handle::alias(const std::string& request, PlanState* st)
+    {
+        if(mAlias.size() >= MAX_ALIASES)
+            mAlias.clear(); // aliases only save a re-planning on the host
+        mAlias[request] = st;
+    }
+
+    PlanState* Handle::lookup(const std::string& request)
+    {
+        std::lock_guard<std::mutex> g(mLock);
+        auto                        it = mAlias.find(request);
+        if(it == mAlias.end())
+            return nullptr;
+        it->second->last_use.store(next_use_tick(), std::memory_order_relaxed);
+        return it->second;
+    }
+
+    PlanState* Handle::findDecision(const std::string& request, const std::string& decision)
+    {
+        std::lock_guard<std::mutex> g(mLock);
+        auto                        it = mPlans.find(decision);
+        if(it == mPlans.end())
+            return nullptr;
+        it->second->last_use.store(next_use_tick(), std::memory_order_relaxed);
+        alias(request, it->second.get());
+        return it->second.get();
+    }
+
+    PlanState* Handle::intern(const std::string& request, const std::string& decision, std::unique_ptr<PlanState> fresh)
+    {
+        std::unique_ptr<PlanState> victim;
+        PlanState*                 raw = nullptr;
         {
-            PlanState* p = kv.second.get();
-            if(p && p->dev_block)
+            std::lock_guard<std::mutex> g(mLock);
+            auto                        it = mPlans.find(decision);
+            if(it != mPlans.end())
             {
-                (void)hipFree(p->dev_block);
-                p->dev_block = nullptr;
+                if(fresh && fresh->dev_block)
+                    (void)hipFree(fresh->dev_block);
+                alias(request, it->second.get());
+                return it->second.get();
             }
-            if(p)
-                p->magic = 0;
+            if(mPlans.size() >= mMaxPlans)
+            {
+                // retire the least recently planned-or-executed state
+                auto lru = mPlans.begin();
+                for(auto jt = mPlans.begin(); jt != mPlans.end(); ++jt)
+                    if(jt->second->last_use.load(std::memory_order_relaxed) < lru->second->last_use.load(std::memory_order_relaxed))
+                        lru = jt;
+                for(auto at = mAlias.begin(); at != mAlias.end();)
+                    at = at->second == lru->second.get() ? mAlias.erase(at) : std::next(at);
+                victim = std::move(lru->second);
+                mPlans.erase(lru);
+            }
+            raw = fresh.get();
+            raw->last_use.store(next_use_tick(), std::memory_order_relaxed);
+            mPlans.emplace(decision, std::move(fresh));
+            alias(request, raw);
         }
-    }
-
-    PlanState* Handle::intern(const std::string& key, std::unique_ptr<PlanState> fresh)
-    {
-        std::lock_guard<std::mutex> g(mLock);
-        auto                        it = mPlans.find(key);
-        if(it != mPlans.end())
-        {
-            if(fresh && fresh->dev_block)
-                (void)hipFree(fresh->dev_block);
-            return it->second.get();
-        }
-        PlanState* raw = fresh.get();
-        mPlans.emplace(key, std::move(fresh));
+        retire(std::move(victim));
         return raw;
-    }
-
-    PlanState* Handle::lookup(const std::string& key)
-    {
-        std::lock_guard<std::mutex> g(mLock);
-        auto                        it = mPlans.find(key);
-        return it == mPlans.end() ? nullptr : it->second.get();
     }
 
     size_t Handle::planCount()
     {
         std::lock_guard<std::mutex> g(mLock);
         return mPlans.size();
+    }
+
+    size_t Handle::aliasCount()
+    {
+        std::lock_guard<std::mutex> g(mLock);
+        return mAlias.size();
     }
 }

@@ -7,6 +7,7 @@
 // are read once per handle rather than on every call, and the handle owns every plan
 // state it created, because the API has no call that destroys a plan.
 #pragma once
+#include <atomic>
 #include <cstdint>
 #include <map>
 #include <memory>
@@ -35,8 +36,17 @@ namespace hipta
         int             compute   = 0; // hiptensorComputeType_t (how alpha / beta are read)
         std::string     kernel_name;
         double          est_us = 0.0;
-        static constexpr uint64_t MAGIC = 0x504c414e68697074ull;
+        // last planning or execution that touched this state (a process-wide tick): the handle's
+        // cache retires the least recently used state when it is full
+        mutable std::atomic<uint64_t> last_use{0};
+        static constexpr uint64_t MAGIC   = 0x504c414e68697074ull;
+        // a state whose device tables were released: its handle was destroyed, or the handle's cache
+        // retired it.  The (small) object itself stays allocated until the process ends, so a plan
+        // that still points at it is refused instead of reading freed memory.
+        static constexpr uint64_t RETIRED = 0x5245544952454421ull;
     };
+
+    uint64_t next_use_tick();
 
     class Handle
     {
@@ -54,10 +64,21 @@ namespace hipta
         const DeviceModel& model() const { return mModel; }
         const std::string& arch() const { return mArch; }
 
-        // Returns the cached state for `key`, or adopts `fresh` under that key.
-        PlanState* intern(const std::string& key, std::unique_ptr<PlanState> fresh);
-        PlanState* lookup(const std::string& key);
+        // The cache has two levels.  A *request* key names what the caller asked for (problem,
+        // algorithm, workspace size, overrides); a *decision* key names what planning made of it
+        // (problem, kernel, split-K, packed copies).  Many requests (e.g. every workspace size) share
+        // one decision, and only decisions own a PlanState and device tables: their number is bounded
+        // by the kernel registry, not by the values callers pass.
+        PlanState* lookup(const std::string& request);
+        PlanState* findDecision(const std::string& request, const std::string& decision);
+        // Adopts `fresh` under `decision` (or returns the state another thread adopted first, freeing
+        // fresh's device block) and remembers `request` as an alias of it.
+        PlanState* intern(const std::string& request, const std::string& decision, std::unique_ptr<PlanState> fresh);
         size_t     planCount();
+        size_t     aliasCount();
+        // most states / aliases a handle keeps (HIPTENSOR_AMD_PLAN_CACHE=<states> overrides the first)
+        static constexpr size_t MAX_PLANS   = 4096;
+        static constexpr size_t MAX_ALIASES = 16384;
 
     private:
         Handle() = default;
@@ -66,6 +87,10 @@ namespace hipta
         std::string                                       mArch;
         DeviceModel                                       mModel;
         std::mutex                                        mLock;
-        std::map<std::string, std::unique_ptr<PlanState>> mPlans;
+        std::map<std::string, std::unique_ptr<PlanState>> mPlans; // by decision key
+        std::map<std::string, PlanState*>                 mAlias; // request key -> state
+        size_t                                            mMaxPlans = MAX_PLANS;
+        void retire(std::unique_ptr<PlanState> p); // releases the device tables, keeps the header
+        void alias(const std::string& request, PlanState* st);
     };
 }

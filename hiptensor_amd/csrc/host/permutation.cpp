@@ -222,12 +222,25 @@ hiptensorStatus_t hiptensorPermutation(const hiptensorHandle_t*           handle
     // alpha is read as typeScalar and widened to float (permutation_solution_impl.hpp:108-113)
     prob.alpha = typeScalar == HIP_R_16F ? halfToFloat(*(const uint16_t*)alpha) : *(const float*)alpha;
 
-    const bool timed = (log.mask() & HIPTENSOR_LOG_LEVEL_PERF_TRACE) != 0;
+    bool       timed = (log.mask() & HIPTENSOR_LOG_LEVEL_PERF_TRACE) != 0;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if(timed)
     {
-        if(hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
+        // timing synchronises with the stream, which would invalidate a capture in progress: the
+        // call is then enqueued untimed (no PERF_TRACE line)
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if(hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone)
+            timed = false;
+    }
+    if(timed)
+    {
+        if(hipEventCreate(&e0) != hipSuccess)
             return HIPTENSOR_STATUS_HIP_ERROR;
+        if(hipEventCreate(&e1) != hipSuccess)
+        {
+            (void)hipEventDestroy(e0);
+            return HIPTENSOR_STATUS_HIP_ERROR;
+        }
         (void)hipEventRecord(e0, stream);
     }
     int hipErr = 0;

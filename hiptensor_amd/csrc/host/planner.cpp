@@ -81,6 +81,7 @@ namespace hipta
             }
         }
 
+        // (the per-tensor check in build_view has already ruled out products that overflow)
         int64_t extent(const std::vector<Dim>& d)
         {
             int64_t e = 1;
@@ -241,6 +242,35 @@ namespace hipta
                     why = "a mode has extent 0";
                     return PlanStatus::UNSUPPORTED_SHAPE;
                 }
+
+        // Strides: the kernels address with unsigned 32-bit element offsets from each tensor's
+        // base, so a negative stride would reach outside the tensor; D must not map two indices
+        // of a mode onto one element (several work-items would write it).  Extents whose product
+        // overflows cannot be a tensor of fewer than 2^31 elements either.
+        for(const TensorIn* t : {&A, &B, &D, &C})
+        {
+            if(t == &C && !in.bilinear)
+                continue;
+            int64_t total = 1;
+            for(size_t i = 0; i < t->len.size(); i++)
+            {
+                if(t->stride[i] < 0)
+                {
+                    why = "a stride is negative";
+                    return PlanStatus::INVALID;
+                }
+                if(t == &D && t->stride[i] == 0 && t->len[i] > 1)
+                {
+                    why = "a mode of D of extent > 1 has stride 0";
+                    return PlanStatus::INVALID;
+                }
+                if(__builtin_mul_overflow(total, t->len[i], &total))
+                {
+                    why = "a tensor's extents overflow 64 bits";
+                    return PlanStatus::UNSUPPORTED_SHAPE;
+                }
+            }
+        }
 
         // ---- classify modes: M = D and A, N = D and B, K = A and B ----
         struct Raw

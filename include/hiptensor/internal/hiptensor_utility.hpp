@@ -58,10 +58,15 @@ namespace hiptensor_detail
 #endif
 
 // Half-precision values print as float (the stream has no inserter of its own for them).
-#ifdef __FLT16_MANT_DIG__
-inline std::ostream& operator<<(std::ostream& os, const _Float16& v)
+// (internal/types_ext.hpp offers the same inserter: whichever header comes first defines it)
+#if defined(__FLT16_MANT_DIG__) && !defined(HIPTENSOR_FLOAT16_INSERTER_DEFINED)
+#define HIPTENSOR_FLOAT16_INSERTER_DEFINED
+namespace std
 {
-    return os << static_cast<float>(v);
+    inline ostream& operator<<(ostream& os, const _Float16& v)
+    {
+        return os << static_cast<float>(v);
+    }
 }
 #endif
 

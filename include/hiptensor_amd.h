@@ -178,6 +178,12 @@ typedef struct hiptensorAmdPlanInfo
     char     pack_a_kernel[96], pack_b_kernel[96];
 } hiptensorAmdPlanInfo_t;
 int hiptensorAmdPlanInfo(const void* plan, hiptensorAmdPlanInfo_t* out);
+/* Size of a handle's plan cache: `states` = plan states it holds (each owns its offset tables on the
+ * device; one per distinct planning decision, at most 4096, the least recently used is retired beyond
+ * that), `requests` = distinct planning requests (problem x workspace size ...) that map onto them.
+ * No counterpart in the reference, whose plans point into process-wide singletons. */
+int hiptensorAmdPlanCacheInfo(const void* handle, int64_t* states, int64_t* requests);
+
 /* Copies offset table `which` (0 xp, 1 xk, 2 yq, 3 yk, 4 cp, 5 cq, 6 dp, 7 dq; logical
  * length only, without padding) into out[0..cap); returns the logical length. */
 int64_t hiptensorAmdPlanTable(const void* plan, int which, int32_t* out, int64_t cap);

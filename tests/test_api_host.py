@@ -209,3 +209,66 @@ def test_folded_extent_limit(host_handle):
     with pytest.raises(api.HiptensorError) as e:
         wl.Contraction(host_handle, w)
     assert e.value.status == api.HIPTENSOR_STATUS_NOT_SUPPORTED
+
+
+def test_strides_are_validated(host_handle):
+    """Negative strides anywhere, and a zero stride on a mode of D longer than 1, are refused at plan
+    time (the kernels address with unsigned offsets; a repeated D element would be written by several
+    work-items).  A zero stride on an input mode (a broadcast) plans."""
+    h = host_handle
+    base = cases.rank_case(2, "f32", 1.0, 2.0)
+    for tensor, value, ok in (("A", -1, False), ("B", -4, False), ("C", -1, False), ("D", -1, False), ("D", 0, False), ("A", 0, True)):
+        w = dict(base, strides={k: list(v) for k, v in base["strides"].items()})
+        w["strides"][tensor][1] = value
+        if ok:
+            c = wl.Contraction(h, w)
+            c.close()
+        else:
+            with pytest.raises(api.HiptensorError) as e:
+                wl.Contraction(h, w)
+            assert e.value.status == S.HIPTENSOR_STATUS_INVALID_VALUE, (tensor, value)
+    # extents whose product overflows 64 bits (the folded-extent limit catches smaller ones)
+    big = 1 << 33
+    ext = {0: big, 10: big, 20: big}
+    w = wl.make_workload("f32", api.HIPTENSOR_COMPUTE_32F, [0, 20], [10, 20], [0, 10], ext, 1.0, None)
+    with pytest.raises(api.HiptensorError) as e:
+        wl.Contraction(h, w)
+    assert e.value.status in (S.HIPTENSOR_STATUS_NOT_SUPPORTED, S.HIPTENSOR_STATUS_INVALID_VALUE)
+
+
+def test_plan_cache_is_bounded_by_decisions_not_by_workspace_sizes(host_handle):
+    """Planning one contraction with 10 000 different workspace sizes must not grow the handle's
+    cache with them: states are keyed by what planning decided (kernel, split-K, packed copies)."""
+    w = cases.rank_case(4, "f32", 1.0, 2.0)
+    c = wl.Contraction(host_handle, w)
+    before, _ = api.planCacheInfo(host_handle)
+    plans = []
+    for i in range(10000):
+        st, p = api.hiptensorInitContractionPlan(host_handle, c.desc, c.find, 1000 + 4097 * i)
+        assert st == 0
+        plans.append(p)
+    states, requests = api.planCacheInfo(host_handle)
+    assert states - before <= 16, (before, states)  # a handful of (tile, split-K) decisions at most
+    assert requests <= 16384 + 1
+    for p in plans:
+        api.destroy("plan", p)
+    c.close()
+
+
+def test_plan_cache_retires_least_recently_used_states(monkeypatch):
+    """With the cache capped at 3 states, a 4th problem retires the oldest: executing its plan is
+    refused with a clear status instead of touching released tables; a handle's plans are refused
+    after hiptensorDestroy."""
+    monkeypatch.setenv("HIPTENSOR_AMD_PLAN_CACHE", "3")
+    h = api.check(api.hiptensorCreateHostOnly())
+    cs = [wl.Contraction(h, cases.rank_case(r, "f32", 1.0, None)) for r in (2, 3, 4, 5)]
+    states, _ = api.planCacheInfo(h)
+    assert states == 3
+    # host-only handles refuse execution before they look at the plan: the retired state is visible
+    # through the inspection call instead
+    with pytest.raises(api.HiptensorError):
+        api.planInfo(cs[0].plan)
+    assert api.planInfo(cs[3].plan)["kernel_name"]
+    api.hiptensorDestroy(h)
+    with pytest.raises(api.HiptensorError):
+        api.planInfo(cs[3].plan)

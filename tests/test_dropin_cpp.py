@@ -28,6 +28,19 @@ def test_dropin_program_builds_and_links():
     assert os.path.exists(BIN) and os.path.exists(BIN_PERM)
 
 
+def test_internal_headers_build_and_hold_their_values(tmp_path):
+    """<hiptensor/internal/{types,config}.hpp> (element type names, numeric_limits of the 16-bit
+    types, maxExactInteger, convert, __half host operators, inserters) compile together with the
+    public header and compute what their names promise (a host-only program)."""
+    src = os.path.join(ROOT, "tests", "cpp", "internal_headers.cpp")
+    out = tmp_path / "internal_headers"
+    subprocess.run([HIPCC, "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"), src, "-o", str(out),
+                    "-L" + os.path.dirname(_lib.LIB_PATH), "-lhiptensor_amd",
+                    "-Wl,-rpath," + os.path.dirname(_lib.LIB_PATH)], check=True, capture_output=True)
+    r = subprocess.run([str(out)], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0 and r.stdout.startswith("ok"), (r.stdout, r.stderr)
+
+
 @pytest.mark.skipif(not os.path.isdir(REF_SAMPLES), reason="reference tree not mounted")
 @pytest.mark.parametrize("sample", [
     "simple_bilinear_contraction_f32_f32_f32_f32_compute_f32",

@@ -1,10 +1,14 @@
 """The reference's validation matrix written out in its own YAML schema.
 
-The documents are produced from the shape data in cases.py (ranks 1..6 with the reference's
-type rows, alpha / beta rows, algorithm and workspace lists; the mode-permutation rows), so
-the tests exercise hiptensor_amd.testconfig on the exact key names and nesting the reference's
-files use without carrying those files.  When the reference tree is mounted, the CPU tests
-also read its real files."""
+The parameter rows (type rows, algorithms, workspace preferences, alpha / beta rows, Lengths,
+Strides, Modes) are the reference's own: tests/golden/validation_rows.json holds them as data,
+taken from test/01_contraction/configs/validation/*.yaml and configs/mode_test_params.yaml by
+tests/golden/make_validation_rows.py.  They are written back out as documents with the key names
+and nesting the reference's files use, so that hiptensor_amd.testconfig (the reader) is exercised
+on that schema.  When the reference tree is mounted, the CPU tests also read its real files."""
+import json
+import os
+
 import cases
 
 REAL_TYPES = [["HIP_R_16F"] * 4 + ["HIP_R_32F"], ["HIP_R_16BF"] * 4 + ["HIP_R_32F"], ["HIP_R_32F"] * 5,
@@ -37,36 +41,30 @@ def document(type_rows, scale, alphas, betas, lengths, modes, algos=ALGOS, prefs
     return "\n".join(out) + "\n"
 
 
+def validation_rows():
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "validation_rows.json")) as f:
+        return json.load(f)["files"]
+
+
 def rank_lengths(rank):
-    """Three length rows per rank, like the reference's validation files."""
-    if rank == 1:
-        return [list(s) for s in cases.RANK1_SHAPES], [[0, 1], [2, 1], [0, 2]]
-    ms, ns, ks = list(range(rank)), list(range(rank, 2 * rank)), list(range(2 * rank, 3 * rank))
-    rows = []
-    for ext in ([5, 6, 3, 4, 3, 4, 2, 3, 4, 4, 3, 4, 2, 3, 1, 2, 3, 2], [4, 3, 6, 5, 1, 3, 1, 2, 4, 5, 1, 3, 2, 1, 3, 4, 2, 2],
-                [4, 2, 3, 1, 2, 4, 2, 4, 3, 1, 2, 4, 3, 2, 2, 1, 4, 3]):
-        e = {m: ext[j % len(ext)] for j, m in enumerate(ms + ns + ks)}
-        rows.append([[e[m] for m in ms + ks], [e[m] for m in ns + ks], [e[m] for m in ms + ns]])
-    return rows, [ms + ks, ns + ks, ms + ns]
+    """The Lengths rows and the Modes row of the reference's bilinear validation file of one rank."""
+    r = validation_rows()[f"bilinear_test_params_rank{rank}"]
+    return r["lengths"], r["modes"][0]
 
 
 def validation_documents():
-    """(name, expansion, yaml text) for every family x rank, plus the mode-permutation file."""
+    """(name, expansion, yaml text) for every family x rank of the reference's validation files,
+    plus its mode-permutation file."""
     docs = []
-    for rank in range(1, 7):
-        lens, modes = rank_lengths(rank)
-        docs.append((f"bilinear_rank{rank}", "combined",
-                     document(REAL_TYPES, False, [[0], [1], [1]], [[2], [0], [2]], lens, [modes])))
-        docs.append((f"scale_rank{rank}", "combined",
-                     document(REAL_TYPES, True, [[0], [1], [1]], None, lens, [modes])))
-        docs.append((f"complex_bilinear_rank{rank}", "combined",
-                     document(COMPLEX_TYPES, False, [[0, 0], [1, 1], [1.1, 1.2]], [[2, 2], [0, 0], [2.2, 2.3]], lens, [modes])))
-        docs.append((f"complex_scale_rank{rank}", "combined",
-                     document(COMPLEX_TYPES, True, [[0, 0], [1, 1], [1.1, 1.2]], None, lens, [modes])))
-    docs.append(("mode_permutations", "sequence",
-                 document([["HIP_C_32F", "HIP_C_32F", "NONE_TYPE", "HIP_C_32F", "HIP_C_32F"]], False, [[1.1, 1.2]], [[2.2, 2.3]],
-                          [c[0] for c in cases.MODE_CASES], [c[1] for c in cases.MODE_CASES],
-                          algos=ALGOS[:1], prefs=PREFS[:1])))
+    rows = validation_rows()
+    for fname in sorted(n for n in rows if n != "mode_test_params") + ["mode_test_params"]:
+        r = rows[fname]
+        name = "mode_permutations" if fname == "mode_test_params" else fname.replace("_test_params", "")
+        scale = "betas" not in r
+        docs.append((name, r["expansion"],
+                     document(r["data_types"], False, r["alphas"], None if scale else r["betas"], r["lengths"], r["modes"],
+                              algos=r["algos"], prefs=r["prefs"],
+                              strides=[x for x in r.get("strides", []) if x] or None)))
     return docs
 
 
