@@ -273,7 +273,8 @@ def main():
     ap.add_argument("--workload", default="cfg2_f16_scale",
                     help="a baseline configuration (cfg1 ... cfg5); rowmajor_{f16,bf16}_{scale,bilinear}: 4096^3 in "
                          "the reference's default (NULL-stride) layout; interleaved_f16 / interleaved_f16_d_too / "
-                         "interleaved_f32: operands with interleaved modes, contracted from packed copies")
+                         "interleaved_f32: operands with interleaved modes, contracted from packed copies; "
+                         "skinny_{f16,f32}_n16 / longk_{f16,f32}: bandwidth-bound shapes (roofline against HBM)")
     ap.add_argument("--all", action="store_true", help="also time every other configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-target", action="store_true", help="skip the bilinear f16 / bf16 rows of the default line")
@@ -308,7 +309,7 @@ def main():
         print(json.dumps(out))
         return
     cfgs = wl.baseline_configs()
-    w = cfgs[a.workload] if a.workload in cfgs else {**wl.interleaved_configs(), **wl.row_major_configs()}[a.workload]
+    w = cfgs[a.workload] if a.workload in cfgs else {**wl.interleaved_configs(), **wl.row_major_configs(), **wl.skinny_configs()}[a.workload]
     r = measure(handle, w, a.steps, a.warmup, a.settle)
     fl = wl.flops(w)
     tflops = fl / (r["kernel_ms"] * 1e-3) / 1e12
@@ -333,6 +334,12 @@ def main():
                      "hbm_GBs_algorithmic": wl.algorithmic_bytes(w) / (r["kernel_ms"] * 1e-3) / 1e9},
         "device": {"name": prop.name, "cus": cus, "clock_ghz": clock_ghz},
     }
+    if wl.flops(w) / wl.algorithmic_bytes(w) < 300.0:
+        # below the machine balance (2.5 PFLOP/s / 8 TB/s = 315 flop / byte): the kernel is priced
+        # against HBM, algorithmic bytes (every tensor touched once) over the launch duration
+        gbs = wl.algorithmic_bytes(w) / (r["kernel_ms"] * 1e-3) / 1e9
+        out["roofline"].update({"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                                "tflops": tflops, "algorithmic_bytes": wl.algorithmic_bytes(w)})
     # what a loop of nothing but this type's MFMA instruction sustains on this device
     ceil = {}
     for label, rnd in (("constant_operands", 0), ("random_operands", 1)):

@@ -74,13 +74,13 @@ namespace hiptk
     // stay resident in that XCD's L2.
     __device__ inline void tile_coords(int wg, int tiles_p, int tiles_q, int& tp, int& tq)
     {
+        // XCD x runs the workgroups wg = x, x + 8, ...: base = total / 8 of them, one more for the
+        // first total % 8 XCDs; give it the contiguous range of tiles that starts after its
+        // predecessors' shares
         const int total = tiles_p * tiles_q;
-        int       lin   = wg;
-        if(total % 8 == 0)
-        {
-            const int per = total / 8;
-            lin           = (wg & 7) * per + (wg >> 3);
-        }
+        const int xcd = wg & 7, nth = wg >> 3;
+        const int base = total >> 3, rem = total & 7;
+        const int lin  = xcd * base + (xcd < rem ? xcd : rem) + nth;
         constexpr int GROUP = 4;
         const int     band  = GROUP * tiles_q;
         const int     g     = lin / band;

@@ -274,6 +274,23 @@ def row_major_configs():
     return out
 
 
+def skinny_configs():
+    """Bandwidth-bound shapes (packed column-major, f16 and f32): contractions whose arithmetic
+    intensity is far below the machine balance, so that the figure of merit is GB/s of
+    algorithmic bytes against the HBM rate rather than TFLOP/s.
+      skinny_*_n16:  M = 8192, N = 16, K = 8192   (A dominates the traffic: read once, 16 columns of work)
+      longk_*:       M = N = 256, K = 65536        (a small output over a long reduction: split-K)"""
+    out = {}
+    for dtype, compute in (("f16", api.HIPTENSOR_COMPUTE_32F), ("f32", api.HIPTENSOR_COMPUTE_32F)):
+        ext = {0: 128, 1: 64, 10: 16, 20: 128, 21: 64}
+        out[f"skinny_{dtype}_n16"] = make_workload(dtype, compute, [0, 1, 20, 21], [10, 20, 21], [0, 1, 10], ext, 1.0, None,
+                                                   name=f"skinny_{dtype}_scale_8192x16x8192")
+        ext = {0: 16, 1: 16, 10: 16, 11: 16, 20: 256, 21: 256}
+        out[f"longk_{dtype}"] = make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None,
+                                              name=f"longk_{dtype}_scale_256x256x65536")
+    return out
+
+
 def interleaved_configs():
     """Layouts outside the baseline set: A and B stored with free and contracted modes
     interleaved (A[m0,k0,m1,k1], runs of 15 elements), 4845 x 4845 x 1001.  In place they can only
