@@ -38,6 +38,20 @@ HBM_PEAK_GBS = 8000.0
 # They are properties of (workload, kernel) and are not re-measured by a run of this script: a kernel
 # that has no profile reports null.
 MEASURED_TRAFFIC_KIB = {
+    # profiles/contract_hd_kernel_4096cubed.md
+    ("cfg2_f16_scale_4096", "TraitsF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (100080.0, 34560.0),
+    ("cfg2_f16_bilinear_4096", "TraitsF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (116540.0, 34591.0),
+    ("cfg2_bf16_bilinear_4096", "TraitsBF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (115910.0, 32770.0),
+    # profiles/contract_kernels_configs_1_3_4_5_counters.md (split-K: contraction kernel + reduction kernel)
+    ("cfg1_f32_bilinear_256", "WTraitsF32_64x64x16_00"): (823.0 + 1187.5, 2048.0 + 256.0),
+    ("cfg3_f64_bilinear_1920x1920x768", "WTraitsF64_64x64x16_00"): (74014.4, 28800.0),
+    ("cfg4_c32_bilinear_1024x1024x512", "WTraitsC32_64x64x8_00"): (12368.0 + 12348.0, 16384.0 + 8192.0),
+    ("cfg5_f16_bilinear_rank6_permuted", "TraitsF16_256x192x64_xfalse8_ytrue8_kafffalse_pipe4x2"): (325638.6, 102232.8),
+    # profiles/contract_bandwidth_bound_shapes.md
+    ("skinny_f16_scale_8192x16x8192", "TraitsF16_64x64x64_xfalse8_yfalse8_kafftrue"): (66629.0 + 1060.0, 2048.0 + 256.0),
+    ("longk_f16_scale_256x256x65536", "TraitsF16_64x64x64_xfalse8_yfalse8_kafftrue"): (98695.0 + 4123.5, 8192.0 + 128.0),
+    ("skinny_f32_scale_8192x16x8192", "WTraitsF32_64x64x16_00"): (133440.0 + 1060.0, 2048.0 + 512.0),
+    ("longk_f32_scale_256x256x65536", "WTraitsF32_128x128x16_00"): (132190.0 + 8219.5, 16384.0 + 256.0),
     # profiles/permute_kernels_1GiB_tensors.md
     ("perm_f32_512x64x128x64_2031", "permute_tiled_f32_128x128_r4_w4"): (524329.9, 1049097.7),
 }
@@ -334,9 +348,10 @@ def main():
                      "hbm_GBs_algorithmic": wl.algorithmic_bytes(w) / (r["kernel_ms"] * 1e-3) / 1e9},
         "device": {"name": prop.name, "cus": cus, "clock_ghz": clock_ghz},
     }
-    if wl.flops(w) / wl.algorithmic_bytes(w) < 300.0:
-        # below the machine balance (2.5 PFLOP/s / 8 TB/s = 315 flop / byte): the kernel is priced
-        # against HBM, algorithmic bytes (every tensor touched once) over the launch duration
+    if wl.flops(w) / wl.algorithmic_bytes(w) < peak * 1e12 / (HBM_PEAK_GBS * 1e9):
+        # below the machine balance of this type (peak flop/s over 8 TB/s: 315 flop / byte for f16 / bf16,
+        # 19.7 for f32, 9.8 for f64): the kernel is priced against HBM, algorithmic bytes (every tensor
+        # touched once) over the launch duration
         gbs = wl.algorithmic_bytes(w) / (r["kernel_ms"] * 1e-3) / 1e9
         out["roofline"].update({"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
                                 "tflops": tflops, "algorithmic_bytes": wl.algorithmic_bytes(w)})
@@ -379,6 +394,7 @@ def main():
             others[name] = {"kernel_ms": rr["kernel_ms"], "tflops": tf, "frac_peak": tf / PEAK_TFLOPS[cw["dtype"]],
                             "mfma_only_sustained_tflops": sustained,
                             "hbm_GBs_algorithmic": wl.algorithmic_bytes(cw) / (rr["kernel_ms"] * 1e-3) / 1e9,
+                            "traffic": measured_traffic(cw["name"], rr["info"]["kernel_name"]),
                             "kernel": rr["info"]["kernel_name"], "split_k": rr["info"]["split_k"], "dtype": cw["dtype"]}
         if not a.no_cpu:
             # the reference's CPU contraction beside the other configurations too: in full where
