@@ -830,6 +830,7 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         p.cq_stride = (int32_t)v.cq_stride;
         p.shift_p   = v.shift_p;
         p.shift_q   = v.shift_q;
+        p.xy_aligned = v.xy_aligned;
         p.xk_stride            = (int32_t)v.xk_stride;
         p.yk_stride            = (int32_t)v.yk_stride;
         fresh->kernel_name     = hiptk_kernel_name(&p);

@@ -90,6 +90,7 @@ namespace hipta
         p.cq_stride = (int32_t)v.cq_stride;
         p.shift_p   = v.shift_p;
         p.shift_q   = v.shift_q;
+        p.xy_aligned = v.xy_aligned;
         p.xk_stride = (int32_t)v.xk_stride;
         p.yk_stride = (int32_t)v.yk_stride;
         p.xp      = base + offs[0];

@@ -494,6 +494,26 @@ namespace hipta
             return PlanStatus::UNSUPPORTED_SHAPE;
         }
 
+        // 16-byte vectors that start on 16-byte multiples of the tensor's base (16-bit classes)
+        {
+            auto aligned = [](const std::vector<int32_t>& rows, int64_t nrows, const std::vector<int32_t>& ks, int64_t nk,
+                              bool kfast, int vec, bool shifted) {
+                if(vec != 8 || (!kfast && shifted))
+                    return false;
+                for(int64_t r = 0; r < nrows; r += kfast ? 1 : vec)
+                    if(rows[(size_t)r] % vec != 0)
+                        return false;
+                for(int64_t k = 0; k < nk; k += kfast ? vec : 1)
+                    if(ks[(size_t)k] % vec != 0)
+                        return false;
+                return true;
+            };
+            v.xy_aligned = (v.elem_bytes == 2 && aligned(v.xp, v.P, v.xk, v.K, v.x_kfast != 0, v.x_vec, v.shift_p != 0)
+                            && aligned(v.yq, v.Q, v.yk, v.K, v.y_kfast != 0, v.y_vec, v.shift_q != 0))
+                               ? 1
+                               : 0;
+        }
+
         v.spanA = span_elems(A.len, A.stride);
         v.spanB = span_elems(B.len, B.stride);
         v.spanD = span_elems(D.len, D.stride);

@@ -64,6 +64,8 @@ namespace hipta
         // vectors run along a row (column) index that is one contiguous run whose extent is not a
         // multiple of the vector: tiles that would overhang are moved back to end at P (Q)
         int shift_p = 0, shift_q = 0;
+        // every 16-byte vector of X and Y starts a multiple of 16 bytes from its tensor's base
+        int xy_aligned = 0;
         int elem_bytes = 0;
         // bytes each tensor spans in memory (1 + sum (len-1)*stride elements)
         int64_t spanA = 0, spanB = 0, spanC = 0, spanD = 0;

@@ -80,6 +80,7 @@ namespace hipta
         p.K        = v.K;
         p.shift_p  = v.shift_p;
         p.shift_q  = v.shift_q;
+        p.xy_aligned = v.xy_aligned;
         return hiptk_kernel_available(&p) != 0;
     }
 

@@ -1,10 +1,10 @@
-// f16 kernels that load their operand tiles straight into LDS (affine K, K a multiple of 32).
+// f16 kernels that load their operand tiles straight into LDS: 256 x 256 tile, affine K.
 #include "contract_hd.hpp"
 
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
-        HIPTK_HD_TILE(TraitsF16, 9),
+        HIPTK_HD_TILE(TraitsF16, 9, 256, true),
     };
 
     const KernelEntry* entries_f16_hd(int* count)

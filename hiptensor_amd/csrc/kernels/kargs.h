@@ -43,7 +43,7 @@ namespace hiptk
         int32_t     bp, bq, bk, threads, lds_bytes;
         const char* name;
         launch_fn   launch;
-        int32_t     k_multiple; // 0: any K; else K must be a multiple of this (no tail handling)
+        int32_t     k_multiple; // 0: any K; else K must be a multiple of this and at least bk
     };
 
     // Each kernel translation unit contributes its table.
@@ -54,7 +54,13 @@ namespace hiptk
     const KernelEntry* entries_bf16_vec(int* count);
     const KernelEntry* entries_bf16_gen(int* count);
     const KernelEntry* entries_f16_hd(int* count);
+    const KernelEntry* entries_f16_hd_tab(int* count);
+    const KernelEntry* entries_f16_hd192(int* count);
+    const KernelEntry* entries_f16_hd192_tab(int* count);
     const KernelEntry* entries_bf16_hd(int* count);
+    const KernelEntry* entries_bf16_hd_tab(int* count);
+    const KernelEntry* entries_bf16_hd192(int* count);
+    const KernelEntry* entries_bf16_hd192_tab(int* count);
     const KernelEntry* entries_f16_v4(int* count);
     const KernelEntry* entries_f16_v2(int* count);
     const KernelEntry* entries_bf16_v4(int* count);

@@ -19,7 +19,13 @@ namespace hiptk
             {
                 typedef const KernelEntry* (*src_fn)(int*);
                 const src_fn sources[] = {entries_f16_hd,
+                                          entries_f16_hd_tab,
+                                          entries_f16_hd192,
+                                          entries_f16_hd192_tab,
                                           entries_bf16_hd,
+                                          entries_bf16_hd_tab,
+                                          entries_bf16_hd192,
+                                          entries_bf16_hd192_tab,
                                           entries_f16_aff,
                                           entries_bf16_aff,
                                           entries_f16_vec,
@@ -170,8 +176,8 @@ namespace hiptk
                     // a tile can only be moved back to end at P / Q if it fits into P / Q
                     if((p->shift_p && p->P < e.bp) || (p->shift_q && p->Q < e.bq))
                         continue;
-                    // kernels without a K tail
-                    if(e.k_multiple > 0 && p->K % e.k_multiple != 0)
+                    // the direct-load kernels: a restricted K tail, vectors on 16-byte multiples
+                    if(e.k_multiple > 0 && (p->K % e.k_multiple != 0 || p->K < e.bk || !p->xy_aligned))
                         continue;
                     if(e.k_affine && p->k_affine)
                         return &e;
@@ -180,6 +186,26 @@ namespace hiptk
                 }
             }
             return table;
+        }
+
+        // The largest register-staged tile of the problem's class and layout: what runs in place of
+        // a direct-load kernel when an operand's base address is not 16-byte aligned.
+        const KernelEntry* staged_entry(const hiptk_problem_t* p)
+        {
+            const KernelEntry* best = nullptr;
+            hiptk_problem_t    q    = *p;
+            for(const KernelEntry& t : registry().all)
+            {
+                if(t.cls != p->cls || t.k_multiple > 0)
+                    continue;
+                q.tile_id            = t.tile_id;
+                const KernelEntry* e = find_entry(&q);
+                if(e && e->k_multiple == 0
+                   && (!best || e->bp * e->bq > best->bp * best->bq
+                       || (e->bp * e->bq == best->bp * best->bq && e->threads > best->threads)))
+                    best = e;
+            }
+            return best;
         }
     }
 }
@@ -259,6 +285,8 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
     if(bil && (!C || !beta || !prob->cp || !prob->cq))
         return HIPTK_ERR_ARG;
     const KernelEntry* e = find_entry(prob);
+    if(e && e->k_multiple > 0 && ((((uintptr_t)X) | ((uintptr_t)Y)) & 15) != 0)
+        e = staged_entry(prob);
     if(!e)
         return HIPTK_ERR_NO_KERNEL;
 

@@ -95,6 +95,12 @@ typedef struct hiptk_problem
                         its neighbour's rows and stores only its own).  Needs P >= the tile's rows;
                         tiles that do not fit are reported as unavailable                          */
     int32_t shift_q; /* likewise for the columns                                                    */
+    int32_t xy_aligned; /* 1: every 16-byte vector of X and Y starts a multiple of 16 bytes from its
+                           tensor's base (table entries at vector starts are multiples of the vector,
+                           no tile is moved back along a vector direction).  The kernels that load
+                           their operand tiles straight into LDS take only such problems, and only
+                           when the base addresses are 16-byte aligned too (checked at the launch,
+                           which otherwise runs the class's largest register-staged tile instead)  */
 } hiptk_problem_t;
 
 /* Number of tile configurations of a class, and their description. */

@@ -1,0 +1,306 @@
+// Host-side check of the direct-load contraction kernels' addressing (kernels/hd_addr.hpp, the
+// functions the kernels themselves call): a direct load has no bounds check and no mask, so for a
+// list of problems planned by the library's own planner this program walks every 16-byte request
+// of every lane, K tile, split-K slice and (sampled) output tile and checks that it
+//   * reads table entries inside the padded tables,
+//   * starts a multiple of 16 bytes from the tensor's base and ends inside the tensor's span,
+//   * covers 8 elements that are contiguous in memory (the planner's vector promise),
+// that the 16-byte slots of a stage tile it exactly once, that a k-contiguous operand's chunk is
+// the same for all of a lane's loads (the table form reads one entry per lane for them), and that
+// the K tiles of all slices multiply every k exactly once.  Exit code 0 and "ok" on success.
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "../../hiptensor_amd/csrc/host/planner.hpp"
+#include "../../hiptensor_amd/csrc/kernels/hd_addr.hpp"
+#include "../../include/hiptk_kernels.h"
+
+using namespace hipta;
+using hiptk::hd_next_origin;
+using hiptk::hd_slice;
+using hiptk::hd_slot;
+using hiptk::HdSlice;
+using hiptk::HdSlot;
+
+static int g_fail = 0;
+#define CHECK(cond, ...)                                                  \
+    do                                                                    \
+    {                                                                     \
+        if(!(cond))                                                       \
+        {                                                                 \
+            if(g_fail < 20)                                               \
+            {                                                             \
+                std::printf("FAIL %s:%d %s: ", __FILE__, __LINE__, #cond); \
+                std::printf(__VA_ARGS__);                                 \
+                std::printf("\n");                                        \
+            }                                                             \
+            g_fail++;                                                     \
+        }                                                                 \
+    } while(0)
+
+struct Case
+{
+    std::string                              name;
+    std::vector<int32_t>                     mA, mB, mD; // modes as listed
+    std::vector<std::pair<int32_t, int64_t>> ext;
+    std::vector<int32_t>                     oA, oB, oD; // storage order, fastest first (empty: as listed)
+    int64_t                                  padD = 0; // elements added after D's fastest mode
+    bool                                     bilinear = false;
+};
+
+static int64_t extent(const Case& c, int32_t m)
+{
+    for(auto& e : c.ext)
+        if(e.first == m)
+            return e.second;
+    return 0;
+}
+
+static TensorIn tensor(const Case& c, const std::vector<int32_t>& modes, std::vector<int32_t> order, int64_t pad)
+{
+    if(order.empty())
+        order = modes;
+    TensorIn t;
+    t.dtype = 2; // HIP_R_16F
+    t.mode  = modes;
+    t.len.resize(modes.size());
+    t.stride.resize(modes.size());
+    int64_t s = 1;
+    for(size_t i = 0; i < order.size(); i++)
+    {
+        const size_t at = std::find(modes.begin(), modes.end(), order[i]) - modes.begin();
+        t.len[at]       = extent(c, order[i]);
+        t.stride[at]    = s;
+        s *= t.len[at];
+        if(i == 0)
+            s += pad;
+    }
+    t.align = 256;
+    return t;
+}
+
+template <bool KF, int BR>
+static void check_operand(const char* what, const Case& c, const GemmView& v, bool is_x, int r0, const std::vector<int>& origins,
+                          bool affine)
+{
+    const std::vector<int32_t>& rtab    = is_x ? v.xp : v.yq;
+    const std::vector<int32_t>& ktab    = is_x ? v.xk : v.yk;
+    const int64_t               kstride = is_x ? v.xk_stride : v.yk_stride;
+    const int64_t               nrows   = is_x ? v.P : v.Q;
+    const int64_t               span    = (is_x != v.swapped) ? v.spanA : v.spanB;
+    std::vector<int>            seen(BR * 32 / 8, 0);
+    constexpr int               NL = BR / 64;
+    for(int wave = 0; wave < 4; wave++)
+        for(int lane = 0; lane < 64; lane++)
+        {
+            int k_first = -1;
+            for(int i = 0; i < NL; i++)
+            {
+                const int    s  = (wave * NL + i) * 64 + lane;
+                const HdSlot sl = hd_slot<KF, BR>(s);
+                CHECK(sl.row >= 0 && sl.row + (KF ? 1 : 8) <= BR && sl.k >= 0 && sl.k + (KF ? 8 : 1) <= 32, "%s %s slot %d -> row %d k %d",
+                      c.name.c_str(), what, s, sl.row, sl.k);
+                seen[KF ? sl.row * 4 + sl.k / 8 : sl.k * (BR / 8) + sl.row / 8]++;
+                if(KF)
+                {
+                    CHECK(k_first < 0 || k_first == sl.k, "%s %s lane %d: chunk differs between its loads", c.name.c_str(), what, lane);
+                    k_first = sl.k;
+                }
+                CHECK((size_t)(r0 + sl.row) < rtab.size(), "%s %s row table index %d of %zu", c.name.c_str(), what, r0 + sl.row, rtab.size());
+                const int64_t rowpart = rtab[(size_t)(r0 + sl.row)];
+                for(int o : origins)
+                {
+                    CHECK(o >= 0 && (size_t)(o + sl.k + 7) < ktab.size(), "%s %s k table index %d", c.name.c_str(), what, o + sl.k);
+                    const int64_t off = rowpart + (affine ? (int64_t)(o + sl.k) * kstride : (int64_t)ktab[(size_t)(o + sl.k)]);
+                    CHECK(off >= 0 && off + 8 <= span, "%s %s r0 %d slot %d origin %d: elements %lld..+8 of %lld", c.name.c_str(), what, r0, s, o,
+                          (long long)off, (long long)span);
+                    CHECK(off % 8 == 0, "%s %s r0 %d slot %d origin %d: offset %lld not a multiple of 8", c.name.c_str(), what, r0, s, o,
+                          (long long)off);
+                    // the 8 elements are the tile's (row, k .. k + 7) or (row .. row + 7, k)
+                    if(KF)
+                    {
+                        for(int j = 1; j < 8 && o + sl.k + j < v.K; j++)
+                            CHECK(ktab[(size_t)(o + sl.k + j)] - ktab[(size_t)(o + sl.k)] == j, "%s %s k run broken at %d", c.name.c_str(), what,
+                                  o + sl.k);
+                    }
+                    else
+                    {
+                        for(int j = 1; j < 8 && r0 + sl.row + j < nrows; j++)
+                            CHECK(rtab[(size_t)(r0 + sl.row + j)] - rowpart == j, "%s %s row run broken at %d", c.name.c_str(), what,
+                                  r0 + sl.row);
+                    }
+                    if(affine)
+                        CHECK(o + sl.k >= v.K || ktab[(size_t)(o + sl.k)] == (int64_t)(o + sl.k) * kstride, "%s %s affine k offset", c.name.c_str(), what);
+                }
+            }
+        }
+    for(size_t i = 0; i < seen.size(); i++)
+        CHECK(seen[i] == 1, "%s %s chunk %zu filled %d times", c.name.c_str(), what, i, seen[i]);
+}
+
+template <int BQ>
+static long check_tile_size(const Case& c, const GemmView& v)
+{
+    long      walked = 0;
+    const int K      = (int)v.K;
+    const int tiles_p = (int)((v.P + 255) / 256), tiles_q = (int)((v.Q + BQ - 1) / BQ);
+    const int ktiles  = (K + 31) / 32;
+    for(int want = 1; want <= 5; want++)
+    {
+        int split = std::min(want, ktiles);
+        int per   = (ktiles + split - 1) / split;
+        split     = (ktiles + per - 1) / per;
+        std::vector<int> covered((size_t)K, 0);
+        std::vector<int> origins; // every origin any slice requests, affine or table form
+        for(int z = 0; z < split; z++)
+        {
+            const HdSlice sl = hd_slice(K, z * per, per);
+            CHECK(sl.nt >= 0 && sl.n_load >= 1, "%s K %d slice %d/%d: nt %d n_load %d", c.name.c_str(), K, z, split, sl.nt, sl.n_load);
+            for(int u = 0; u < sl.nt; u++)
+                for(int k = 0; k < 32; k++)
+                    covered[(size_t)((z * per + u) * 32 + k)]++;
+            if(sl.half)
+                for(int k = K - 16; k < K; k++)
+                    covered[(size_t)k]++;
+            // affine form: running origin; table form: clamped tile index (both as the kernel steps them)
+            int ko = sl.k00, tk = z * per * 32;
+            for(int u = 0; u < sl.n_load + 12; u++)
+            {
+                const int to = std::min(tk, sl.kmax);
+                CHECK(ko >= 0 && ko <= K - 32 && to >= 0 && to <= K - 32, "%s origin out of range", c.name.c_str());
+                if(u < sl.nt)
+                    CHECK(ko == (z * per + u) * 32 && to == ko, "%s whole tile %d origin %d / %d", c.name.c_str(), u, ko, to);
+                else if(u == sl.nt && sl.half)
+                    CHECK(ko == K - 32 && to == K - 32, "%s tail tile origin %d / %d", c.name.c_str(), ko, to);
+                origins.push_back(ko);
+                origins.push_back(to);
+                ko = hd_next_origin(ko, sl.klast);
+                tk += 32;
+            }
+        }
+        for(int k = 0; k < K; k++)
+            CHECK(covered[(size_t)k] == 1, "%s K %d split %d: k %d multiplied %d times", c.name.c_str(), K, split, k, covered[(size_t)k]);
+        std::sort(origins.begin(), origins.end());
+        origins.erase(std::unique(origins.begin(), origins.end()), origins.end());
+        // sampled output tiles: the corners and the middle
+        std::vector<int> tps = {0, tiles_p / 2, tiles_p - 1}, tqs = {0, tiles_q / 2, tiles_q - 1};
+        for(int tp : tps)
+            for(int tq : tqs)
+            {
+                const int p_own = tp * 256, q_own = tq * BQ;
+                const int p0 = (v.shift_p && p_own + 256 > v.P) ? (int)v.P - 256 : p_own;
+                const int q0 = (v.shift_q && q_own + BQ > v.Q) ? (int)v.Q - BQ : q_own;
+                if(v.x_kfast)
+                    check_operand<true, 256>("X", c, v, true, p0, origins, v.k_affine != 0);
+                else
+                    check_operand<false, 256>("X", c, v, true, p0, origins, v.k_affine != 0);
+                if(v.y_kfast)
+                    check_operand<true, BQ>("Y", c, v, false, q0, origins, v.k_affine != 0);
+                else
+                    check_operand<false, BQ>("Y", c, v, false, q0, origins, v.k_affine != 0);
+                walked += (long)origins.size() * (256 + BQ) * 4;
+            }
+        if(want > 1 && split == 1)
+            break;
+    }
+    return walked;
+}
+
+int main()
+{
+    std::vector<Case> cases;
+    auto rank4 = [&](const char* name, std::vector<int32_t> mA, std::vector<int32_t> mB, std::vector<int32_t> mD, int64_t m0, int64_t m1,
+                     int64_t n0, int64_t n1, int64_t k0, int64_t k1) {
+        Case c;
+        c.name = name;
+        c.mA = mA, c.mB = mB, c.mD = mD;
+        c.ext = {{0, m0}, {1, m1}, {10, n0}, {11, n1}, {20, k0}, {21, k1}};
+        cases.push_back(c);
+    };
+    for(auto kk : std::vector<std::pair<int, int>>{{16, 3}, {16, 13}, {32, 1}, {32, 5}, {32, 11}, {16, 2}})
+    {
+        const std::string t = "k" + std::to_string(kk.first * kk.second);
+        rank4((t + "_rowfast").c_str(), {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 40, 9, 24, 13, kk.first, kk.second);
+        rank4((t + "_kfast").c_str(), {20, 21, 0, 1}, {20, 21, 10, 11}, {10, 11, 0, 1}, 40, 9, 24, 13, kk.first, kk.second);
+        rank4((t + "_mixed").c_str(), {0, 1, 20, 21}, {20, 21, 10, 11}, {10, 11, 0, 1}, 40, 9, 24, 13, kk.first, kk.second);
+        rank4((t + "_mixed2").c_str(), {20, 21, 0, 1}, {10, 11, 20, 21}, {0, 1, 10, 11}, 40, 9, 24, 13, kk.first, kk.second);
+    }
+    // 4096^3 (benchmark configuration 2) and its row-major form
+    rank4("cfg2", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 64, 64, 64, 64, 64, 64);
+    rank4("cfg2_rowmajor", {21, 20, 1, 0}, {21, 20, 11, 10}, {11, 10, 1, 0}, 64, 64, 64, 64, 64, 64);
+    // rows that are one ragged run (tiles moved back), K modes in different orders (tables), odd leading strides
+    rank4("ragged_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 15, 19, 17, 21, 16, 9);
+    rank4("ktable_rowfast", {0, 1, 20, 21}, {10, 11, 21, 20}, {0, 1, 10, 11}, 40, 9, 24, 13, 16, 27);
+    {
+        // three K modes, the outer two in different orders in A and B
+        for(int form = 0; form < 4; form++)
+        {
+            Case c;
+            c.name = std::string("ktab3_") + (form == 0 ? "rowfast" : form == 1 ? "kfast" : form == 2 ? "mixed" : "mixed2");
+            c.ext  = {{0, 40}, {1, 9}, {10, 24}, {11, 13}, {20, 16}, {21, 3}, {22, 5}};
+            const bool akf = form == 1 || form == 3, bkf = form == 1 || form == 2;
+            c.mA = akf ? std::vector<int32_t>{20, 21, 22, 0, 1} : std::vector<int32_t>{0, 1, 20, 21, 22};
+            c.mB = bkf ? std::vector<int32_t>{20, 22, 21, 10, 11} : std::vector<int32_t>{10, 11, 20, 22, 21};
+            c.mD = {0, 1, 10, 11};
+            cases.push_back(c);
+        }
+    }
+    {
+        // benchmark configuration 5 (rank 6, A and B stored permuted, D padded) at full and at reduced size
+        for(int small = 0; small < 3; small++)
+        {
+            Case c;
+            c.name = small == 0 ? "cfg5" : small == 1 ? "cfg5_small_k400" : "cfg5_small_k320";
+            if(small == 0)
+                c.ext = {{0, 32}, {1, 7}, {2, 24}, {10, 24}, {11, 9}, {12, 32}, {20, 17}, {21, 8}, {22, 30}};
+            else
+                c.ext = {{0, 32}, {1, 7}, {2, 8}, {10, 24}, {11, 2}, {12, 32}, {20, small == 1 ? 5 : 4}, {21, 8}, {22, 10}};
+            c.mA = {0, 1, 2, 20, 21, 22}, c.mB = {10, 11, 12, 20, 21, 22}, c.mD = {0, 1, 2, 10, 11, 12};
+            c.oA = {21, 0, 20, 2, 1, 22}, c.oB = {12, 20, 10, 22, 21, 11};
+            c.padD = 8, c.bilinear = true;
+            cases.push_back(c);
+        }
+    }
+    long walked = 0;
+    int  offered = 0;
+    for(const Case& c : cases)
+    {
+        ProblemIn in;
+        in.A = tensor(c, c.mA, c.oA, 0);
+        in.B = tensor(c, c.mB, c.oB, 0);
+        in.D = tensor(c, c.mD, c.oD, c.padD);
+        in.bilinear = c.bilinear;
+        if(c.bilinear)
+            in.C = in.D;
+        in.compute = 4; // HIPTENSOR_COMPUTE_32F
+        GemmView    v;
+        std::string why;
+        const PlanStatus st = build_view(in, v, why);
+        CHECK(st == PlanStatus::OK, "%s: %s", c.name.c_str(), why.c_str());
+        if(st != PlanStatus::OK)
+            continue;
+        // is a direct-load tile offered for it?  (tile ids 9: 256 x 256, 10: 256 x 192)
+        for(int tile : {9, 10})
+        {
+            hiptk_problem_t p{};
+            p.cls = v.cls, p.tile_id = tile, p.x_kfast = v.x_kfast, p.y_kfast = v.y_kfast, p.x_vec = v.x_vec, p.y_vec = v.y_vec;
+            p.k_affine = v.k_affine, p.P = v.P, p.Q = v.Q, p.K = v.K, p.shift_p = v.shift_p, p.shift_q = v.shift_q;
+            p.xy_aligned = v.xy_aligned;
+            const bool avail = hiptk_kernel_available(&p) != 0;
+            std::printf("%-22s P %5lld Q %5lld K %5lld xkf %d ykf %d vec %d/%d kaff %d shift %d/%d aligned %d tile %2d: %s\n", c.name.c_str(),
+                        (long long)v.P, (long long)v.Q, (long long)v.K, v.x_kfast, v.y_kfast, v.x_vec, v.y_vec, v.k_affine, v.shift_p, v.shift_q,
+                        v.xy_aligned, tile, avail ? "offered" : "not offered");
+            if(!avail)
+                continue;
+            CHECK(v.x_vec == 8 && v.y_vec == 8 && v.K % 16 == 0 && v.K >= 32 && v.xy_aligned, "%s offered outside its restrictions", c.name.c_str());
+            offered++;
+            walked += tile == 9 ? check_tile_size<256>(c, v) : check_tile_size<192>(c, v);
+        }
+    }
+    CHECK(offered >= 40, "only %d (case, tile) pairs were offered a direct-load kernel", offered);
+    std::printf("%s: %d problems x tiles, %ld requests walked, %d failures\n", g_fail ? "FAILED" : "ok", offered, walked, g_fail);
+    return g_fail ? 1 : 0;
+}

@@ -84,3 +84,17 @@ def test_dropin_permutation_program_runs():
     r = subprocess.run([BIN_PERM], capture_output=True, text=True, timeout=120)
     print(r.stdout, r.stderr, flush=True)
     assert r.returncode == 0 and "dropin_permutation: ok" in r.stdout
+
+
+def test_direct_load_kernels_request_only_what_exists(tmp_path):
+    """tests/cpp/hd_bounds.cpp: every 16-byte request of the kernels that load operand tiles straight
+    into LDS, walked on the host with the planner's own tables and the kernels' own address functions
+    (kernels/hd_addr.hpp), lies inside its tensor, is 16-byte aligned and contiguous; every stage
+    slot is filled once; every k is multiplied once (K tails, split-K slices, table-driven K)."""
+    src = os.path.join(ROOT, "tests", "cpp", "hd_bounds.cpp")
+    out = tmp_path / "hd_bounds"
+    subprocess.run(["g++", "-std=c++17", "-O1", "-I" + os.path.join(ROOT, "include"), "-isystem", "/opt/rocm/include",
+                    "-D__HIP_PLATFORM_AMD__", src, "-o", str(out), "-L" + os.path.dirname(_lib.LIB_PATH), "-lhiptensor_amd",
+                    "-Wl,-rpath," + os.path.dirname(_lib.LIB_PATH)], check=True, capture_output=True)
+    r = subprocess.run([str(out)], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip().splitlines()[-1].startswith("ok"), (r.stdout[-2000:], r.stderr)

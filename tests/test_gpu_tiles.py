@@ -69,9 +69,9 @@ def layouts(dtype, compute, big):
         out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], rk, a, None,
                                     name=f"tiles_ragged_{tag}_mixed_{dtype}"))
     if big:
-        # K a multiple of 32 with one stride per operand: the kernels that load their operand tiles
-        # straight into LDS have no K tail and take only these; 1, 4, 5 and 11 K tiles, row-fast,
-        # k-fast and mixed operands, whole and partial 256 x 256 output tiles
+        # K a multiple of 32 with one stride per operand, for the kernels that load their operand tiles
+        # straight into LDS (K a multiple of 16, operands in 16-byte vectors): 1, 4, 5 and 11 K tiles,
+        # row-fast, k-fast and mixed operands, whole and partial 256 x 256 / 256 x 192 output tiles
         for kk in ((32, 1), (32, 4), (32, 5), (32, 11)):
             dk = {0: 40, 1: 9, 10: 24, 11: 13, 20: kk[0], 21: kk[1]}
             tag = f"k{kk[0] * kk[1]}"
@@ -83,6 +83,32 @@ def layouts(dtype, compute, big):
                                         name=f"tiles_{tag}_mixed_{dtype}"))
             out.append(wl.make_workload(dtype, compute, [20, 21, 0, 1], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, None,
                                         name=f"tiles_{tag}_mixed2_{dtype}"))
+    if big:
+        # The same kernels with a K that ends 16 into a K tile of 32 (48 = 1.5 tiles, 208 = 6.5), and with
+        # K offsets from tables: three K modes whose outer two are stored in different orders in A and B
+        # (K = 240 = 7.5 tiles), row-fast, k-fast and mixed; and the rank-6 benchmark layout at reduced
+        # size (X in runs of 32 rows, Y in runs of 8 k; K = 400 and 320)
+        for kk in ((16, 3), (16, 13)):
+            dk = {0: 40, 1: 9, 10: 24, 11: 13, 20: kk[0], 21: kk[1]}
+            tag = f"k{kk[0] * kk[1]}"
+            out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, b,
+                                        name=f"tiles_{tag}_rowfast_{dtype}"))
+            out.append(wl.make_workload(dtype, compute, [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], dk, a, None,
+                                        name=f"tiles_{tag}_kfast_{dtype}"))
+            out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], dk, a, b,
+                                        name=f"tiles_{tag}_mixed_{dtype}"))
+        e3 = {0: 40, 1: 9, 10: 24, 11: 13, 20: 16, 21: 3, 22: 5}
+        out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21, 22], [10, 11, 20, 22, 21], [0, 1, 10, 11], e3, a, b,
+                                    name=f"tiles_ktab3_rowfast_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [20, 21, 22, 0, 1], [20, 22, 21, 10, 11], [10, 11, 0, 1], e3, a, None,
+                                    name=f"tiles_ktab3_kfast_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21, 22], [20, 22, 21, 10, 11], [10, 11, 0, 1], e3, a, b,
+                                    name=f"tiles_ktab3_mixed_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [20, 21, 22, 0, 1], [10, 11, 20, 22, 21], [0, 1, 10, 11], e3, a, None,
+                                    name=f"tiles_ktab3_mixed2_{dtype}"))
+        if dtype == "f16":
+            out.append(wl.config5(extents=(32, 2, 8, 24, 2, 16, 5, 8, 10)))
+            out.append(wl.config5(extents=(32, 2, 8, 24, 2, 16, 4, 8, 10)))
     # odd extents with the modes interleaved, so that no index is one contiguous run: scalar
     # gathers on every operand
     odd = {0: 7, 1: 23, 10: 5, 11: 29, 20: 3, 21: 37 if big else 21}
