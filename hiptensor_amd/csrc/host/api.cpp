@@ -831,6 +831,8 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         p.shift_p   = v.shift_p;
         p.shift_q   = v.shift_q;
         p.xy_aligned = v.xy_aligned;
+        p.x_max_off = (int32_t)v.x_max_off;
+        p.y_max_off = (int32_t)v.y_max_off;
         p.xk_stride            = (int32_t)v.xk_stride;
         p.yk_stride            = (int32_t)v.yk_stride;
         fresh->kernel_name     = hiptk_kernel_name(&p);

@@ -91,6 +91,8 @@ namespace hipta
         p.shift_p   = v.shift_p;
         p.shift_q   = v.shift_q;
         p.xy_aligned = v.xy_aligned;
+        p.x_max_off = (int32_t)v.x_max_off;
+        p.y_max_off = (int32_t)v.y_max_off;
         p.xk_stride = (int32_t)v.xk_stride;
         p.yk_stride = (int32_t)v.yk_stride;
         p.xp      = base + offs[0];

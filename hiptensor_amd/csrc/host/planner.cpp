@@ -494,6 +494,8 @@ namespace hipta
             return PlanStatus::UNSUPPORTED_SHAPE;
         }
 
+        v.x_max_off = mxp + mxk;
+        v.y_max_off = myq + myk;
         // 16-byte vectors that start on 16-byte multiples of the tensor's base (16-bit classes)
         {
             auto aligned = [](const std::vector<int32_t>& rows, int64_t nrows, const std::vector<int32_t>& ks, int64_t nk,

@@ -66,6 +66,8 @@ namespace hipta
         int shift_p = 0, shift_q = 0;
         // every 16-byte vector of X and Y starts a multiple of 16 bytes from its tensor's base
         int xy_aligned = 0;
+        // largest element offset of X / Y that the tables address
+        int64_t x_max_off = 0, y_max_off = 0;
         int elem_bytes = 0;
         // bytes each tensor spans in memory (1 + sum (len-1)*stride elements)
         int64_t spanA = 0, spanB = 0, spanC = 0, spanD = 0;

@@ -165,12 +165,14 @@ namespace hipta
         TileRate     r       = tile_rate(v.cls, s.bp * s.bq);
         if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152 && s.bk == 32)
         {
-            // the 256 x 256 tile whose operand tiles are loaded straight into LDS (four waves, K in
-            // steps of 32).  4096^3, both operands contiguous along their row index: 117.2 us against
+            // the 256 x 256 and 256 x 192 tiles whose operand tiles are loaded straight into LDS (four waves,
+            // K in steps of 32).  4096^3, both operands contiguous along their row index: 117.2 us against
             // 126.0 on eight waves (f16 scale), 115.5 against 125.9 (f16 bilinear), 108.5 against 118.4
             // (bf16 bilinear); both contiguous along k (64-byte runs per row and K step): 125.8 against
-            // 120.3
-            const double f = kper / s.bk < 16 ? 0.9 : (v.x_kfast || v.y_kfast) ? 0.95 : 1.08;
+            // 120.3; one of each (5376 x 6912 x 4080, 256 x 192 tiles): 274.5 against 286.8 (scale), 305.9
+            // against 307.3 (bilinear), and with the rank-6 benchmark's permuted storage and K tables 320.7
+            // against 354.7
+            const double f = kper / s.bk < 16 ? 0.9 : (v.x_kfast && v.y_kfast) ? 0.95 : (v.x_kfast || v.y_kfast) ? 1.03 : 1.08;
             r.alone *= f;
             r.full *= f;
         }

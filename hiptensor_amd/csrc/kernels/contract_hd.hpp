@@ -104,11 +104,14 @@ namespace hiptk
         uint32_t     voff[NL]; // byte offsets of this lane's 16 bytes (affine K: relative to the tile's k origin)
         uint32_t     rowb[KAFF ? 1 : NL]; // table form: the row part of voff, in bytes
         lds_u32_cptr kent[(KAFF || KF) ? 1 : NL]; // table form: this lane's entry in slot 0 of the wave's table ring
+        uint32_t     last; // table form: byte offset of the last vector the tables address
 
         // rtab: row offset table; r0: first row of the tile; kstride: element stride of k (affine form);
         // tab0: slot 0 of the wave's k-table ring; tabofs: first entry of this operand in a slot
-        __device__ inline void init(const int32_t* rtab, int r0, int kstride, int wave, int lane, lds_u32_cptr tab0, int tabofs)
+        __device__ inline void init(const int32_t* rtab, int r0, int kstride, int wave, int lane, lds_u32_cptr tab0, int tabofs,
+                                    uint32_t last_vec)
         {
+            last = last_vec;
 #pragma unroll
             for(int i = 0; i < NL; i++)
             {
@@ -140,13 +143,18 @@ namespace hiptk
                     e[i] = kent[i][S * 64];
             }
         }
+        // (clamped to the last vector the tables address: an entry that did not come out of LDS as it
+        // went in must not become a request outside the tensor)
         __device__ inline void set_offsets(const uint32_t (&e)[NL], uint32_t (&out)[NL]) const
         {
             if constexpr(!KAFF)
             {
 #pragma unroll
                 for(int i = 0; i < NL; i++)
-                    out[i] = rowb[i] + 2u * e[KF ? 0 : i];
+                {
+                    const uint32_t o = rowb[i] + 2u * e[KF ? 0 : i];
+                    out[i]           = o < last ? o : last;
+                }
             }
         }
     };
@@ -243,8 +251,8 @@ namespace hiptk
 
         HdLoader<XKF, BP, KAFF> gx;
         HdLoader<YKF, BQ, KAFF> gy;
-        gx.init(a.xp, p0, a.xk_stride, wave, lane, tab0, 0);
-        gy.init(a.yq, q0, a.yk_stride, wave, lane, tab0, 32);
+        gx.init(a.xp, p0, a.xk_stride, wave, lane, tab0, 0, a.x_last_vec);
+        gy.init(a.yq, q0, a.yk_stride, wave, lane, tab0, 32, a.y_last_vec);
         HdFrag<XKF, BP> fx;
         HdFrag<YKF, BQ> fy;
         fx.init(wp * 128, lane);

@@ -29,7 +29,9 @@ namespace hiptk
         // stores only the rows (columns) of its own range.  Lets vectors run along a contiguous
         // row (column) index whose extent is not a multiple of the vector.
         int32_t shift_p, shift_q;
-        double  alpha[2], beta[2];
+        // byte offset of the last 16-byte vector of X / Y that the tables address (direct-load kernels, table form)
+        uint32_t x_last_vec, y_last_vec;
+        double   alpha[2], beta[2];
     };
 
     // Tile-level launcher: returns hipError_t as int.

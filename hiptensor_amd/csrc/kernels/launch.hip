@@ -319,6 +319,8 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
     a.cd_vec    = prob->cd_vec;
     a.shift_p   = prob->shift_p ? 1 : 0;
     a.shift_q   = prob->shift_q ? 1 : 0;
+    a.x_last_vec = prob->x_max_off >= 7 ? 2u * (uint32_t)(prob->x_max_off - 7) : 0u;
+    a.y_last_vec = prob->y_max_off >= 7 ? 2u * (uint32_t)(prob->y_max_off - 7) : 0u;
     // A moved-back tile stores whole 8-element vectors of D that reach into its neighbour's
     // columns (same values).  When D is updated in place (C == D) the neighbour's elements must
     // not be read and written twice, so that case stores element by element.

@@ -101,6 +101,9 @@ typedef struct hiptk_problem
                            their operand tiles straight into LDS take only such problems, and only
                            when the base addresses are 16-byte aligned too (checked at the launch,
                            which otherwise runs the class's largest register-staged tile instead)  */
+    int32_t x_max_off, y_max_off; /* largest element offset xp[p] + xk[k] (yq[q] + yk[k]) over p < P, k < K:
+                                     the kernels that build load addresses from table entries they have
+                                     themselves moved through LDS clamp every address to it */
 } hiptk_problem_t;
 
 /* Number of tile configurations of a class, and their description. */

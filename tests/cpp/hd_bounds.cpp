@@ -117,6 +117,8 @@ static void check_operand(const char* what, const Case& c, const GemmView& v, bo
                     const int64_t off = rowpart + (affine ? (int64_t)(o + sl.k) * kstride : (int64_t)ktab[(size_t)(o + sl.k)]);
                     CHECK(off >= 0 && off + 8 <= span, "%s %s r0 %d slot %d origin %d: elements %lld..+8 of %lld", c.name.c_str(), what, r0, s, o,
                           (long long)off, (long long)span);
+                    // (the table form clamps every request to the last vector the tables address)
+                    CHECK(off <= (is_x ? v.x_max_off : v.y_max_off) - 7, "%s %s offset %lld beyond the last vector", c.name.c_str(), what, (long long)off);
                     CHECK(off % 8 == 0, "%s %s r0 %d slot %d origin %d: offset %lld not a multiple of 8", c.name.c_str(), what, r0, s, o,
                           (long long)off);
                     // the 8 elements are the tile's (row, k .. k + 7) or (row .. row + 7, k)
