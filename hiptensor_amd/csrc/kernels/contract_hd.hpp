@@ -55,18 +55,34 @@ namespace hiptk
     // states of a VALU instruction writing it (the compiler reloads spilled SGPRs with v_readlane,
     // possibly right in front of the asm statement), and M0 needs 1 wait state before the load that
     // reads it: s_nop 4 in front of the load covers both.
+    // The operands that must be scalar are passed through readfirstlane: an "s" constraint does not
+    // make the compiler move a (wave-uniform) value that it chose to compute in vector registers, and
+    // readfirstlane of a value that is in scalar registers already costs nothing.
+    __device__ __forceinline__ uint32_t hd_scalar(uint32_t v)
+    {
+        return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
+    }
+    __device__ __forceinline__ const void* hd_scalar(const void* p)
+    {
+        const uint64_t v = (uint64_t)p;
+        return (const void*)(((uint64_t)hd_scalar((uint32_t)(v >> 32)) << 32) | (uint64_t)hd_scalar((uint32_t)v));
+    }
     template <int OFF>
     __device__ __forceinline__ void dma_dst(uint32_t lds_base)
     {
-        asm volatile("s_add_u32 m0, %0, %1" : : "s"(lds_base), "n"(OFF) : "scc");
+        asm volatile("s_add_u32 m0, %0, %1" : : "s"(hd_scalar(lds_base)), "n"(OFF) : "scc");
+    }
+    __device__ __forceinline__ void dma_dst_at(uint32_t lds_base, uint32_t off)
+    {
+        asm volatile("s_add_u32 m0, %0, %1" : : "s"(hd_scalar(lds_base)), "s"(hd_scalar(off)) : "scc");
     }
     __device__ __forceinline__ void dma_load(uint32_t voff, const void* base)
     {
-        asm volatile("s_nop 4\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(base) : "memory");
+        asm volatile("s_nop 4\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
     }
     __device__ __forceinline__ void dma_load1(uint32_t voff, const void* base)
     {
-        asm volatile("s_nop 4\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(base) : "memory");
+        asm volatile("s_nop 4\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
     }
 
     // s_waitcnt immediates (gfx9 encoding): vmcnt(N) with the other counters left alone
@@ -395,6 +411,10 @@ namespace hiptk
                     }
                 }
                 acc[m / TQ][m % TQ] = Tr::mfma(xf[slot][m / TQ], yf[slot][m % TQ], acc[m / TQ][m % TQ]);
+                // (an MFMA has no side effect, so instruction selection may place it anywhere between its
+                // operands and the first use of its result, before the scheduler ever sees the barrier
+                // below: an empty ordered statement that reads the result keeps it here)
+                asm volatile("" : : "a"(acc[m / TQ][m % TQ]));
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -432,7 +452,7 @@ namespace hiptk
 #pragma unroll
                 for(int u = 0; u < NS; u++)
                 {
-                    asm volatile("s_add_u32 m0, %0, %1" : : "s"(wtab), "s"(u * 256) : "scc");
+                    dma_dst_at(wtab, u * 256);
                     dma_load1(tvoff, t_src());
                 }
                 __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
@@ -455,7 +475,7 @@ namespace hiptk
 #pragma unroll
                 for(int i = 0; i < 4; i++)
                 {
-                    asm volatile("s_add_u32 m0, %0, %1" : : "s"(xdst), "s"(i * 1024) : "scc");
+                    dma_dst_at(xdst, i * 1024);
                     dma_load(KAFF ? gx.voff[i] : pxv[KAFF ? 0 : t][i], xsrc);
                 }
                 if(t == 0) x_next(I1{});
@@ -467,13 +487,13 @@ namespace hiptk
                     if constexpr(!KAFF)
                     {
                         // entries of tile 4 + t, in the place the loop gives them: in front of a tile's Y loads
-                        asm volatile("s_add_u32 m0, %0, %1" : : "s"(wtab), "s"(t * 256) : "scc");
+                        dma_dst_at(wtab, t * 256);
                         dma_load1(tvoff, t_src());
                     }
 #pragma unroll
                     for(int i = 0; i < NYL; i++)
                     {
-                        asm volatile("s_add_u32 m0, %0, %1" : : "s"(ydst), "s"(i * 1024) : "scc");
+                        dma_dst_at(ydst, i * 1024);
                         dma_load(KAFF ? gy.voff[i] : pyv[KAFF ? 0 : t][i], ysrc);
                     }
                     if(t == 0) y_next(I1{});
@@ -578,7 +598,9 @@ namespace hiptk
     }
 }
 
-// Registry lines of the direct-load kernels: K a multiple of 16, at least 32.
+// Registry lines of the direct-load kernels: K a multiple of 16, at least 32.  (The table form is
+// instantiated for the 256 x 192 tile only: beside 256 accumulator registers the 256 x 256 tile has
+// no room for the table offsets, and spills in its main loop.)
 #define HIPTK_HD_ENTRY(TR, ID, BQ, XKF, YKF, KAFF)                                                \
     {                                                                                             \
         TR::CLS, ID, XKF, YKF, 8, 8, KAFF, 256, BQ, 32, 256, hiptk::HdGeom<BQ, KAFF>::LDS_BYTES,  \

@@ -56,11 +56,9 @@ namespace hiptk
     const KernelEntry* entries_bf16_vec(int* count);
     const KernelEntry* entries_bf16_gen(int* count);
     const KernelEntry* entries_f16_hd(int* count);
-    const KernelEntry* entries_f16_hd_tab(int* count);
     const KernelEntry* entries_f16_hd192(int* count);
     const KernelEntry* entries_f16_hd192_tab(int* count);
     const KernelEntry* entries_bf16_hd(int* count);
-    const KernelEntry* entries_bf16_hd_tab(int* count);
     const KernelEntry* entries_bf16_hd192(int* count);
     const KernelEntry* entries_bf16_hd192_tab(int* count);
     const KernelEntry* entries_f16_v4(int* count);

@@ -19,11 +19,9 @@ namespace hiptk
             {
                 typedef const KernelEntry* (*src_fn)(int*);
                 const src_fn sources[] = {entries_f16_hd,
-                                          entries_f16_hd_tab,
                                           entries_f16_hd192,
                                           entries_f16_hd192_tab,
                                           entries_bf16_hd,
-                                          entries_bf16_hd_tab,
                                           entries_bf16_hd192,
                                           entries_bf16_hd192_tab,
                                           entries_f16_aff,
