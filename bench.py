@@ -47,6 +47,7 @@ MEASURED_TRAFFIC_KIB = {
     ("cfg3_f64_bilinear_1920x1920x768", "WTraitsF64_64x64x16_00"): (74014.4, 28800.0),
     ("cfg4_c32_bilinear_1024x1024x512", "WTraitsC32_64x64x8_00"): (12368.0 + 12348.0, 16384.0 + 8192.0),
     ("cfg5_f16_bilinear_rank6_permuted", "TraitsF16_256x192x64_xfalse8_ytrue8_kafffalse_pipe4x2"): (325638.6, 102232.8),
+    ("cfg5_f16_bilinear_rank6_permuted", "TraitsF16_256x192x32_xfalse8_ytrue8_kafffalse_direct2x2"): (327800.0, 102000.0),
     # profiles/contract_bandwidth_bound_shapes.md
     ("skinny_f16_scale_8192x16x8192", "TraitsF16_64x64x64_xfalse8_yfalse8_kafftrue"): (66629.0 + 1060.0, 2048.0 + 256.0),
     ("longk_f16_scale_256x256x65536", "TraitsF16_64x64x64_xfalse8_yfalse8_kafftrue"): (98695.0 + 4123.5, 8192.0 + 128.0),
