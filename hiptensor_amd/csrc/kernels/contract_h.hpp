@@ -581,16 +581,49 @@ namespace hiptk
                 bool     ok[NVEC];
             };
             Slab sl[2];
+            // Offsets from tables, in a kernel with registers to spare (DEEP): the row look-ups of all
+            // slabs are made here, before the first store.  Inside the loop a look-up sits behind the
+            // stores of the slab before it, and the wait for it (its result is the address of a C
+            // load) is then also a wait for those stores: one store drain per slab.
+            // (The tables are padded beyond every index a tile reaches, so these need no guard.)
+            constexpr bool HOIST = DEEP && TP * NVEC <= 32;
+            uint32_t       hd[HOIST ? TP : 1][NVEC], hc[HOIST ? TP : 1][NVEC];
+            if constexpr(HOIST)
+            {
+                if(!aff)
+                {
+#pragma unroll
+                    for(int i = 0; i < TP; i++)
+#pragma unroll
+                        for(int v = 0; v < NVEC; v++)
+                        {
+                            const int p = pw + i * 32 + (v * 64 + lane) / VPR;
+                            hd[i][v]    = (uint32_t)a.dp[p] + dqo[v];
+                            hc[i][v]    = bil ? (uint32_t)a.cp[p] + cqo[v] : 0u;
+                        }
+                }
+            }
             auto prefetch = [&](int i, Slab& s) {
 #pragma unroll
                 for(int v = 0; v < NVEC; v++)
                 {
                     const int p = pw + i * 32 + (v * 64 + lane) / VPR;
                     s.ok[v]     = qok[v] && p_in(p);
-                    s.doff[v]   = !s.ok[v] ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
-                    u32x4_t c4  = {0u, 0u, 0u, 0u};
+                    uint32_t dof, cof;
+                    if(HOIST && !aff)
+                    {
+                        dof = hd[HOIST ? i : 0][v];
+                        cof = hc[HOIST ? i : 0][v];
+                    }
+                    else
+                    {
+                        dof = !s.ok[v] ? 0u : (aff ? (uint32_t)p * (uint32_t)a.dp_stride : (uint32_t)a.dp[p]) + dqo[v];
+                        cof = !(s.ok[v] && bil) ? 0u : (aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p]) + cqo[v];
+                    }
+                    s.doff[v]  = s.ok[v] ? dof : 0u;
+                    u32x4_t c4 = {0u, 0u, 0u, 0u};
                     if(s.ok[v] && bil)
-                        c4 = *(const u32x4_t*)(Cp + ((aff ? (uint32_t)p * (uint32_t)a.cp_stride : (uint32_t)a.cp[p]) + cqo[v]));
+                        c4 = *(const u32x4_t*)(Cp + cof);
                     s.c[v] = c4;
                 }
             };
