@@ -163,18 +163,22 @@ namespace hipta
         const double per_cu  = std::ceil(wgs / dev.cus); // workgroups the busiest CU runs
         const double sharing = std::min<double>(resident, per_cu);
         TileRate     r       = tile_rate(v.cls, s.bp * s.bq);
+        double round_extra_us = 0.0;
         if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152 && s.bk == 32)
         {
-            // the 256 x 256 and 256 x 192 tiles whose operand tiles are loaded straight into LDS (four waves,
-            // K in steps of 32).  4096^3, both operands contiguous along their row index: 117.2 us against
-            // 126.0 on eight waves (f16 scale), 115.5 against 125.9 (f16 bilinear), 108.5 against 118.4
-            // (bf16 bilinear); both contiguous along k (64-byte runs per row and K step): 125.8 against
-            // 120.3; one of each (5376 x 6912 x 4080, 256 x 192 tiles): 274.5 against 286.8 (scale), 305.9
-            // against 307.3 (bilinear), and with the rank-6 benchmark's permuted storage and K tables 320.7
-            // against 354.7
-            const double f = kper / s.bk < 16 ? 0.9 : (v.x_kfast && v.y_kfast) ? 0.95 : (v.x_kfast || v.y_kfast) ? 1.03 : 1.08;
+            // The 256 x 256 and 256 x 192 tiles whose operand tiles are loaded straight into LDS (four waves,
+            // K in steps of 32): a faster main loop, but one workgroup has the CU to itself, so nothing
+            // overlaps its prologue and epilogue.  Fitted to 4096 x 4096 x K, one round of 256 x 256 tiles, f16
+            // scale, against the eight-wave tile (us at K = 512 / 1024 / 2048 / 4096):
+            //   both operands row-contiguous  25.4 / 38.8 / 62.2 / 110.1  against  23.9 / 37.0 / 64.9 / 121.3
+            //   one of them k-contiguous      26.5 / 40.2 / 64.5 / 113.3  against  21.8 / 36.7 / 62.9 / 115.6
+            //   both k-contiguous             25.8 / 40.0 / 65.2 / 118.8  against  21.6 / 35.3 / 60.8 / 112.0
+            // i.e. 23.4 / 24.4 / 26.8 us per 1024 of K against 28.1 / 26.4 / 25.6, and 15.4 against 8.8 us that do
+            // not depend on K; four rounds (8192 x 8192 x 512): 103.3 against 85.8 us.
+            const double f = (v.x_kfast && v.y_kfast) ? 0.955 : (v.x_kfast || v.y_kfast) ? 1.08 : 1.20;
             r.alone *= f;
             r.full *= f;
+            round_extra_us = 6.5;
         }
         else if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152)
         {
@@ -210,7 +214,7 @@ namespace hipta
         // launch, and prologue + epilogue of every round of workgroups on a CU
         // (a workgroup's epilogue moves its output tile, and C, at about 30 GB/s per CU)
         const double tile_io = (double)s.bp * s.bq * v.elem_bytes * (v.bilinear ? 2.0 : 1.0) / 30e3;
-        us += 2.0 + (1.0 + tile_io) * std::ceil(per_cu / sharing);
+        us += 2.0 + (1.0 + tile_io + round_extra_us) * std::ceil(per_cu / sharing);
         if(split > 1)
         {
             const double ws = (double)split * v.P * v.Q * class_acc_bytes(v.cls);
