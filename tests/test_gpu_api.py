@@ -144,9 +144,26 @@ def test_contraction_inside_a_hip_graph(gpu_handle, oracle_mod):
     operand values written between the replays; every replay must equal the eager result."""
     import torch
 
-    for w in (wl.config1(), wl._rank4("f16", cases.COMPUTE["f16"], (16, 12), (8, 20), (8, 24), 1.0, 0.5, "graph_f16")):
+    import os
+
+    # (the last two pin the kernels that load operand tiles straight into LDS: one K stride, single pass;
+    # K offsets from tables with split-K)
+    e3 = {0: 40, 1: 9, 10: 24, 11: 13, 20: 16, 21: 3, 22: 5}
+    todo = [(wl.config1(), None),
+            (wl._rank4("f16", cases.COMPUTE["f16"], (16, 12), (8, 20), (8, 24), 1.0, 0.5, "graph_f16"), None),
+            (wl._rank4("f16", cases.COMPUTE["f16"], (40, 9), (24, 13), (16, 13), 1.0, 0.5, "graph_f16_direct"), "9,1"),
+            (wl.make_workload("bf16", cases.COMPUTE["bf16"], [0, 1, 20, 21, 22], [20, 22, 21, 10, 11], [10, 11, 0, 1], e3, 1.5, 0.75,
+                              name="graph_bf16_direct_tables"), "10,2")]
+    for w, force in todo:
         inp = wl.host_inputs(w)
-        c = wl.Contraction(gpu_handle, w, pref=api.HIPTENSOR_WORKSPACE_RECOMMENDED)
+        if force:
+            os.environ["HIPTENSOR_AMD_FORCE_KERNEL"] = force
+        try:
+            c = wl.Contraction(gpu_handle, w, pref=api.HIPTENSOR_WORKSPACE_MAX if force else api.HIPTENSOR_WORKSPACE_RECOMMENDED)
+        finally:
+            os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
+        assert not force or "direct" in c.info["kernel_name"], c.info
+        print(f"[case] {w['name']} {c.info['kernel_name']} split {c.info['split_k']}", flush=True)
         A, B, Cd = (gpu_util.to_device(inp[k]) for k in ("A", "B", "C"))
         D = gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"]))
         De = torch.empty_like(D)
