@@ -142,8 +142,10 @@ namespace hipta
                                        : TileRate{0.107, 0.21};
             case HIPTK_F64:
             case HIPTK_C64:
+                // (the 64 x 64 tile runs on eight waves, 16 x 32 outputs each: alone on a CU it reaches 0.64 of
+                // nominal on 1024^3 f64 against 0.53 on four waves; 1920^2 x 768: 104.9 against 108.1 us)
                 return area >= 16384  ? TileRate{0.76, 0.76}
-                       : area >= 4096 ? TileRate{0.45, 0.78}
+                       : area >= 4096 ? TileRate{0.60, 0.78}
                                       : TileRate{0.12, 0.69};
             case HIPTK_C32: return area >= 16384 ? TileRate{0.78, 0.78} : TileRate{0.48, 0.77};
             default: return area >= 16384 ? TileRate{0.73, 0.73} : TileRate{0.36, 0.66};

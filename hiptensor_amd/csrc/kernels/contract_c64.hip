@@ -4,7 +4,7 @@
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
-        HIPTK_W_TILE(WTraitsC64, 0, 64, 64, 8, 2, 2),
+        HIPTK_W_TILE(WTraitsC64, 0, 64, 64, 8, 4, 2),
         HIPTK_W_TILE(WTraitsC64, 1, 32, 32, 8, 2, 2),
         HIPTK_W_TILE(WTraitsC64, 2, 128, 128, 8, 2, 4),
     };

@@ -5,7 +5,7 @@ namespace hiptk
 {
     static const KernelEntry k_entries[] = {
         HIPTK_W_TILE(WTraitsF64, 0, 128, 128, 16, 2, 4),
-        HIPTK_W_TILE(WTraitsF64, 1, 64, 64, 16, 2, 2),
+        HIPTK_W_TILE(WTraitsF64, 1, 64, 64, 16, 4, 2),
     };
 
     const KernelEntry* entries_f64(int* count)
