@@ -496,11 +496,12 @@ namespace hipta
 
         v.x_max_off = mxp + mxk;
         v.y_max_off = myq + myk;
-        // 16-byte vectors that start on 16-byte multiples of the tensor's base (16-bit classes)
+        // 16-byte vectors that start on 16-byte multiples of the tensor's base
         {
-            auto aligned = [](const std::vector<int32_t>& rows, int64_t nrows, const std::vector<int32_t>& ks, int64_t nk,
-                              bool kfast, int vec, bool shifted) {
-                if(vec != 8 || (!kfast && shifted))
+            const int want = v.elem_bytes >= 1 && v.elem_bytes <= 16 ? 16 / v.elem_bytes : 0;
+            auto aligned = [want](const std::vector<int32_t>& rows, int64_t nrows, const std::vector<int32_t>& ks, int64_t nk,
+                                  bool kfast, int vec, bool shifted) {
+                if(want == 0 || vec != want || (!kfast && shifted))
                     return false;
                 for(int64_t r = 0; r < nrows; r += kfast ? 1 : vec)
                     if(rows[(size_t)r] % vec != 0)
@@ -510,7 +511,7 @@ namespace hipta
                         return false;
                 return true;
             };
-            v.xy_aligned = (v.elem_bytes == 2 && aligned(v.xp, v.P, v.xk, v.K, v.x_kfast != 0, v.x_vec, v.shift_p != 0)
+            v.xy_aligned = (aligned(v.xp, v.P, v.xk, v.K, v.x_kfast != 0, v.x_vec, v.shift_p != 0)
                             && aligned(v.yq, v.Q, v.yk, v.K, v.y_kfast != 0, v.y_vec, v.shift_q != 0))
                                ? 1
                                : 0;

@@ -30,6 +30,7 @@ namespace hipta
                 s.bk        = ti.bk;
                 s.threads   = ti.threads;
                 s.lds_bytes = ti.lds_bytes;
+                s.direct    = ti.k_multiple > 0;
                 s.name      = ti.name;
                 uint64_t h  = 0x68697074656e73ull;
                 for(uint64_t x : {(uint64_t)cls, (uint64_t)t, (uint64_t)ti.bp, (uint64_t)ti.bq, (uint64_t)ti.bk})
@@ -81,6 +82,8 @@ namespace hipta
         p.shift_p  = v.shift_p;
         p.shift_q  = v.shift_q;
         p.xy_aligned = v.xy_aligned;
+        p.x_max_off  = (int32_t)v.x_max_off;
+        p.y_max_off  = (int32_t)v.y_max_off;
         return hiptk_kernel_available(&p) != 0;
     }
 
@@ -146,9 +149,10 @@ namespace hipta
                 // nominal on 1024^3 f64 against 0.53 on four waves; 1920^2 x 768: 104.9 against 108.1 us)
                 return area >= 16384  ? TileRate{0.76, 0.76}
                        : area >= 4096 ? TileRate{0.60, 0.78}
-                                      : TileRate{0.12, 0.69};
-            case HIPTK_C32: return area >= 16384 ? TileRate{0.78, 0.78} : TileRate{0.48, 0.77};
-            default: return area >= 16384 ? TileRate{0.73, 0.73} : TileRate{0.36, 0.66};
+                                      : TileRate{0.25, 0.69}; // (640 x 640 x 64 complex f64 on 32 x 32 tiles: 10.5 us)
+            // (128 x 128 on 4096 x 4096 x 512, four tiles per CU: complex f32 548 us, f32 140.5 us)
+            case HIPTK_C32: return area >= 16384 ? TileRate{0.78, 0.82} : TileRate{0.48, 0.77};
+            default: return area >= 16384 ? TileRate{0.73, 0.85} : TileRate{0.36, 0.66};
             }
         }
     }
@@ -193,6 +197,23 @@ namespace hipta
             r.alone *= f;
             r.full *= f;
         }
+        if(s.direct && class_flops_per_clk_cu(v.cls) != 4096.0)
+        {
+            // The 32/64-bit 64 x 64 tiles whose operand tiles are loaded straight into LDS (four waves, two
+            // workgroups per CU): slopes of 1024 x 1024 x K (one workgroup per CU) and 2048 x 2048 x K scans
+            switch(v.cls)
+            {
+            case HIPTK_F32: r = TileRate{0.81, 0.89}; break;
+            case HIPTK_F64: r = TileRate{0.82, 0.90}; break;
+            case HIPTK_C32: r = TileRate{0.71, 0.80}; break;
+            default: break;
+            }
+            // ... whose prologue (tables, then the first tiles' flight) and epilogue nothing overlaps when a
+            // CU runs one or two rounds of them: 2048 x 2048 x K f32 fits 13.9 us + 60.5 us per 1024 of K
+            // (256^3 f32: one pass 9.2-9.8 us, four slices of four K tiles 7.8-8.1 us with the reduction: a
+            // slice shorter than the ring has less in flight to wait for)
+            round_extra_us = 2.0 * std::min(1.0, kper / s.bk / 16.0);
+        }
         if(class_max_vec(v.cls) > 1)
         {
             // narrower gathers are issue bound: measured on 2040^3 f16 problems whose runs
@@ -223,7 +244,9 @@ namespace hipta
             // partials out and back, second launch; partials that fit the 256 MiB last-level
             // cache never reach HBM
             const double bw = ws <= 160e6 ? dev.hbm_gbs * 1e3 * 1.0 : dev.hbm_gbs * 1e3 * 0.6;
-            us += 2.0 * ws / bw + 3.0 + 0.12 * split; // the reduction walks the slices one after another
+            // the reduction walks the slices one after another; and short slices are mostly prologue
+            // (512^3 in 8 slices against 4: f32 14.0 / 11.9 us, complex f32 24.5 / 20.5, 256^3 complex f64 13.5 / 11.3)
+            us += 2.0 * ws / bw + 3.0 + 0.25 * split;
         }
         return us;
     }

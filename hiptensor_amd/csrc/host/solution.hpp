@@ -23,6 +23,7 @@ namespace hipta
         uint64_t    uid; // stable id: hash of (class, tile shape)
         int         cls, tile_id;
         int         bp, bq, bk, threads, lds_bytes;
+        bool        direct; // operand tiles go from global memory straight into LDS
         std::string name;
     };
 

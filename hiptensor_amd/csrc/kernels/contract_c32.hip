@@ -1,11 +1,12 @@
 // complex f32 kernels (two v_mfma_f32_32x32x2_f32 per complex k).
-#include "contract_w.hpp"
+#include "contract_wd.hpp"
 
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
         HIPTK_W_TILE(WTraitsC32, 0, 128, 128, 8, 2, 4),
         HIPTK_W_TILE(WTraitsC32, 1, 64, 64, 8, 2, 2),
+        HIPTK_WD_ENTRY(WTraitsC32, 2, 8, 8),
     };
 
     const KernelEntry* entries_c32(int* count)

@@ -1,11 +1,12 @@
 // f32 kernels (v_mfma_f32_32x32x2_f32).
-#include "contract_w.hpp"
+#include "contract_wd.hpp"
 
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
         HIPTK_W_TILE(WTraitsF32, 0, 128, 128, 16, 2, 4),
         HIPTK_W_TILE(WTraitsF32, 1, 64, 64, 16, 2, 2),
+        HIPTK_WD_ENTRY(WTraitsF32, 2, 16, 8),
     };
 
     const KernelEntry* entries_f32(int* count)

@@ -1,11 +1,12 @@
 // f64 kernels (v_mfma_f64_16x16x4_f64).
-#include "contract_w.hpp"
+#include "contract_wd.hpp"
 
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
         HIPTK_W_TILE(WTraitsF64, 0, 128, 128, 16, 2, 4),
         HIPTK_W_TILE(WTraitsF64, 1, 64, 64, 16, 4, 2),
+        HIPTK_WD_ENTRY(WTraitsF64, 2, 8, 8),
     };
 
     const KernelEntry* entries_f64(int* count)

@@ -40,59 +40,11 @@
 // multiple of 16 and at least 32.
 #pragma once
 #include "contract_h.hpp"
+#include "dma_lds.hpp"
 #include "hd_addr.hpp"
 
 namespace hiptk
 {
-    // Direct load, in two halves so that another instruction (an MFMA) can sit between the write of
-    // M0 and the load that reads it (one wait state is required there):
-    //   dma_dst:  M0 <- LDS byte address lds_base + off (wave-uniform)
-    //   dma_load: 16 bytes per lane from global memory (base + 32-bit byte offset voff) to LDS address
-    //             M0 + 16 * lane (dma_load1: 4 bytes per lane to M0 + 4 * lane).  Counted by vmcnt.
-    // Nothing else in these kernels uses M0.
-    // The compiler's hazard recognizer does not look inside inline assembly, so the wait states an
-    // instruction needs are provided here: a VMEM instruction must not read an SGPR within 5 wait
-    // states of a VALU instruction writing it (the compiler reloads spilled SGPRs with v_readlane,
-    // possibly right in front of the asm statement), and M0 needs 1 wait state before the load that
-    // reads it: s_nop 4 in front of the load covers both.
-    // The operands that must be scalar are passed through readfirstlane: an "s" constraint does not
-    // make the compiler move a (wave-uniform) value that it chose to compute in vector registers, and
-    // readfirstlane of a value that is in scalar registers already costs nothing.
-    __device__ __forceinline__ uint32_t hd_scalar(uint32_t v)
-    {
-        return (uint32_t)__builtin_amdgcn_readfirstlane((int)v);
-    }
-    __device__ __forceinline__ const void* hd_scalar(const void* p)
-    {
-        const uint64_t v = (uint64_t)p;
-        return (const void*)(((uint64_t)hd_scalar((uint32_t)(v >> 32)) << 32) | (uint64_t)hd_scalar((uint32_t)v));
-    }
-    template <int OFF>
-    __device__ __forceinline__ void dma_dst(uint32_t lds_base)
-    {
-        asm volatile("s_add_u32 m0, %0, %1" : : "s"(hd_scalar(lds_base)), "n"(OFF) : "scc");
-    }
-    __device__ __forceinline__ void dma_dst_at(uint32_t lds_base, uint32_t off)
-    {
-        asm volatile("s_add_u32 m0, %0, %1" : : "s"(hd_scalar(lds_base)), "s"(hd_scalar(off)) : "scc");
-    }
-    __device__ __forceinline__ void dma_load(uint32_t voff, const void* base)
-    {
-        asm volatile("s_nop 4\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
-    }
-    __device__ __forceinline__ void dma_load1(uint32_t voff, const void* base)
-    {
-        asm volatile("s_nop 4\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
-    }
-
-    // s_waitcnt immediates (gfx9 encoding): vmcnt(N) with the other counters left alone
-    constexpr int waitcnt_vm(int n)
-    {
-        return (n & 15) | ((n >> 4) << 14) | 0x0F70;
-    }
-    // lgkmcnt(0) with the other counters left alone
-    constexpr int waitcnt_lgkm0 = 0xC07F;
-
     template <int BQ_, bool KAFF>
     struct HdGeom
     {

@@ -397,6 +397,104 @@ namespace hiptk
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
 
+    // Epilogue of the 32/64-bit kernels: D = alpha * acc (+ beta * C) for one wave tile, or the partial
+    // sums of a split-K slice into the workspace.  pw / qw: the first row of the wave tile and this
+    // lane's column in it; rows / columns from p_own / q_own on are the workgroup tile's to store.
+    template <typename Tr, int TP, int TQ>
+    __device__ __forceinline__ void
+        epilogue_w(const KArgs& a, typename Tr::Acc (&acc)[TP][TQ], int pw, int qw, int p_own, int q_own, int lane)
+    {
+        typedef typename Tr::E E;
+        typedef typename Tr::O O;
+        constexpr int          TILE = Tr::TILE;
+        auto                   p_in = [&](int p) { return p >= p_own && p < a.P; };
+        auto                   q_in = [&](int q) { return q >= q_own && q < a.Q; };
+        if(a.split_k > 1)
+        {
+            O* ws = (O*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+#pragma unroll
+                for(int r = 0; r < Tr::NREG; r++)
+                {
+                    const int p = pw + i * TILE + Tr::p_of(r, lane);
+                    if(!p_in(p))
+                        continue;
+                    O* wrow = ws + (size_t)p * a.Q;
+#pragma unroll
+                    for(int j = 0; j < TQ; j++)
+                    {
+                        const int q = qw + j * TILE;
+                        if(q_in(q))
+                            wrow[q] = Tr::get(acc[i][j], r);
+                    }
+                }
+            return;
+        }
+        E*         Dp  = (E*)a.D;
+        const E*   Cp  = (const E*)a.C;
+        const bool bil = a.bilinear != 0;
+        const bool aff = a.cd_affine != 0; // C / D offsets are index * stride: no table lookups
+        // D may alias C (and, for all the compiler knows, the offset tables), so written naively
+        // every element is one dependent round trip: offset, C element, D store.  The offsets and C
+        // elements of four accumulator rows are therefore fetched together, ahead of their stores.
+        // A lane outside the extents fetches element (0, 0) instead, a valid address, and stores
+        // nothing.
+        uint32_t dqo[TQ], cqo[TQ];
+        bool     qok[TQ];
+#pragma unroll
+        for(int j = 0; j < TQ; j++)
+        {
+            const int q  = qw + j * TILE;
+            qok[j]       = q_in(q);
+            const int qv = qok[j] ? q : 0;
+            dqo[j]       = aff ? (uint32_t)qv * (uint32_t)a.dq_stride : (uint32_t)a.dq[qv];
+            cqo[j]       = !bil ? 0u : aff ? (uint32_t)qv * (uint32_t)a.cq_stride : (uint32_t)a.cq[qv];
+        }
+        constexpr int RB = 4;
+        static_assert(Tr::NREG % RB == 0, "accumulator rows are fetched four at a time");
+#pragma unroll
+        for(int i = 0; i < TP; i++)
+#pragma unroll
+            for(int rb = 0; rb < Tr::NREG; rb += RB)
+            {
+                uint32_t dpo[RB], cpo[RB];
+                bool     pok[RB];
+#pragma unroll
+                for(int t = 0; t < RB; t++)
+                {
+                    const int p  = pw + i * TILE + Tr::p_of(rb + t, lane);
+                    pok[t]       = p_in(p);
+                    const int pv = pok[t] ? p : 0;
+                    dpo[t]       = aff ? (uint32_t)pv * (uint32_t)a.dp_stride : (uint32_t)a.dp[pv];
+                    cpo[t]       = !bil ? 0u : aff ? (uint32_t)pv * (uint32_t)a.cp_stride : (uint32_t)a.cp[pv];
+                }
+                E cv[RB][TQ];
+                if(bil)
+                {
+#pragma unroll
+                    for(int t = 0; t < RB; t++)
+#pragma unroll
+                        for(int j = 0; j < TQ; j++)
+                            cv[t][j] = Cp[cpo[t] + cqo[j]];
+                }
+#pragma unroll
+                for(int t = 0; t < RB; t++)
+#pragma unroll
+                    for(int j = 0; j < TQ; j++)
+                    {
+                        if(pok[t] && qok[j])
+                        {
+                            const E val = Tr::finish(Tr::get(acc[i][j], rb + t), a.alpha, a.beta, bil, &cv[t][j]);
+                            if constexpr(std::is_arithmetic<E>::value)
+                                __builtin_nontemporal_store(val, Dp + (dpo[t] + dqo[j]));
+                            else
+                                Dp[dpo[t] + dqo[j]] = val;
+                        }
+                    }
+            }
+    }
+
     template <typename Tr, int BP, int BQ, int BK, int WP, int WQ, int XM, int YM>
     __global__ void __launch_bounds__(WP* WQ * 64, 2) contract_w_kernel(const KArgs a)
     {
@@ -564,93 +662,7 @@ namespace hiptk
             buf ^= 1;
         }
 
-        // ---- epilogue ----
-        const int pw = p0 + wp * WTP;
-        const int qw = q0 + wq * WTQ + Tr::q_of(lane);
-        if(a.split_k > 1)
-        {
-            O* ws = (O*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
-#pragma unroll
-            for(int i = 0; i < TP; i++)
-#pragma unroll
-                for(int r = 0; r < Tr::NREG; r++)
-                {
-                    const int p = pw + i * TILE + Tr::p_of(r, lane);
-                    if(!p_in(p))
-                        continue;
-                    O* wrow = ws + (size_t)p * a.Q;
-#pragma unroll
-                    for(int j = 0; j < TQ; j++)
-                    {
-                        const int q = qw + j * TILE;
-                        if(q_in(q))
-                            wrow[q] = Tr::get(acc[i][j], r);
-                    }
-                }
-            return;
-        }
-        E*         Dp  = (E*)a.D;
-        const E*   Cp  = (const E*)a.C;
-        const bool bil = a.bilinear != 0;
-        const bool aff = a.cd_affine != 0; // C / D offsets are index * stride: no table lookups
-        // D may alias C (and, for all the compiler knows, the offset tables), so written naively
-        // every element is one dependent round trip: offset, C element, D store.  The offsets and C
-        // elements of four accumulator rows are therefore fetched together, ahead of their stores.
-        // A lane outside the extents fetches element (0, 0) instead, a valid address, and stores
-        // nothing.
-        uint32_t dqo[TQ], cqo[TQ];
-        bool     qok[TQ];
-#pragma unroll
-        for(int j = 0; j < TQ; j++)
-        {
-            const int q  = qw + j * TILE;
-            qok[j]       = q_in(q);
-            const int qv = qok[j] ? q : 0;
-            dqo[j]       = aff ? (uint32_t)qv * (uint32_t)a.dq_stride : (uint32_t)a.dq[qv];
-            cqo[j]       = !bil ? 0u : aff ? (uint32_t)qv * (uint32_t)a.cq_stride : (uint32_t)a.cq[qv];
-        }
-        constexpr int RB = 4;
-        static_assert(Tr::NREG % RB == 0, "accumulator rows are fetched four at a time");
-#pragma unroll
-        for(int i = 0; i < TP; i++)
-#pragma unroll
-            for(int rb = 0; rb < Tr::NREG; rb += RB)
-            {
-                uint32_t dpo[RB], cpo[RB];
-                bool     pok[RB];
-#pragma unroll
-                for(int t = 0; t < RB; t++)
-                {
-                    const int p  = pw + i * TILE + Tr::p_of(rb + t, lane);
-                    pok[t]       = p_in(p);
-                    const int pv = pok[t] ? p : 0;
-                    dpo[t]       = aff ? (uint32_t)pv * (uint32_t)a.dp_stride : (uint32_t)a.dp[pv];
-                    cpo[t]       = !bil ? 0u : aff ? (uint32_t)pv * (uint32_t)a.cp_stride : (uint32_t)a.cp[pv];
-                }
-                E cv[RB][TQ];
-                if(bil)
-                {
-#pragma unroll
-                    for(int t = 0; t < RB; t++)
-#pragma unroll
-                        for(int j = 0; j < TQ; j++)
-                            cv[t][j] = Cp[cpo[t] + cqo[j]];
-                }
-#pragma unroll
-                for(int t = 0; t < RB; t++)
-#pragma unroll
-                    for(int j = 0; j < TQ; j++)
-                    {
-                        if(pok[t] && qok[j])
-                        {
-                            const E val = Tr::finish(Tr::get(acc[i][j], rb + t), a.alpha, a.beta, bil, &cv[t][j]);
-                            if constexpr(std::is_arithmetic<E>::value)
-                                __builtin_nontemporal_store(val, Dp + (dpo[t] + dqo[j]));
-                            else
-                                Dp[dpo[t] + dqo[j]] = val;
-                        }
-                    }
-            }
+        epilogue_w<Tr, TP, TQ>(a, acc, p0 + wp * WTP, q0 + wq * WTQ + Tr::q_of(lane), p_own, q_own, lane);
     }
 
     template <typename Tr, int BP, int BQ, int BK>

@@ -58,6 +58,26 @@ namespace hiptk
         int row, k;
     };
 
+    // The 32/64-bit direct-load kernels (contract_wd.hpp): K tiles of bk, no tail (K is a multiple of
+    // bk); tiles requested beyond the slice's last one repeat it.
+    HIPTK_HD_FN int wd_next_origin(int ko, int klast, int bk)
+    {
+        return ko + bk < klast ? ko + bk : klast;
+    }
+
+    // ... their operand stages are tile[k][64 rows] of elements of 16 / V bytes, unpadded and
+    // unswizzled (one element per lane and MFMA operand: consecutive lanes read consecutive rows):
+    // the 16-byte slot s holds the V rows from `row` on at `k`.
+    template <int V>
+    HIPTK_HD_FN HdSlot wd_slot(int s)
+    {
+        HdSlot        o;
+        constexpr int cpr = 64 / V;
+        o.k               = s / cpr;
+        o.row             = V * (s % cpr);
+        return o;
+    }
+
     template <bool KF, int BR>
     HIPTK_HD_FN HdSlot hd_slot(int s)
     {

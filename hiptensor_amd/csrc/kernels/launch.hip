@@ -67,6 +67,21 @@ namespace hiptk
             }
         }
 
+        // bytes of one operand element in memory
+        int operand_bytes(int cls)
+        {
+            switch(cls)
+            {
+            case HIPTK_F16:
+            case HIPTK_BF16: return 2;
+            case HIPTK_F64:
+            case HIPTK_F64_AS_F32:
+            case HIPTK_C32: return 8;
+            case HIPTK_C64: return 16;
+            default: return 4;
+            }
+        }
+
         // ---- split-K reduction: sum the partials in slice order, apply alpha / beta ----
 
         struct FinF16
@@ -177,6 +192,14 @@ namespace hiptk
                     // the direct-load kernels: a restricted K tail, vectors on 16-byte multiples
                     if(e.k_multiple > 0 && (p->K % e.k_multiple != 0 || p->K < e.bk || !p->xy_aligned))
                         continue;
+                    // ... and they address an operand with 32-bit byte offsets
+                    if(e.k_multiple > 0)
+                    {
+                        const uint64_t eb   = (uint64_t)operand_bytes(p->cls);
+                        const int32_t  most = p->x_max_off > p->y_max_off ? p->x_max_off : p->y_max_off;
+                        if(most < 0 || ((uint64_t)most + 16 / eb) * eb > 0xFFFFFFFFull)
+                            continue;
+                    }
                     if(e.k_affine && p->k_affine)
                         return &e;
                     if(!e.k_affine && !table)
@@ -231,6 +254,7 @@ extern "C" int hiptk_tile_info(int cls, int tile_id, hiptk_tile_info_t* out)
             out->bk        = e.bk;
             out->threads   = e.threads;
             out->lds_bytes = e.lds_bytes;
+            out->k_multiple = e.k_multiple;
             std::snprintf(out->name, sizeof(out->name), "cls%d_%dx%dx%d", cls, e.bp, e.bq, e.bk);
             return HIPTK_OK;
         }

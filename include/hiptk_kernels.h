@@ -61,6 +61,9 @@ typedef struct hiptk_tile_info
     int32_t threads;    /* workgroup size                                    */
     int32_t lds_bytes;  /* static LDS                                        */
     char    name[64];
+    int32_t k_multiple; /* 0: operand tiles staged through registers, any K.  Otherwise the tile loads
+                           them straight into LDS: K must be a multiple of this and at least bk, and the
+                           problem xy_aligned                                  */
 } hiptk_tile_info_t;
 
 typedef struct hiptk_problem
@@ -103,7 +106,9 @@ typedef struct hiptk_problem
                            which otherwise runs the class's largest register-staged tile instead)  */
     int32_t x_max_off, y_max_off; /* largest element offset xp[p] + xk[k] (yq[q] + yk[k]) over p < P, k < K:
                                      the kernels that build load addresses from table entries they have
-                                     themselves moved through LDS clamp every address to it */
+                                     themselves moved through LDS clamp every address to it, and the
+                                     direct-load kernels are offered only while the byte offset of the
+                                     last vector fits 32 bits */
 } hiptk_problem_t;
 
 /* Number of tile configurations of a class, and their description. */

@@ -7,7 +7,9 @@
 //   * covers 8 elements that are contiguous in memory (the planner's vector promise),
 // that the 16-byte slots of a stage tile it exactly once, that a k-contiguous operand's chunk is
 // the same for all of a lane's loads (the table form reads one entry per lane for them), and that
-// the K tiles of all slices multiply every k exactly once.  Exit code 0 and "ok" on success.
+// the K tiles of all slices multiply every k exactly once.  The same for the 32/64-bit direct-load
+// kernels (64 x 64 tile, vectors of 16 / sizeof(element) rows, byte offsets that must fit 32 bits).
+// Exit code 0 and "ok" on success.
 #include <algorithm>
 #include <cstdint>
 #include <cstdio>
@@ -24,6 +26,8 @@ using hiptk::hd_slice;
 using hiptk::hd_slot;
 using hiptk::HdSlice;
 using hiptk::HdSlot;
+using hiptk::wd_next_origin;
+using hiptk::wd_slot;
 
 static int g_fail = 0;
 #define CHECK(cond, ...)                                                  \
@@ -59,12 +63,14 @@ static int64_t extent(const Case& c, int32_t m)
     return 0;
 }
 
+static int g_dtype = 2; // HIP_R_16F
+
 static TensorIn tensor(const Case& c, const std::vector<int32_t>& modes, std::vector<int32_t> order, int64_t pad)
 {
     if(order.empty())
         order = modes;
     TensorIn t;
-    t.dtype = 2; // HIP_R_16F
+    t.dtype = g_dtype;
     t.mode  = modes;
     t.len.resize(modes.size());
     t.stride.resize(modes.size());
@@ -211,6 +217,116 @@ static long check_tile_size(const Case& c, const GemmView& v)
     return walked;
 }
 
+// ---- the 32/64-bit kernels: V rows per 16-byte vector, K tiles of BK, NLW loads per wave and operand ----
+template <int V>
+static void check_wide_operand(const char* what, const Case& c, const GemmView& v, bool is_x, int r0, int BK, int NLW,
+                               const std::vector<int>& origins)
+{
+    const std::vector<int32_t>& rtab    = is_x ? v.xp : v.yq;
+    const std::vector<int32_t>& ktab    = is_x ? v.xk : v.yk;
+    const int64_t               kstride = is_x ? v.xk_stride : v.yk_stride;
+    const int64_t               nrows   = is_x ? v.P : v.Q;
+    const int64_t               span    = (is_x != v.swapped) ? v.spanA : v.spanB;
+    const int64_t               es      = 16 / V;
+    std::vector<int>            seen((size_t)BK * 64 / V, 0);
+    CHECK(4 * NLW * 64 == BK * 64 / V, "%s %s: %d loads do not tile a stage", c.name.c_str(), what, 4 * NLW * 64);
+    for(int wave = 0; wave < 4; wave++)
+        for(int lane = 0; lane < 64; lane++)
+            for(int i = 0; i < NLW; i++)
+            {
+                const int    s  = (wave * NLW + i) * 64 + lane;
+                const HdSlot sl = wd_slot<V>(s);
+                CHECK(sl.row >= 0 && sl.row + V <= 64 && sl.row % V == 0 && sl.k >= 0 && sl.k < BK, "%s %s slot %d -> row %d k %d", c.name.c_str(),
+                      what, s, sl.row, sl.k);
+                // the LDS bytes 16 s .. 16 s + 15 of a stage laid out [k][64 rows] are exactly these V rows at this k
+                CHECK((int64_t)16 * s == ((int64_t)sl.k * 64 + sl.row) * es, "%s %s slot %d is not where the readers look", c.name.c_str(), what, s);
+                seen[(size_t)(sl.k * (64 / V) + sl.row / V)]++;
+                CHECK((size_t)(r0 + sl.row) < rtab.size(), "%s %s row table index %d of %zu", c.name.c_str(), what, r0 + sl.row, rtab.size());
+                const int64_t rowpart = rtab[(size_t)(r0 + sl.row)];
+                for(int j = 1; j < V && r0 + sl.row + j < nrows; j++)
+                    CHECK(rtab[(size_t)(r0 + sl.row + j)] - rowpart == j, "%s %s row run broken at %d", c.name.c_str(), what, r0 + sl.row);
+                // the lane's part of the address, as the kernel computes it in 32 bits
+                const uint64_t lanepart = (uint64_t)es * ((uint64_t)rowpart + (uint64_t)sl.k * (uint64_t)kstride);
+                CHECK(lanepart <= 0xFFFFFFFFull, "%s %s lane offset overflows 32 bits", c.name.c_str(), what);
+                for(int o : origins)
+                {
+                    CHECK(o >= 0 && o + sl.k < v.K, "%s %s k %d of %lld", c.name.c_str(), what, o + sl.k, (long long)v.K);
+                    const uint64_t origin = (uint64_t)es * (uint64_t)o * (uint64_t)kstride;
+                    CHECK(origin <= 0xFFFFFFFFull, "%s %s origin overflows 32 bits", c.name.c_str(), what);
+                    const int64_t off = rowpart + (int64_t)(o + sl.k) * kstride;
+                    CHECK((uint64_t)off * es == lanepart + origin, "%s %s address parts", c.name.c_str(), what);
+                    CHECK(off >= 0 && off + V <= span, "%s %s r0 %d slot %d origin %d: elements %lld..+%d of %lld", c.name.c_str(), what, r0, s, o,
+                          (long long)off, V, (long long)span);
+                    CHECK(off % V == 0, "%s %s r0 %d slot %d origin %d: offset %lld not a multiple of %d", c.name.c_str(), what, r0, s, o,
+                          (long long)off, V);
+                    CHECK(ktab[(size_t)(o + sl.k)] == (int64_t)(o + sl.k) * kstride, "%s %s affine k offset", c.name.c_str(), what);
+                }
+            }
+    for(size_t i = 0; i < seen.size(); i++)
+        CHECK(seen[i] == 1, "%s %s vector %zu filled %d times", c.name.c_str(), what, i, seen[i]);
+}
+
+template <int V>
+static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
+{
+    long      walked = 0;
+    const int K      = (int)v.K;
+    const int tiles_p = (int)((v.P + 63) / 64), tiles_q = (int)((v.Q + 63) / 64);
+    const int ktiles  = K / BK;
+    CHECK(K % BK == 0 && K >= BK, "%s K %d offered to K tiles of %d", c.name.c_str(), K, BK);
+    for(int want = 1; want <= 7; want++)
+    {
+        int split = std::min(want, ktiles);
+        int per   = (ktiles + split - 1) / split;
+        split     = (ktiles + per - 1) / per;
+        std::vector<int> covered((size_t)K, 0);
+        std::vector<int> origins;
+        for(int z = 0; z < split; z++)
+        {
+            // as the kernel: the slice's tiles, then repeats of its last one (a ring of up to 8 stages)
+            const int kt_begin = z * per;
+            const int nt       = std::min(kt_begin + per, ktiles) - kt_begin;
+            CHECK(nt >= 1, "%s K %d slice %d/%d is empty", c.name.c_str(), K, z, split);
+            const int klast = (kt_begin + nt - 1) * BK;
+            int       ko    = kt_begin * BK;
+            for(int u = 0; u < nt + 12; u++)
+            {
+                CHECK(ko >= 0 && ko + BK <= K, "%s origin %d out of range", c.name.c_str(), ko);
+                if(u < nt)
+                {
+                    CHECK(ko == (kt_begin + u) * BK, "%s tile %d origin %d", c.name.c_str(), u, ko);
+                    for(int k = 0; k < BK; k++)
+                        covered[(size_t)(ko + k)]++;
+                }
+                else
+                    CHECK(ko == klast, "%s tile %d beyond the slice at %d, not at its last one %d", c.name.c_str(), u, ko, klast);
+                origins.push_back(ko);
+                ko = wd_next_origin(ko, klast, BK);
+            }
+        }
+        for(int k = 0; k < K; k++)
+            CHECK(covered[(size_t)k] == 1, "%s K %d split %d: k %d multiplied %d times", c.name.c_str(), K, split, k, covered[(size_t)k]);
+        std::sort(origins.begin(), origins.end());
+        origins.erase(std::unique(origins.begin(), origins.end()), origins.end());
+        for(int tp : {0, tiles_p / 2, tiles_p - 1})
+            for(int tq : {0, tiles_q / 2, tiles_q - 1})
+            {
+                check_wide_operand<V>("X", c, v, true, tp * 64, BK, NLW, origins);
+                check_wide_operand<V>("Y", c, v, false, tq * 64, BK, NLW, origins);
+                walked += (long)origins.size() * 2 * BK * 64 / V;
+            }
+        if(want > 1 && split == 1)
+            break;
+    }
+    return walked;
+}
+
+struct WideTile
+{
+    const char* type;
+    int         dtype, compute, elem_bytes, tile, bk;
+};
+
 int main()
 {
     std::vector<Case> cases;
@@ -290,7 +406,7 @@ int main()
             hiptk_problem_t p{};
             p.cls = v.cls, p.tile_id = tile, p.x_kfast = v.x_kfast, p.y_kfast = v.y_kfast, p.x_vec = v.x_vec, p.y_vec = v.y_vec;
             p.k_affine = v.k_affine, p.P = v.P, p.Q = v.Q, p.K = v.K, p.shift_p = v.shift_p, p.shift_q = v.shift_q;
-            p.xy_aligned = v.xy_aligned;
+            p.xy_aligned = v.xy_aligned, p.x_max_off = (int32_t)v.x_max_off, p.y_max_off = (int32_t)v.y_max_off;
             const bool avail = hiptk_kernel_available(&p) != 0;
             std::printf("%-22s P %5lld Q %5lld K %5lld xkf %d ykf %d vec %d/%d kaff %d shift %d/%d aligned %d tile %2d: %s\n", c.name.c_str(),
                         (long long)v.P, (long long)v.Q, (long long)v.K, v.x_kfast, v.y_kfast, v.x_vec, v.y_vec, v.k_affine, v.shift_p, v.shift_q,
@@ -303,6 +419,64 @@ int main()
         }
     }
     CHECK(offered >= 40, "only %d (case, tile) pairs were offered a direct-load kernel", offered);
-    std::printf("%s: %d problems x tiles, %ld requests walked, %d failures\n", g_fail ? "FAILED" : "ok", offered, walked, g_fail);
+
+    // ---- 32/64-bit classes ----
+    // benchmark configurations 1 (256^3), 3 (1920^2 x 768), 4 (1024^2 x 512) and a tensor of 2^32 bytes and more
+    rank4("cfg1", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 16, 16, 16, 16, 16, 16);
+    rank4("cfg3", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 48, 40, 48, 40, 32, 24);
+    rank4("cfg4", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 32, 32, 32, 32, 32, 16);
+    rank4("k8_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 40, 9, 24, 13, 8, 1);
+    rank4("k24_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 42, 9, 25, 13, 8, 3);
+    rank4("big_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 8192, 16, 64, 1, 64, 64);
+    const WideTile wide[] = {{"f32", 0, 4, 4, 2, 16}, {"f64", 1, 16, 8, 2, 8},
+                             {"c32", 4, 2048, 8, 2, 8}};
+    int offered_wide = 0, refused_big = 0;
+    for(const WideTile& w : wide)
+        for(const Case& c : cases)
+        {
+            g_dtype = w.dtype;
+            ProblemIn in;
+            in.A = tensor(c, c.mA, c.oA, 0);
+            in.B = tensor(c, c.mB, c.oB, 0);
+            in.D = tensor(c, c.mD, c.oD, c.padD);
+            in.bilinear = c.bilinear;
+            if(c.bilinear)
+                in.C = in.D;
+            in.compute = w.compute;
+            GemmView    v;
+            std::string why;
+            const PlanStatus st = build_view(in, v, why);
+            CHECK(st == PlanStatus::OK, "%s %s: %s", w.type, c.name.c_str(), why.c_str());
+            if(st != PlanStatus::OK)
+                continue;
+            hiptk_problem_t p{};
+            p.cls = v.cls, p.tile_id = w.tile, p.x_kfast = v.x_kfast, p.y_kfast = v.y_kfast, p.x_vec = v.x_vec, p.y_vec = v.y_vec;
+            p.k_affine = v.k_affine, p.P = v.P, p.Q = v.Q, p.K = v.K, p.shift_p = v.shift_p, p.shift_q = v.shift_q;
+            p.xy_aligned = v.xy_aligned, p.x_max_off = (int32_t)v.x_max_off, p.y_max_off = (int32_t)v.y_max_off;
+            const bool avail = hiptk_kernel_available(&p) != 0;
+            std::printf("%s %-22s P %5lld Q %5lld K %5lld xkf %d ykf %d vec %d/%d kaff %d shift %d/%d aligned %d tile %2d: %s\n", w.type,
+                        c.name.c_str(), (long long)v.P, (long long)v.Q, (long long)v.K, v.x_kfast, v.y_kfast, v.x_vec, v.y_vec, v.k_affine,
+                        v.shift_p, v.shift_q, v.xy_aligned, w.tile, avail ? "offered" : "not offered");
+            const bool big = (std::max(v.x_max_off, v.y_max_off) + 16 / w.elem_bytes) * (int64_t)w.elem_bytes > 0xFFFFFFFFll;
+            if(c.name == "big_rowfast" && big)
+            {
+                CHECK(!avail, "%s %s: offered although byte offsets pass 2^32", w.type, c.name.c_str());
+                refused_big++;
+            }
+            if(!avail)
+                continue;
+            const int V = 16 / w.elem_bytes;
+            CHECK(v.x_vec == V && v.y_vec == V && (V == 1 || (!v.x_kfast && !v.y_kfast)) && v.k_affine && v.K % w.bk == 0 && v.xy_aligned && !v.shift_p
+                      && !v.shift_q,
+                  "%s %s offered outside its restrictions", w.type, c.name.c_str());
+            offered_wide++;
+            const int nlw = w.bk * 64 * w.elem_bytes / 4096;
+            walked += V == 4 ? check_wide_tile<4>(c, v, w.bk, nlw) : check_wide_tile<2>(c, v, w.bk, nlw);
+        }
+    g_dtype = 2;
+    CHECK(offered_wide >= 30, "only %d (case, type, tile) triples were offered a 32/64-bit direct-load kernel", offered_wide);
+    CHECK(refused_big >= 2, "the tensor past 2^32 bytes was not exercised (%d)", refused_big);
+    std::printf("%s: %d + %d problems x tiles, %ld requests walked, %d failures\n", g_fail ? "FAILED" : "ok", offered, offered_wide, walked,
+                g_fail);
     return g_fail ? 1 : 0;
 }

@@ -109,6 +109,21 @@ def layouts(dtype, compute, big):
         if dtype == "f16":
             out.append(wl.config5(extents=(32, 2, 8, 24, 2, 16, 5, 8, 10)))
             out.append(wl.config5(extents=(32, 2, 8, 24, 2, 16, 4, 8, 10)))
+    if not big and compute == cases.COMPUTE[dtype]:
+        # The 32/64-bit kernels that load their operand tiles straight into LDS (row-fast operands in
+        # 16-byte vectors, one K stride, K a multiple of their K tile of 8 or 16; a ring of 4 or 8 tiles):
+        # a single K tile, fewer tiles than the ring holds, exactly one ring, several rings with a
+        # remainder; partial and whole 64 x 64 output tiles (complex f64 has no such kernel)
+        for kk in ((8, 1), (16, 1), (16, 3), (16, 8), (16, 13), (16, 17)):
+            dk = {0: 40, 1: 5, 10: 24, 11: 7, 20: kk[0], 21: kk[1]}
+            tag = f"k{kk[0] * kk[1]}"
+            out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, b,
+                                        name=f"tiles_{tag}_rowfast_{dtype}"))
+        dk = {0: 64, 1: 2, 10: 64, 11: 3, 20: 16, 21: 5}
+        out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, None,
+                                    name=f"tiles_k80_whole_tiles_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], dk, a, b,
+                                    name=f"tiles_k80_kfast_{dtype}"))
     # odd extents with the modes interleaved, so that no index is one contiguous run: scalar
     # gathers on every operand
     odd = {0: 7, 1: 23, 10: 5, 11: 29, 20: 3, 21: 37 if big else 21}
@@ -159,7 +174,7 @@ def _tile_exists(cls, tile):
     class TileInfo(ctypes.Structure):
         _fields_ = [("tile_id", ctypes.c_int32), ("bp", ctypes.c_int32), ("bq", ctypes.c_int32),
                     ("bk", ctypes.c_int32), ("threads", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
-                    ("name", ctypes.c_char * 64)]
+                    ("name", ctypes.c_char * 64), ("k_multiple", ctypes.c_int32)]
 
     ti = TileInfo()
     return lib.hiptk_tile_info(cls, tile, ctypes.byref(ti)) == 0
