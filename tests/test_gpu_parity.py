@@ -145,44 +145,53 @@ def test_non_finite_values_propagate_like_the_reference(gpu_handle, oracle_mod):
             assert fin.sum() > 0 and np.allclose(got[fin], ref[fin], rtol=cases.contract_tolerance(w), atol=cases.contract_tolerance(w))
 
 
-def test_direct_load_kernels_and_operand_alignment(gpu_handle, oracle_mod):
+@pytest.mark.parametrize("dtype,force,odd_ld", [("f16", "9,1", 364), ("f32", "2,1", 362), ("f64", "2,1", 361), ("c32", "2,2", 361)])
+def test_direct_load_kernels_and_operand_alignment(gpu_handle, oracle_mod, dtype, force, odd_ld):
     """The kernels that load operand tiles straight into LDS want every 16-byte vector of A and B on a
     16-byte boundary.  (1) Aligned problem: the pinned direct-load tile runs.  (2) The same plan executed
     with A and B one element off their allocation's alignment: the launch falls back to a register-staged
-    kernel and the result is the same.  (3) A leading dimension that is not a multiple of the vector:
-    the direct-load tiles are not offered at all, the default selection still contracts correctly."""
+    kernel and the result is the same (bit for bit in the 32/64-bit classes, whose two kernels multiply
+    and add in the same order).  (3) A leading dimension that is not a multiple of the vector: the
+    direct-load tiles are not offered at all, the default selection still contracts correctly."""
     import os
 
     import torch
 
     ext = {0: 40, 1: 9, 10: 24, 11: 13, 20: 32, 21: 5}
-    w = wl.make_workload("f16", cases.COMPUTE["f16"], [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.5, 0.75,
-                         name="aligned_rowfast_f16")
+    a, b = (1.5 + 0.5j, 0.75 - 0.25j) if dtype == "c32" else (1.5, 0.75)
+    w = wl.make_workload(dtype, cases.COMPUTE[dtype], [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, a, b,
+                         name=f"aligned_rowfast_{dtype}")
     inp = wl.host_inputs(w)
     exp = cases.logical_view(w, oracle_mod.contract(w, inp["A"], inp["B"], inp["C"]))
-    os.environ["HIPTENSOR_AMD_FORCE_KERNEL"] = "9,1"
+    os.environ["HIPTENSOR_AMD_FORCE_KERNEL"] = force
     try:
         c = wl.Contraction(gpu_handle, w, pref=api.HIPTENSOR_WORKSPACE_MAX)
         assert "direct" in c.info["kernel_name"], c.info
         stream = torch.cuda.current_stream().cuda_stream
+        ws = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
+        results = []
         for shift in (0, 1):
-            item = 2
+            item = wl.ELEM_BYTES[dtype]
             pad = np.zeros(shift, dtype=inp["A"].dtype)
             A = gpu_util.to_device(np.concatenate([pad, inp["A"]]))
             B = gpu_util.to_device(np.concatenate([pad, inp["B"]]))
             Cd = gpu_util.to_device(inp["C"])
             D = gpu_util.to_device(wl.nan_buffer(w["dtype"], inp["spanD"]))
             print(f"[case] {w['name']} operands shifted by {shift} element(s)", flush=True)
-            st = c.run(A.data_ptr() + shift * item, B.data_ptr() + shift * item, Cd.data_ptr(), D.data_ptr(), None, stream)
+            st = c.run(A.data_ptr() + shift * item, B.data_ptr() + shift * item, Cd.data_ptr(), D.data_ptr(),
+                       ws.data_ptr() if c.workspace_bytes else None, stream)
             torch.cuda.synchronize()
             api.check(st, "hiptensorContraction")
             got = D.cpu().numpy().view(wl.NP_STORE[w["dtype"]])
             cases.assert_parity(w, cases.logical_view(w, got), exp, f"{c.info['kernel_name']} shift {shift}")
+            results.append(got.copy())
+        if dtype != "f16":
+            assert np.array_equal(results[0].view(np.uint8), results[1].view(np.uint8)), "the two kernels' results differ"
         c.close()
-        # leading dimension of A = 364 elements (not a multiple of 8): no direct-load tile for this problem
-        sA = [1, 40, 364, 364 * 32]
-        w2 = wl.make_workload("f16", cases.COMPUTE["f16"], [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.5, 0.75,
-                              strideA=sA, name="odd_ld_rowfast_f16")
+        # a leading dimension of A that is not a multiple of the vector: no direct-load tile for this problem
+        sA = [1, 40, odd_ld, odd_ld * 32]
+        w2 = wl.make_workload(dtype, cases.COMPUTE[dtype], [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, a, b,
+                              strideA=sA, name=f"odd_ld_rowfast_{dtype}")
         with pytest.raises(api.HiptensorError):
             wl.Contraction(gpu_handle, w2, pref=api.HIPTENSOR_WORKSPACE_MAX)
     finally:
