@@ -144,14 +144,16 @@ namespace hipta
                        : area >= 16384 ? TileRate{0.265, 0.315}
                                        : TileRate{0.107, 0.21};
             case HIPTK_F64:
-            case HIPTK_C64:
                 // (the 64 x 64 tile runs on eight waves, 16 x 32 outputs each: alone on a CU it reaches 0.64 of
                 // nominal on 1024^3 f64 against 0.53 on four waves; 1920^2 x 768: 104.9 against 108.1 us)
-                return area >= 16384  ? TileRate{0.76, 0.76}
-                       : area >= 4096 ? TileRate{0.60, 0.78}
-                                      : TileRate{0.25, 0.69}; // (640 x 640 x 64 complex f64 on 32 x 32 tiles: 10.5 us)
-            // (128 x 128 on 4096 x 4096 x 512, four tiles per CU: complex f32 548 us, f32 140.5 us)
-            case HIPTK_C32: return area >= 16384 ? TileRate{0.78, 0.82} : TileRate{0.48, 0.77};
+                return area >= 16384 ? TileRate{0.76, 0.76} : TileRate{0.60, 0.78};
+            case HIPTK_C64:
+                // (2048^2 x 1024: 527 us on either tile; 1920^2 x 768: 406 us on 900 tiles of 64 x 64, 375 us on
+                // 3600 of 32 x 32; 512^3, one tile per CU: 74.8 us on 64 of the one, 26.6 us on 256 of the other)
+                return area >= 4096 ? TileRate{0.70, 0.82} : TileRate{0.50, 0.82};
+            // (128 x 128 on 4096 x 4096 x 512, four tiles per CU: complex f32 535 us, f32 140.5 us; complex f32 on
+            // 64 x 64: 1024^2 x 512 in one pass 50.7 us, 3072 x 1024 x 1024 203.6 us)
+            case HIPTK_C32: return area >= 16384 ? TileRate{0.84, 0.86} : TileRate{0.62, 0.82};
             default: return area >= 16384 ? TileRate{0.73, 0.85} : TileRate{0.36, 0.66};
             }
         }
@@ -205,7 +207,7 @@ namespace hipta
             {
             case HIPTK_F32: r = TileRate{0.81, 0.89}; break;
             case HIPTK_F64: r = TileRate{0.82, 0.90}; break;
-            case HIPTK_C32: r = TileRate{0.71, 0.80}; break;
+            case HIPTK_C32: r = TileRate{0.90, 0.91}; break;
             default: break;
             }
             // ... whose prologue (tables, then the first tiles' flight) and epilogue nothing overlaps when a
