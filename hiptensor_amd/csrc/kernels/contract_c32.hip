@@ -7,6 +7,7 @@ namespace hiptk
         HIPTK_W_TILE(WTraitsC32, 0, 128, 128, 8, 2, 4),
         HIPTK_W_TILE(WTraitsC32, 1, 64, 64, 8, 2, 2),
         HIPTK_WD_ENTRY(WTraitsC32, 2, 8, 8),
+        HIPTK_WK_ENTRY(WTraitsC32, 3, 8, 4),
     };
 
     const KernelEntry* entries_c32(int* count)

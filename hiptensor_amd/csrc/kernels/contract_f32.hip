@@ -7,6 +7,7 @@ namespace hiptk
         HIPTK_W_TILE(WTraitsF32, 0, 128, 128, 16, 2, 4),
         HIPTK_W_TILE(WTraitsF32, 1, 64, 64, 16, 2, 2),
         HIPTK_WD_ENTRY(WTraitsF32, 2, 16, 8),
+        HIPTK_WK_ENTRY(WTraitsF32, 3, 16, 4),
     };
 
     const KernelEntry* entries_f32(int* count)

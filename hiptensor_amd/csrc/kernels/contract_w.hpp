@@ -69,6 +69,7 @@ namespace hiptk
         }
         static __device__ inline int q_of(int lane) { return lane & 31; }
         static __device__ inline O   get(const Acc& a, int r) { return a.v[r]; }
+        static __device__ inline void put(Acc& a, int r, O x) { a.v[r] = x; }
         // alpha * x + beta * c with separately rounded products, as the CPU path does.
         static __device__ inline E finish(O x, const double* al, const double* be, bool bil, const E* c)
         {
@@ -109,6 +110,7 @@ namespace hiptk
         static __device__ inline int p_of(int r, int lane) { return 4 * r + (lane >> 4); }
         static __device__ inline int q_of(int lane) { return lane & 15; }
         static __device__ inline O   get(const Acc& a, int r) { return a.v[r]; }
+        static __device__ inline void put(Acc& a, int r, O x) { a.v[r] = x; }
         // alpha and beta are narrowed to float first: the reference's Bilinear / Scale
         // functors hold them as float even for f64 data.
         static __device__ inline E finish(O x, const double* al, const double* be, bool bil, const E* c)
@@ -182,6 +184,12 @@ namespace hiptk
         }
         static __device__ inline int q_of(int lane) { return lane & 31; }
         static __device__ inline O   get(const Acc& a, int r) { return make_float2(__fsub_rn(a.rr[r], a.ii[r]), a.im[r]); }
+        static __device__ inline void put(Acc& a, int r, O x)
+        {
+            a.rr[r] = x.x;
+            a.ii[r] = 0.f;
+            a.im[r] = x.y;
+        }
         static __device__ inline E finish(O x, const double* al, const double* be, bool bil, const E* c)
         {
             const float ar = (float)al[0], ai = (float)al[1];
@@ -236,6 +244,12 @@ namespace hiptk
         static __device__ inline int p_of(int r, int lane) { return 4 * r + (lane >> 4); }
         static __device__ inline int q_of(int lane) { return lane & 15; }
         static __device__ inline O   get(const Acc& a, int r) { return make_double2(__dsub_rn(a.rr[r], a.ii[r]), a.im[r]); }
+        static __device__ inline void put(Acc& a, int r, O x)
+        {
+            a.rr[r] = x.x;
+            a.ii[r] = 0.0;
+            a.im[r] = x.y;
+        }
         static __device__ inline E finish(O x, const double* al, const double* be, bool bil, const E* c)
         {
             const double ar = al[0], ai = al[1];

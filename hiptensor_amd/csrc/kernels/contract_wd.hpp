@@ -16,7 +16,7 @@
 //   * A wave holds the operands of two K tiles in registers: while tile t is multiplied, tile t + 1 is
 //     read from LDS and tile t + NS is requested into the stage tile t has just left, so a load has
 //     NS - 1 tiles of MFMA time to land and an LDS read one: the lead a single resident workgroup
-//     needs (1024 x 1024 x 512 complex f32 in one pass: 59 us through registers, 48 us here).  The
+//     needs (1024 x 1024 x 512 complex f32 in one pass: 50.7 us through registers, 38.7 us here).  The
 //     order of MFMAs, requests and reads inside a K tile is fixed by hand (see `step`).
 //   * The loads are inline assembly (dma_lds.hpp), invisible to the compiler, so the waits are placed
 //     by hand: loads complete in issue order, and before the barrier that hands tile t + 1 to the
@@ -48,28 +48,60 @@ namespace hiptk
         wd_static_for_impl(f, std::make_integer_sequence<int, N>{});
     }
 
-    template <typename Tr, int BK, int NS>
+    // WK = false: 64 x 64 tile, the four waves (2 x 2) share one ring.  WK = true: 32 x 32 tile, every wave
+    // multiplies all of it over its own quarter of the K range out of a ring of its own (no barrier in the
+    // loop), and the four partial tiles are added through LDS at the end: for outputs too small to fill the
+    // device with 64 x 64 tiles, in one launch.
+    template <typename Tr, int BK, int NS, bool WK>
     struct WdGeom
     {
-        static constexpr int BP = 64, BQ = 64;
+        static constexpr int ROWS = WK ? 32 : 64; // rows of an operand tile
+        static constexpr int BP = ROWS, BQ = ROWS;
         static constexpr int ES       = (int)sizeof(typename Tr::S);
         static constexpr int V        = 16 / ES; // elements per 16-byte vector
-        static constexpr int OP_BYTES = BK * 64 * ES; // one operand in one stage
-        static constexpr int NLW      = OP_BYTES / 4096; // direct loads (1 KiB) per wave, operand and K tile
+        static constexpr int OP_BYTES = BK * ROWS * ES; // one operand in one stage
+        static constexpr int NLW      = WK ? OP_BYTES / 1024 : OP_BYTES / 4096; // direct loads (1 KiB) per wave, operand and K tile
         static constexpr int STAGE_BYTES = 2 * OP_BYTES;
         static constexpr int RING        = NS * STAGE_BYTES;
-        static constexpr int SPARE       = RING; // NLW KiB per wave: where loads beyond the K range land
-        static constexpr int LDS_BYTES   = RING + 4 * NLW * 1024;
-        static_assert(OP_BYTES % 4096 == 0 && NLW >= 1, "every wave loads whole KiB of an operand stage");
+        static constexpr int RINGS       = WK ? 4 : 1;
+        static constexpr int SPARE       = RINGS * RING; // NLW KiB per wave: where loads beyond the K range land
+        static constexpr int LDS_BYTES   = SPARE + 4 * NLW * 1024;
+        static_assert(OP_BYTES % (WK ? 1024 : 4096) == 0 && NLW >= 1, "every wave loads whole KiB of an operand stage");
         static_assert(std::is_same<typename Tr::S, typename Tr::E>::value, "a direct load cannot convert");
         static_assert(NS >= 4 && NS % 2 == 0 && (NS - 1) * 2 * NLW < 64, "the wait counts must fit vmcnt");
+        static_assert(!WK || RING >= (32 / Tr::TILE) * (32 / Tr::TILE) * Tr::NREG * 64 * (int)sizeof(typename Tr::O),
+                      "a wave's partial tile is handed over in its own ring");
         static_assert(LDS_BYTES <= 160 * 1024, "LDS of one CU");
     };
 
-    template <typename Tr, int BK, int NS>
+    __device__ __forceinline__ float   wd_add(float x, float y) { return __fadd_rn(x, y); }
+    __device__ __forceinline__ double  wd_add(double x, double y) { return __dadd_rn(x, y); }
+    __device__ __forceinline__ float2  wd_add(float2 x, float2 y) { return make_float2(__fadd_rn(x.x, y.x), __fadd_rn(x.y, y.y)); }
+    __device__ __forceinline__ double2 wd_add(double2 x, double2 y) { return make_double2(__dadd_rn(x.x, y.x), __dadd_rn(x.y, y.y)); }
+
+    // Tile t + 1 has landed when only the loads of the N / LPT tiles after it are outstanding.  With a common
+    // ring the barrier behind the wait shows it to every wave, and says that every wave has tile t in
+    // registers; a wave with a ring of its own waits for its own LDS reads of tile t instead, before it lets
+    // tile t + NS be written over them.
+    template <bool WK, int N>
+    __device__ __forceinline__ void wd_hand_over()
+    {
+        if(WK)
+        {
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(N) & ~0x0F00); // ... and lgkmcnt(0)
+            asm volatile("" : : : "memory");
+        }
+        else
+        {
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(N));
+            w_lds_barrier();
+        }
+    }
+
+    template <typename Tr, int BK, int NS, bool WK>
     __global__ void __launch_bounds__(256, 2) contract_wd_kernel(const KArgs a)
     {
-        typedef WdGeom<Tr, BK, NS> G;
+        typedef WdGeom<Tr, BK, NS, WK> G;
         typedef typename Tr::S     S;
         constexpr int              TILE = Tr::TILE;
         constexpr int              TP = 32 / TILE, TQ = 32 / TILE;
@@ -83,8 +115,9 @@ namespace hiptk
         const int tid  = threadIdx.x;
         const int lane = tid & 63;
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-        const int wp   = wave >> 1;
-        const int wq   = wave & 1;
+        const int wp   = WK ? 0 : wave >> 1;
+        const int wq   = WK ? 0 : wave & 1;
+        constexpr int ROWS = G::ROWS;
 
         int tp, tq;
         tile_coords(blockIdx.x, a.tiles_p, a.tiles_q, tp, tq);
@@ -92,11 +125,18 @@ namespace hiptk
         // tile that overhangs P or Q reads the padding of the row tables, offset 0, and stores nothing there)
         const int p0 = tp * G::BP, q0 = tq * G::BQ;
 
-        const int kt_begin = blockIdx.z * a.ktiles_per_split;
+        int       kt_begin = blockIdx.z * a.ktiles_per_split;
         int       kt_end   = kt_begin + a.ktiles_per_split;
         const int kt_all   = a.K / BK; // K is a multiple of BK
         if(kt_end > kt_all)
             kt_end = kt_all;
+        if(WK)
+        {
+            // this wave's quarter of the slice (the last waves of a short slice have none)
+            const WdChunk c = wd_wave_chunk(kt_end - kt_begin, wave);
+            kt_begin += c.first;
+            kt_end = kt_begin + c.count;
+        }
         const int nt = kt_end - kt_begin;
 
         // this lane's 16 bytes of each of its loads, as byte offsets from the tile's k origin
@@ -104,7 +144,7 @@ namespace hiptk
 #pragma unroll
         for(int i = 0; i < NLW; i++)
         {
-            const HdSlot sl = wd_slot<G::V>((wave * NLW + i) * 64 + lane);
+            const HdSlot sl = wd_slot<G::V, ROWS>(((WK ? 0 : wave * NLW) + i) * 64 + lane);
             xv[i]           = (uint32_t)ES * ((uint32_t)a.xp[p0 + sl.row] + (uint32_t)sl.k * (uint32_t)a.xk_stride);
             yv[i]           = (uint32_t)ES * ((uint32_t)a.yq[q0 + sl.row] + (uint32_t)sl.k * (uint32_t)a.yk_stride);
         }
@@ -120,7 +160,9 @@ namespace hiptk
 
         typedef unsigned char __attribute__((address_space(3))) * lds_u8_ptr;
         const uint32_t lds0   = (uint32_t)(uintptr_t)(lds_u8_ptr)lds_raw; // LDS byte address of the ring
-        const uint32_t wdx    = lds0 + (uint32_t)wave * (NLW * 1024u); // this wave's share of an X stage
+        // this wave's share of an X stage of the common ring, or its own ring
+        const uint32_t wdx    = lds0 + (uint32_t)wave * (WK ? (uint32_t)G::RING : NLW * 1024u);
+        const unsigned char* const ring = lds_raw + (WK ? wave * G::RING : 0);
         const uint32_t wdy    = wdx + G::OP_BYTES;
         const uint32_t wspare = lds0 + G::SPARE + (uint32_t)wave * (NLW * 1024u);
 
@@ -157,8 +199,8 @@ namespace hiptk
 
         const int row   = lane & (TILE - 1);
         const int kslot = Tr::kslot(lane);
-        const int xfo   = kslot * 64 + wp * 32 + row;
-        const int yfo   = kslot * 64 + wq * 32 + row;
+        const int xfo   = kslot * ROWS + wp * 32 + row;
+        const int yfo   = kslot * ROWS + wq * 32 + row;
 
         // This wave's operands of one K tile, in registers: tile t + 1 is read from LDS while tile t
         // is multiplied, so that a wave alone on its SIMD does not wait for LDS either.
@@ -170,14 +212,14 @@ namespace hiptk
         // the operands of k-step ks of the tile in ring stage ST
         auto read_k = [&](auto st_c, Frags& f, int ks) {
             constexpr int ST = decltype(st_c)::value;
-            const S*      lx = (const S*)(lds_raw + ST * G::STAGE_BYTES);
-            const S*      ly = (const S*)(lds_raw + ST * G::STAGE_BYTES + G::OP_BYTES);
+            const S*      lx = (const S*)(ring + ST * G::STAGE_BYTES);
+            const S*      ly = (const S*)(ring + ST * G::STAGE_BYTES + G::OP_BYTES);
 #pragma unroll
             for(int i = 0; i < TP; i++)
-                f.x[ks][i] = lx[xfo + ks * Tr::KM * 64 + i * TILE];
+                f.x[ks][i] = lx[xfo + ks * Tr::KM * ROWS + i * TILE];
 #pragma unroll
             for(int j = 0; j < TQ; j++)
-                f.y[ks][j] = ly[yfo + ks * Tr::KM * 64 + j * TILE];
+                f.y[ks][j] = ly[yfo + ks * Tr::KM * ROWS + j * TILE];
         };
         auto read_tile = [&](auto st_c, Frags& f) {
 #pragma unroll
@@ -212,10 +254,7 @@ namespace hiptk
             Frags&        nxt = fr[(ST + 1) & 1];
             mma_k(cur, 0);
             __builtin_amdgcn_sched_barrier(0);
-            // tile t + 1 has landed when only the loads of the NS - 2 tiles after it are outstanding;
-            // behind the barrier every wave sees it, and every wave has tile t in registers
-            __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 2) * LPT));
-            w_lds_barrier();
+            wd_hand_over<WK, (NS - 2) * LPT>();
             issue(st_c); // tile t + NS, into tile t's stage
             // (behind the slice's last tile these read a stage nothing was loaded into, for nobody)
             if constexpr(KS == 1)
@@ -236,8 +275,7 @@ namespace hiptk
         if(nt > 0)
         {
             wd_static_for<NS>(issue); // tiles 0 .. NS - 1
-            __builtin_amdgcn_s_waitcnt(waitcnt_vm((NS - 1) * LPT));
-            w_lds_barrier();
+            wd_hand_over<WK, (NS - 1) * LPT>();
             read_tile(std::integral_constant<int, 0>{}, fr[0]);
             while(t + NS <= nt)
                 wd_static_for<NS>(step);
@@ -246,18 +284,57 @@ namespace hiptk
                     step(i_c);
             });
         }
-        epilogue_w<Tr, TP, TQ>(a, acc, p0 + wp * 32, q0 + wq * 32 + Tr::q_of(lane), p0, q0, lane);
-        // the loads beyond the K range (into the spare KiB) must not outlive the workgroup's LDS
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        if constexpr(WK)
+        {
+            // The four partial tiles are added in wave order (the order of split-K slices) by wave 0, which
+            // then stores the tile: a wave's ring is its own again once its last loads have landed.
+            typedef typename Tr::O O;
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0) & ~0x0F00);
+            asm volatile("" : : : "memory");
+            if(wave != 0)
+            {
+                O* mine = (O*)(lds_raw + wave * G::RING);
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+#pragma unroll
+                    for(int j = 0; j < TQ; j++)
+#pragma unroll
+                        for(int r = 0; r < Tr::NREG; r++)
+                            mine[((i * TQ + j) * Tr::NREG + r) * 64 + lane] = Tr::get(acc[i][j], r);
+            }
+            w_lds_barrier();
+            if(wave != 0)
+                return;
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+#pragma unroll
+                    for(int r = 0; r < Tr::NREG; r++)
+                    {
+                        O sum = Tr::get(acc[i][j], r);
+#pragma unroll
+                        for(int w = 1; w < 4; w++)
+                            sum = wd_add(sum, ((const O*)(lds_raw + w * G::RING))[((i * TQ + j) * Tr::NREG + r) * 64 + lane]);
+                        Tr::put(acc[i][j], r, sum);
+                    }
+            epilogue_w<Tr, TP, TQ>(a, acc, p0, q0 + Tr::q_of(lane), p0, q0, lane);
+        }
+        else
+        {
+            epilogue_w<Tr, TP, TQ>(a, acc, p0 + wp * 32, q0 + wq * 32 + Tr::q_of(lane), p0, q0, lane);
+            // the loads beyond the K range (into the spare KiB) must not outlive the workgroup's LDS
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+        }
     }
 
-    template <typename Tr, int BK, int NS>
+    template <typename Tr, int BK, int NS, bool WK>
     int launch_wd(const KArgs& a, hipStream_t stream)
     {
-        typedef WdGeom<Tr, BK, NS> G;
+        typedef WdGeom<Tr, BK, NS, WK> G;
         if(a.K < BK || a.K % BK != 0 || a.shift_p || a.shift_q)
             return (int)hipErrorInvalidValue;
-        auto                    kern = contract_wd_kernel<Tr, BK, NS>;
+        auto                    kern = contract_wd_kernel<Tr, BK, NS, WK>;
         static const hipError_t attr = hipFuncSetAttribute(
             (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
         if(attr != hipSuccess)
@@ -275,6 +352,15 @@ namespace hiptk
     {                                                                                               \
         hiptk::TR::CLS, ID, hiptk::TR::VMAX == 1, hiptk::TR::VMAX == 1, hiptk::TR::VMAX,            \
             hiptk::TR::VMAX, 1, 64, 64, BK, 256,                                                    \
-            hiptk::WdGeom<hiptk::TR, BK, NS>::LDS_BYTES, #TR "_64x64x" #BK "_direct" #NS,        \
-            &hiptk::launch_wd<hiptk::TR, BK, NS>, BK                                                  \
+            hiptk::WdGeom<hiptk::TR, BK, NS, false>::LDS_BYTES, #TR "_64x64x" #BK "_direct" #NS,\
+            &hiptk::launch_wd<hiptk::TR, BK, NS, false>, BK                                         \
+    }
+
+// ... and of the 32 x 32 tile whose four waves split the K range between them.
+#define HIPTK_WK_ENTRY(TR, ID, BK, NS)                                                              \
+    {                                                                                               \
+        hiptk::TR::CLS, ID, hiptk::TR::VMAX == 1, hiptk::TR::VMAX == 1, hiptk::TR::VMAX,            \
+            hiptk::TR::VMAX, 1, 32, 32, BK, 256,                                                    \
+            hiptk::WdGeom<hiptk::TR, BK, NS, true>::LDS_BYTES, #TR "_32x32x" #BK "_direct" #NS "k4", \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, true>, BK                                          \
     }

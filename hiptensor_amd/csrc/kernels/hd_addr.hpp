@@ -65,17 +65,32 @@ namespace hiptk
         return ko + bk < klast ? ko + bk : klast;
     }
 
-    // ... their operand stages are tile[k][64 rows] of elements of 16 / V bytes, unpadded and
+    // ... their operand stages are tile[k][ROWS rows] of elements of 16 / V bytes, unpadded and
     // unswizzled (one element per lane and MFMA operand: consecutive lanes read consecutive rows):
     // the 16-byte slot s holds the V rows from `row` on at `k`.
-    template <int V>
+    template <int V, int ROWS>
     HIPTK_HD_FN HdSlot wd_slot(int s)
     {
         HdSlot        o;
-        constexpr int cpr = 64 / V;
+        constexpr int cpr = ROWS / V;
         o.k               = s / cpr;
         o.row             = V * (s % cpr);
         return o;
+    }
+
+    // ... and where the four waves of a workgroup split a slice of n K tiles between them: wave w takes
+    // `count` tiles from `first` on (none, for the last waves of a short slice).
+    struct WdChunk
+    {
+        int first, count;
+    };
+    HIPTK_HD_FN WdChunk wd_wave_chunk(int n, int w)
+    {
+        const int per = (n + 3) / 4;
+        WdChunk   c;
+        c.first = w * per < n ? w * per : n;
+        c.count = n - c.first < per ? n - c.first : per;
+        return c;
     }
 
     template <bool KF, int BR>

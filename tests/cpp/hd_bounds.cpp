@@ -28,6 +28,8 @@ using hiptk::HdSlice;
 using hiptk::HdSlot;
 using hiptk::wd_next_origin;
 using hiptk::wd_slot;
+using hiptk::wd_wave_chunk;
+using hiptk::WdChunk;
 
 static int g_fail = 0;
 #define CHECK(cond, ...)                                                  \
@@ -217,30 +219,32 @@ static long check_tile_size(const Case& c, const GemmView& v)
     return walked;
 }
 
-// ---- the 32/64-bit kernels: V rows per 16-byte vector, K tiles of BK, NLW loads per wave and operand ----
-template <int V>
+// ---- the 32/64-bit kernels: V rows per 16-byte vector, K tiles of BK, NLW loads per wave and operand; tiles of
+// ROWS x ROWS whose four waves share the stages (ROWS = 64), or load all of them each (ROWS = 32: the waves split K) ----
+template <int V, int ROWS>
 static void check_wide_operand(const char* what, const Case& c, const GemmView& v, bool is_x, int r0, int BK, int NLW,
                                const std::vector<int>& origins)
 {
+    constexpr bool WK = ROWS == 32;
     const std::vector<int32_t>& rtab    = is_x ? v.xp : v.yq;
     const std::vector<int32_t>& ktab    = is_x ? v.xk : v.yk;
     const int64_t               kstride = is_x ? v.xk_stride : v.yk_stride;
     const int64_t               nrows   = is_x ? v.P : v.Q;
     const int64_t               span    = (is_x != v.swapped) ? v.spanA : v.spanB;
     const int64_t               es      = 16 / V;
-    std::vector<int>            seen((size_t)BK * 64 / V, 0);
-    CHECK(4 * NLW * 64 == BK * 64 / V, "%s %s: %d loads do not tile a stage", c.name.c_str(), what, 4 * NLW * 64);
+    std::vector<int>            seen((size_t)BK * ROWS / V, 0);
+    CHECK((WK ? 1 : 4) * NLW * 64 == BK * ROWS / V, "%s %s: %d loads do not tile a stage", c.name.c_str(), what, NLW * 64);
     for(int wave = 0; wave < 4; wave++)
         for(int lane = 0; lane < 64; lane++)
             for(int i = 0; i < NLW; i++)
             {
-                const int    s  = (wave * NLW + i) * 64 + lane;
-                const HdSlot sl = wd_slot<V>(s);
-                CHECK(sl.row >= 0 && sl.row + V <= 64 && sl.row % V == 0 && sl.k >= 0 && sl.k < BK, "%s %s slot %d -> row %d k %d", c.name.c_str(),
+                const int    s  = ((WK ? 0 : wave * NLW) + i) * 64 + lane;
+                const HdSlot sl = wd_slot<V, ROWS>(s);
+                CHECK(sl.row >= 0 && sl.row + V <= ROWS && sl.row % V == 0 && sl.k >= 0 && sl.k < BK, "%s %s slot %d -> row %d k %d", c.name.c_str(),
                       what, s, sl.row, sl.k);
-                // the LDS bytes 16 s .. 16 s + 15 of a stage laid out [k][64 rows] are exactly these V rows at this k
-                CHECK((int64_t)16 * s == ((int64_t)sl.k * 64 + sl.row) * es, "%s %s slot %d is not where the readers look", c.name.c_str(), what, s);
-                seen[(size_t)(sl.k * (64 / V) + sl.row / V)]++;
+                // the LDS bytes 16 s .. 16 s + 15 of a stage laid out [k][ROWS] are exactly these V rows at this k
+                CHECK((int64_t)16 * s == ((int64_t)sl.k * ROWS + sl.row) * es, "%s %s slot %d is not where the readers look", c.name.c_str(), what, s);
+                seen[(size_t)(sl.k * (ROWS / V) + sl.row / V)]++;
                 CHECK((size_t)(r0 + sl.row) < rtab.size(), "%s %s row table index %d of %zu", c.name.c_str(), what, r0 + sl.row, rtab.size());
                 const int64_t rowpart = rtab[(size_t)(r0 + sl.row)];
                 for(int j = 1; j < V && r0 + sl.row + j < nrows; j++)
@@ -263,15 +267,16 @@ static void check_wide_operand(const char* what, const Case& c, const GemmView& 
                 }
             }
     for(size_t i = 0; i < seen.size(); i++)
-        CHECK(seen[i] == 1, "%s %s vector %zu filled %d times", c.name.c_str(), what, i, seen[i]);
+        CHECK(seen[i] == (WK ? 4 : 1), "%s %s vector %zu filled %d times", c.name.c_str(), what, i, seen[i]);
 }
 
-template <int V>
+template <int V, int ROWS>
 static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
 {
+    constexpr bool WK = ROWS == 32;
     long      walked = 0;
     const int K      = (int)v.K;
-    const int tiles_p = (int)((v.P + 63) / 64), tiles_q = (int)((v.Q + 63) / 64);
+    const int tiles_p = (int)((v.P + ROWS - 1) / ROWS), tiles_q = (int)((v.Q + ROWS - 1) / ROWS);
     const int ktiles  = K / BK;
     CHECK(K % BK == 0 && K >= BK, "%s K %d offered to K tiles of %d", c.name.c_str(), K, BK);
     for(int want = 1; want <= 7; want++)
@@ -282,11 +287,21 @@ static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
         std::vector<int> covered((size_t)K, 0);
         std::vector<int> origins;
         for(int z = 0; z < split; z++)
-        {
-            // as the kernel: the slice's tiles, then repeats of its last one (a ring of up to 8 stages)
-            const int kt_begin = z * per;
-            const int nt       = std::min(kt_begin + per, ktiles) - kt_begin;
+          for(int wave = 0; wave < (WK ? 4 : 1); wave++)
+          {
+            // as the kernel: the slice's (or, of it, the wave's) tiles, then repeats of the last one (a ring of up to 8 stages)
+            int kt_begin = z * per;
+            int nt       = std::min(kt_begin + per, ktiles) - kt_begin;
             CHECK(nt >= 1, "%s K %d slice %d/%d is empty", c.name.c_str(), K, z, split);
+            if(WK)
+            {
+                const WdChunk ch = wd_wave_chunk(nt, wave);
+                CHECK(ch.first >= 0 && ch.count >= 0 && ch.first + ch.count <= nt, "%s wave %d chunk %d + %d of %d", c.name.c_str(), wave, ch.first, ch.count, nt);
+                kt_begin += ch.first;
+                nt = ch.count;
+                if(nt == 0)
+                    continue; // the kernel requests nothing then
+            }
             const int klast = (kt_begin + nt - 1) * BK;
             int       ko    = kt_begin * BK;
             for(int u = 0; u < nt + 12; u++)
@@ -303,7 +318,7 @@ static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
                 origins.push_back(ko);
                 ko = wd_next_origin(ko, klast, BK);
             }
-        }
+          }
         for(int k = 0; k < K; k++)
             CHECK(covered[(size_t)k] == 1, "%s K %d split %d: k %d multiplied %d times", c.name.c_str(), K, split, k, covered[(size_t)k]);
         std::sort(origins.begin(), origins.end());
@@ -311,9 +326,9 @@ static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
         for(int tp : {0, tiles_p / 2, tiles_p - 1})
             for(int tq : {0, tiles_q / 2, tiles_q - 1})
             {
-                check_wide_operand<V>("X", c, v, true, tp * 64, BK, NLW, origins);
-                check_wide_operand<V>("Y", c, v, false, tq * 64, BK, NLW, origins);
-                walked += (long)origins.size() * 2 * BK * 64 / V;
+                check_wide_operand<V, ROWS>("X", c, v, true, tp * ROWS, BK, NLW, origins);
+                check_wide_operand<V, ROWS>("Y", c, v, false, tq * ROWS, BK, NLW, origins);
+                walked += (long)origins.size() * 2 * BK * ROWS / V;
             }
         if(want > 1 && split == 1)
             break;
@@ -324,7 +339,7 @@ static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
 struct WideTile
 {
     const char* type;
-    int         dtype, compute, elem_bytes, tile, bk;
+    int         dtype, compute, elem_bytes, tile, bk, rows;
 };
 
 int main()
@@ -428,8 +443,8 @@ int main()
     rank4("k8_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 40, 9, 24, 13, 8, 1);
     rank4("k24_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 42, 9, 25, 13, 8, 3);
     rank4("big_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 8192, 16, 64, 1, 64, 64);
-    const WideTile wide[] = {{"f32", 0, 4, 4, 2, 16}, {"f64", 1, 16, 8, 2, 8},
-                             {"c32", 4, 2048, 8, 2, 8}};
+    const WideTile wide[] = {{"f32", 0, 4, 4, 2, 16, 64}, {"f64", 1, 16, 8, 2, 8, 64}, {"c32", 4, 2048, 8, 2, 8, 64},
+                             {"f32", 0, 4, 4, 3, 16, 32}, {"f64", 1, 16, 8, 3, 8, 32}, {"c32", 4, 2048, 8, 3, 8, 32}};
     int offered_wide = 0, refused_big = 0;
     for(const WideTile& w : wide)
         for(const Case& c : cases)
@@ -470,11 +485,14 @@ int main()
                       && !v.shift_q,
                   "%s %s offered outside its restrictions", w.type, c.name.c_str());
             offered_wide++;
-            const int nlw = w.bk * 64 * w.elem_bytes / 4096;
-            walked += V == 4 ? check_wide_tile<4>(c, v, w.bk, nlw) : check_wide_tile<2>(c, v, w.bk, nlw);
+            const int nlw = w.bk * w.rows * w.elem_bytes / (w.rows == 32 ? 1024 : 4096);
+            if(w.rows == 64)
+                walked += V == 4 ? check_wide_tile<4, 64>(c, v, w.bk, nlw) : check_wide_tile<2, 64>(c, v, w.bk, nlw);
+            else
+                walked += V == 4 ? check_wide_tile<4, 32>(c, v, w.bk, nlw) : check_wide_tile<2, 32>(c, v, w.bk, nlw);
         }
     g_dtype = 2;
-    CHECK(offered_wide >= 30, "only %d (case, type, tile) triples were offered a 32/64-bit direct-load kernel", offered_wide);
+    CHECK(offered_wide >= 60, "only %d (case, type, tile) triples were offered a 32/64-bit direct-load kernel", offered_wide);
     CHECK(refused_big >= 2, "the tensor past 2^32 bytes was not exercised (%d)", refused_big);
     std::printf("%s: %d + %d problems x tiles, %ld requests walked, %d failures\n", g_fail ? "FAILED" : "ok", offered, offered_wide, walked,
                 g_fail);
