@@ -79,6 +79,89 @@ namespace hiptk
     __device__ __forceinline__ float2  wd_add(float2 x, float2 y) { return make_float2(__fadd_rn(x.x, y.x), __fadd_rn(x.y, y.y)); }
     __device__ __forceinline__ double2 wd_add(double2 x, double2 y) { return make_double2(__dadd_rn(x.x, y.x), __dadd_rn(x.y, y.y)); }
 
+    // The epilogue of these kernels in two halves: `fetch`, before the main loop, looks up the wave tile's
+    // C / D offsets and requests its C elements; `store`, after it, writes D = alpha * acc (+ beta * C).
+    // contract_w.hpp's epilogue_w fetches four accumulator rows at a time behind the stores of the four
+    // before (D may alias C), one memory latency per batch, which other workgroups on the CU cover there;
+    // here a workgroup may be alone, and the registers for all of a lane's C elements are free.
+    // (Reading C early is safe when D aliases it: every element is read and written by the same lane,
+    // these kernels never move a tile back over a neighbour's rows.)
+    template <typename Tr, int TP, int TQ>
+    struct WdEpilogue
+    {
+        typedef typename Tr::E E;
+        uint32_t               dpo[TP][Tr::NREG], dqo[TQ];
+        uint32_t               pmask, qmask;
+        E                      cv[TP][Tr::NREG][TQ];
+
+        __device__ __forceinline__ void fetch(const KArgs& a, int pw, int qw, int p_own, int q_own, int lane)
+        {
+            constexpr int TILE = Tr::TILE;
+            static_assert(TP * Tr::NREG <= 32 && TQ <= 32, "one bit per row and column");
+            const E*   Cp  = (const E*)a.C;
+            const bool bil = a.bilinear != 0;
+            const bool aff = a.cd_affine != 0;
+            // A lane outside the extents fetches element (0, 0) instead, a valid address, and stores nothing.
+            uint32_t cqo[TQ], cpo[TP][Tr::NREG];
+            pmask = 0;
+            qmask = 0;
+#pragma unroll
+            for(int j = 0; j < TQ; j++)
+            {
+                const int  q  = qw + j * TILE;
+                const bool ok = q >= q_own && q < a.Q;
+                qmask |= ok ? 1u << j : 0u;
+                const int qv = ok ? q : 0;
+                dqo[j]       = aff ? (uint32_t)qv * (uint32_t)a.dq_stride : (uint32_t)a.dq[qv];
+                cqo[j]       = !bil ? 0u : aff ? (uint32_t)qv * (uint32_t)a.cq_stride : (uint32_t)a.cq[qv];
+            }
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+#pragma unroll
+                for(int r = 0; r < Tr::NREG; r++)
+                {
+                    const int  p  = pw + i * TILE + Tr::p_of(r, lane);
+                    const bool ok = p >= p_own && p < a.P;
+                    pmask |= ok ? 1u << (i * Tr::NREG + r) : 0u;
+                    const int pv = ok ? p : 0;
+                    dpo[i][r]    = aff ? (uint32_t)pv * (uint32_t)a.dp_stride : (uint32_t)a.dp[pv];
+                    cpo[i][r]    = !bil ? 0u : aff ? (uint32_t)pv * (uint32_t)a.cp_stride : (uint32_t)a.cp[pv];
+                }
+            if(bil)
+            {
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+#pragma unroll
+                    for(int r = 0; r < Tr::NREG; r++)
+#pragma unroll
+                        for(int j = 0; j < TQ; j++)
+                            cv[i][r][j] = Cp[cpo[i][r] + cqo[j]];
+            }
+        }
+
+        __device__ __forceinline__ void store(const KArgs& a, typename Tr::Acc (&acc)[TP][TQ])
+        {
+            E*         Dp  = (E*)a.D;
+            const bool bil = a.bilinear != 0;
+#pragma unroll
+            for(int i = 0; i < TP; i++)
+#pragma unroll
+                for(int r = 0; r < Tr::NREG; r++)
+#pragma unroll
+                    for(int j = 0; j < TQ; j++)
+                    {
+                        if(((pmask >> (i * Tr::NREG + r)) & 1u) && ((qmask >> j) & 1u))
+                        {
+                            const E val = Tr::finish(Tr::get(acc[i][j], r), a.alpha, a.beta, bil, &cv[i][r][j]);
+                            if constexpr(std::is_arithmetic<E>::value)
+                                __builtin_nontemporal_store(val, Dp + (dpo[i][r] + dqo[j]));
+                            else
+                                Dp[dpo[i][r] + dqo[j]] = val;
+                        }
+                    }
+        }
+    };
+
     // Tile t + 1 has landed when only the loads of the N / LPT tiles after it are outstanding.  With a common
     // ring the barrier behind the wait shows it to every wave, and says that every wave has tile t in
     // registers; a wave with a ring of its own waits for its own LDS reads of tile t instead, before it lets
@@ -189,6 +272,16 @@ namespace hiptk
             xsrc = (const char*)a.X + (uint64_t)((uint32_t)ko * xkb);
             ysrc = (const char*)a.Y + (uint64_t)((uint32_t)ko * ykb);
         };
+
+        // C and the C / D offsets of the wave tile this wave will store (with waves that split K: wave 0,
+        // all of the tile), unless the launch is a split-K slice, which stores partial sums
+        WdEpilogue<Tr, TP, TQ> epi;
+        const bool             whole_k = a.split_k == 1;
+        const bool             storer  = !WK || wave == 0;
+        if(whole_k && storer)
+            epi.fetch(a, p0 + wp * 32, q0 + wq * 32 + Tr::q_of(lane), p0, q0, lane);
+        // (requested before the first operand tile: loads return in order, so they are back before it)
+        __builtin_amdgcn_sched_barrier(0);
 
         typename Tr::Acc acc[TP][TQ];
 #pragma unroll
@@ -318,11 +411,17 @@ namespace hiptk
                             sum = wd_add(sum, ((const O*)(lds_raw + w * G::RING))[((i * TQ + j) * Tr::NREG + r) * 64 + lane]);
                         Tr::put(acc[i][j], r, sum);
                     }
-            epilogue_w<Tr, TP, TQ>(a, acc, p0, q0 + Tr::q_of(lane), p0, q0, lane);
+            if(whole_k)
+                epi.store(a, acc);
+            else
+                epilogue_w<Tr, TP, TQ>(a, acc, p0, q0 + Tr::q_of(lane), p0, q0, lane);
         }
         else
         {
-            epilogue_w<Tr, TP, TQ>(a, acc, p0 + wp * 32, q0 + wq * 32 + Tr::q_of(lane), p0, q0, lane);
+            if(whole_k)
+                epi.store(a, acc);
+            else
+                epilogue_w<Tr, TP, TQ>(a, acc, p0 + wp * 32, q0 + wq * 32 + Tr::q_of(lane), p0, q0, lane);
             // the loads beyond the K range (into the spare KiB) must not outlive the workgroup's LDS
             __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
         }
