@@ -8,7 +8,7 @@ alone, and doubling alpha doubles the result exactly.  Comparisons go through
 cases.assert_parity (relative error within 1e-5 f32 / c32, 1e-2 f16 / bf16, 1e-12 f64, and
 the reference harness's element-wise metric within its own bound).  Configurations 1 and 4 (f32
 accumulation) are also held against a result accumulated in f64 on the host: on the reference
-harness's element-wise metric the GPU must be no further from it than 2 x the CPU oracle is,
+harness's element-wise metric the GPU must be no further from it than 1.5 x the CPU oracle is,
 which is what "as accurate as the reference's CPU path" means where that path itself is 2e-5 away.
 """
 import numpy as np
@@ -63,9 +63,9 @@ def _full(handle, oracle_mod, w, against_f64=False):
         e_gpu, e_cpu = _elementwise_vs(ref64, to64(got)), _elementwise_vs(ref64, to64(exp))
         print(f"  element-wise distance from the f64-accumulated result: GPU {e_gpu:.3e}, CPU oracle {e_cpu:.3e}", flush=True)
         # (both accumulate in the element type; the order differs.  One pass over K = 512 in MFMA order reads
-        # 3.5e-5 on the complex f32 configuration, two split-K slices 2.9e-5, four 1.6e-5, the CPU order 2.2e-5:
-        # the bound leaves room for the order and none for a narrower accumulator, which is off by 1000 x)
-        assert e_gpu <= 2.0 * e_cpu + 1e-9, f"{w['name']}: GPU {e_gpu:.3e} is further from the f64 result than 2 x the CPU path ({e_cpu:.3e})"
+        # 3.0e-5 on the complex f32 configuration, two split-K slices 1.9e-5, the CPU order 2.2e-5: the bound
+        # leaves room for the order and none for a narrower accumulator, which is off by 1000 x)
+        assert e_gpu <= 1.5 * e_cpu + 1e-9, f"{w['name']}: GPU {e_gpu:.3e} is further from the f64 result than 1.5 x the CPU path ({e_cpu:.3e})"
 
 
 def test_config1_f32(gpu_handle, oracle_mod):
