@@ -154,7 +154,8 @@ namespace hipta
             // (128 x 128 on 4096 x 4096 x 512, four tiles per CU: complex f32 535 us, f32 140.5 us; complex f32 on
             // 64 x 64: 1024^2 x 512 in one pass 50.7 us, 3072 x 1024 x 1024 203.6 us)
             case HIPTK_C32: return area >= 16384 ? TileRate{0.84, 0.86} : TileRate{0.62, 0.82};
-            default: return area >= 16384 ? TileRate{0.73, 0.85} : TileRate{0.36, 0.66};
+            // (f32 128 x 128, one tile per CU: 1920^2 x 768 66 us, 2048^2 x 1024 85 us)
+            default: return area >= 16384 ? TileRate{0.66, 0.85} : TileRate{0.36, 0.66};
             }
         }
     }
@@ -203,20 +204,26 @@ namespace hipta
         {
             // The 32/64-bit 64 x 64 tiles whose operand tiles are loaded straight into LDS (four waves, two
             // workgroups per CU): slopes of 1024 x 1024 x K (one workgroup per CU) and 2048 x 2048 x K scans
+            const bool big = s.bp * s.bq >= 4096; // 64 x 64, or 32 x 32 with the waves splitting K
+            const bool kf  = v.x_kfast && v.y_kfast; // 16-byte vectors of k: shorter runs in memory
             switch(v.cls)
             {
-            // (the 32 x 32 tile whose four waves split K reads twice the operand bytes per flop: 1024^2 x 2048 f32
-            // 41.8 against 38.1 us, 512 x 2048 x 4096 78.6 against 68.8; level with the 64 x 64 tile in f64 and c32)
-            case HIPTK_F32: r = s.bp * s.bq >= 4096 ? TileRate{0.81, 0.89} : TileRate{0.65, 0.70}; break;
-            case HIPTK_F64: r = TileRate{0.82, 0.90}; break;
-            case HIPTK_C32: r = TileRate{0.90, 0.91}; break;
+            // (the 32 x 32 tile reads twice the operand bytes per flop: 1024^2 x 2048 f32 41.8 against 38.1 us,
+            // 512 x 2048 x 4096 78.6 against 68.8; level with the 64 x 64 tile in f64 and c32 on row-contiguous
+            // operands.  k-contiguous operands, 2048^2 x 1024 on 64 x 64: f32 74.8 us, f64 132.2, c32 244.3; on
+            // 32 x 32 a wave's runs are 64 bytes a row and K tile: 1024^2 x 2048 f64 125 against 70.7 us)
+            case HIPTK_F32: r = big ? (kf ? TileRate{0.75, 0.78} : TileRate{0.81, 0.89}) : (kf ? TileRate{0.55, 0.60} : TileRate{0.65, 0.70}); break;
+            case HIPTK_F64: r = big ? (kf ? TileRate{0.80, 0.84} : TileRate{0.82, 0.90}) : (kf ? TileRate{0.45, 0.50} : TileRate{0.82, 0.90}); break;
+            case HIPTK_C32: r = big ? (kf ? TileRate{0.88, 0.90} : TileRate{0.90, 0.91}) : (kf ? TileRate{0.85, 0.88} : TileRate{0.90, 0.91}); break;
             default: break;
             }
             // ... whose prologue (tables, then the first tiles' flight) and epilogue nothing overlaps when a
             // CU runs one or two rounds of them: 2048 x 2048 x K f32 fits 13.9 us + 60.5 us per 1024 of K
             // (256^3 f32: one pass 9.2-9.8 us, four slices of four K tiles 7.8-8.1 us with the reduction: a
-            // slice shorter than the ring has less in flight to wait for)
-            round_extra_us = 2.0 * std::min(1.0, kper / s.bk / 16.0);
+            // slice shorter than the ring has less in flight to wait for); the 32 x 32 tile adds its partial
+            // tiles through LDS (640^2 x 64 f32: 8.4 us against 6.3 on 64 x 64 tiles)
+            // (k-contiguous: 8.6 against 6.5 us)
+            round_extra_us = 2.0 * std::min(1.0, kper / s.bk / 16.0) + (big ? 0.0 : kf ? 2.5 : 1.0);
         }
         if(class_max_vec(v.cls) > 1)
         {

@@ -52,7 +52,7 @@ namespace hiptk
     // multiplies all of it over its own quarter of the K range out of a ring of its own (no barrier in the
     // loop), and the four partial tiles are added through LDS at the end: for outputs too small to fill the
     // device with 64 x 64 tiles, in one launch.
-    template <typename Tr, int BK, int NS, bool WK>
+    template <typename Tr, int BK, int NS, bool WK, bool KF = false>
     struct WdGeom
     {
         static constexpr int ROWS = WK ? 32 : 64; // rows of an operand tile
@@ -72,6 +72,7 @@ namespace hiptk
         static_assert(!WK || RING >= (32 / Tr::TILE) * (32 / Tr::TILE) * Tr::NREG * 64 * (int)sizeof(typename Tr::O),
                       "a wave's partial tile is handed over in its own ring");
         static_assert(LDS_BYTES <= 160 * 1024, "LDS of one CU");
+        static_assert(!KF || (BK / Tr::KM) % V == 0, "a k-contiguous vector feeds whole k-steps");
     };
 
     __device__ __forceinline__ float   wd_add(float x, float y) { return __fadd_rn(x, y); }
@@ -181,10 +182,10 @@ namespace hiptk
         }
     }
 
-    template <typename Tr, int BK, int NS, bool WK>
+    template <typename Tr, int BK, int NS, bool WK, bool KF>
     __global__ void __launch_bounds__(256, 2) contract_wd_kernel(const KArgs a)
     {
-        typedef WdGeom<Tr, BK, NS, WK> G;
+        typedef WdGeom<Tr, BK, NS, WK, KF> G;
         typedef typename Tr::S     S;
         constexpr int              TILE = Tr::TILE;
         constexpr int              TP = 32 / TILE, TQ = 32 / TILE;
@@ -204,8 +205,8 @@ namespace hiptk
 
         int tp, tq;
         tile_coords(blockIdx.x, a.tiles_p, a.tiles_q, tp, tq);
-        // (no tile is moved back: the dispatcher offers this kernel only without shift_p / shift_q; a
-        // tile that overhangs P or Q reads the padding of the row tables, offset 0, and stores nothing there)
+        // (no tile is moved back; a tile that overhangs P or Q reads the padding of the row tables, offset 0,
+        // and stores nothing there)
         const int p0 = tp * G::BP, q0 = tq * G::BQ;
 
         int       kt_begin = blockIdx.z * a.ktiles_per_split;
@@ -227,7 +228,8 @@ namespace hiptk
 #pragma unroll
         for(int i = 0; i < NLW; i++)
         {
-            const HdSlot sl = wd_slot<G::V, ROWS>(((WK ? 0 : wave * NLW) + i) * 64 + lane);
+            const int    s_ = ((WK ? 0 : wave * NLW) + i) * 64 + lane;
+            const HdSlot sl = KF ? wd_slot_kf<G::V, ROWS>(s_) : wd_slot<G::V, ROWS>(s_);
             xv[i]           = (uint32_t)ES * ((uint32_t)a.xp[p0 + sl.row] + (uint32_t)sl.k * (uint32_t)a.xk_stride);
             yv[i]           = (uint32_t)ES * ((uint32_t)a.yq[q0 + sl.row] + (uint32_t)sl.k * (uint32_t)a.yk_stride);
         }
@@ -302,17 +304,48 @@ namespace hiptk
             S x[KS][TP], y[KS][TQ];
         };
         Frags fr[2];
-        // the operands of k-step ks of the tile in ring stage ST
+        // the operands of k-step ks of the tile in ring stage ST (k-contiguous operands: of the V k-steps from
+        // ks on, when ks is the first of them: one 16-byte read per operand row block)
+        struct alignas(16) SVec
+        {
+            S e[G::V];
+        };
         auto read_k = [&](auto st_c, Frags& f, int ks) {
             constexpr int ST = decltype(st_c)::value;
-            const S*      lx = (const S*)(ring + ST * G::STAGE_BYTES);
-            const S*      ly = (const S*)(ring + ST * G::STAGE_BYTES + G::OP_BYTES);
+            if constexpr(KF)
+            {
+                if(ks % G::V != 0)
+                    return;
+                const SVec* lx = (const SVec*)(ring + ST * G::STAGE_BYTES);
+                const SVec* ly = (const SVec*)(ring + ST * G::STAGE_BYTES + G::OP_BYTES);
 #pragma unroll
-            for(int i = 0; i < TP; i++)
-                f.x[ks][i] = lx[xfo + ks * Tr::KM * ROWS + i * TILE];
+                for(int i = 0; i < TP; i++)
+                {
+                    const SVec v = lx[xfo + (ks / G::V) * Tr::KM * ROWS + i * TILE];
 #pragma unroll
-            for(int j = 0; j < TQ; j++)
-                f.y[ks][j] = ly[yfo + ks * Tr::KM * ROWS + j * TILE];
+                    for(int j = 0; j < G::V; j++)
+                        f.x[ks + j][i] = v.e[j];
+                }
+#pragma unroll
+                for(int j2 = 0; j2 < TQ; j2++)
+                {
+                    const SVec v = ly[yfo + (ks / G::V) * Tr::KM * ROWS + j2 * TILE];
+#pragma unroll
+                    for(int j = 0; j < G::V; j++)
+                        f.y[ks + j][j2] = v.e[j];
+                }
+            }
+            else
+            {
+                const S* lx = (const S*)(ring + ST * G::STAGE_BYTES);
+                const S* ly = (const S*)(ring + ST * G::STAGE_BYTES + G::OP_BYTES);
+#pragma unroll
+                for(int i = 0; i < TP; i++)
+                    f.x[ks][i] = lx[xfo + ks * Tr::KM * ROWS + i * TILE];
+#pragma unroll
+                for(int j = 0; j < TQ; j++)
+                    f.y[ks][j] = ly[yfo + ks * Tr::KM * ROWS + j * TILE];
+            }
         };
         auto read_tile = [&](auto st_c, Frags& f) {
 #pragma unroll
@@ -427,13 +460,16 @@ namespace hiptk
         }
     }
 
-    template <typename Tr, int BK, int NS, bool WK>
+    template <typename Tr, int BK, int NS, bool WK, bool KF>
     int launch_wd(const KArgs& a, hipStream_t stream)
     {
-        typedef WdGeom<Tr, BK, NS, WK> G;
-        if(a.K < BK || a.K % BK != 0 || a.shift_p || a.shift_q)
+        typedef WdGeom<Tr, BK, NS, WK, KF> G;
+        // (a tile is never moved back here.  Row-contiguous operands that would need it are not offered this
+        // kernel; with k-contiguous ones the flag can only come from C / D's vectors, which the element-wise
+        // epilogue does not use: an overhanging tile reads the row tables' padding and stores nothing there)
+        if(a.K < BK || a.K % BK != 0 || (!KF && (a.shift_p || a.shift_q)))
             return (int)hipErrorInvalidValue;
-        auto                    kern = contract_wd_kernel<Tr, BK, NS, WK>;
+        auto                    kern = contract_wd_kernel<Tr, BK, NS, WK, KF>;
         static const hipError_t attr = hipFuncSetAttribute(
             (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
         if(attr != hipSuccess)
@@ -452,7 +488,7 @@ namespace hiptk
         hiptk::TR::CLS, ID, hiptk::TR::VMAX == 1, hiptk::TR::VMAX == 1, hiptk::TR::VMAX,            \
             hiptk::TR::VMAX, 1, 64, 64, BK, 256,                                                    \
             hiptk::WdGeom<hiptk::TR, BK, NS, false>::LDS_BYTES, #TR "_64x64x" #BK "_direct" #NS,\
-            &hiptk::launch_wd<hiptk::TR, BK, NS, false>, BK                                         \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, false, false>, BK                                         \
     }
 
 // ... and of the 32 x 32 tile whose four waves split the K range between them.
@@ -461,5 +497,19 @@ namespace hiptk
         hiptk::TR::CLS, ID, hiptk::TR::VMAX == 1, hiptk::TR::VMAX == 1, hiptk::TR::VMAX,            \
             hiptk::TR::VMAX, 1, 32, 32, BK, 256,                                                    \
             hiptk::WdGeom<hiptk::TR, BK, NS, true>::LDS_BYTES, #TR "_32x32x" #BK "_direct" #NS "k4", \
-            &hiptk::launch_wd<hiptk::TR, BK, NS, true>, BK                                          \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, true, false>, BK                                        \
+    }
+
+// ... and of both for operands that are contiguous along k (16-byte vectors of k, one K stride).
+#define HIPTK_WD_ENTRY_KF(TR, ID, BK, NS)                                                           \
+    {                                                                                               \
+        hiptk::TR::CLS, ID, 1, 1, hiptk::TR::VMAX, hiptk::TR::VMAX, 1, 64, 64, BK, 256,             \
+            hiptk::WdGeom<hiptk::TR, BK, NS, false, true>::LDS_BYTES, #TR "_64x64x" #BK "_direct" #NS "kf", \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, false, true>, BK                                   \
+    }
+#define HIPTK_WK_ENTRY_KF(TR, ID, BK, NS)                                                           \
+    {                                                                                               \
+        hiptk::TR::CLS, ID, 1, 1, hiptk::TR::VMAX, hiptk::TR::VMAX, 1, 32, 32, BK, 256,             \
+            hiptk::WdGeom<hiptk::TR, BK, NS, true, true>::LDS_BYTES, #TR "_32x32x" #BK "_direct" #NS "k4kf", \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, true, true>, BK                                    \
     }

@@ -78,6 +78,19 @@ namespace hiptk
         return o;
     }
 
+    // The same kernels for operands that are contiguous along k: a 16-byte vector is V consecutive k of
+    // one row, and a stage is tile[k / V][ROWS rows][V]: slot s holds row `row` from k on.  A lane of the
+    // MFMA's k-slot j then reads one vector for V k-steps: the k-slots of a k-step are V apart in k instead
+    // of adjacent, for both operands alike.
+    template <int V, int ROWS>
+    HIPTK_HD_FN HdSlot wd_slot_kf(int s)
+    {
+        HdSlot o;
+        o.k   = V * (s / ROWS);
+        o.row = s % ROWS;
+        return o;
+    }
+
     // ... and where the four waves of a workgroup split a slice of n K tiles between them: wave w takes
     // `count` tiles from `first` on (none, for the last waves of a short slice).
     struct WdChunk

@@ -28,6 +28,7 @@ using hiptk::HdSlice;
 using hiptk::HdSlot;
 using hiptk::wd_next_origin;
 using hiptk::wd_slot;
+using hiptk::wd_slot_kf;
 using hiptk::wd_wave_chunk;
 using hiptk::WdChunk;
 
@@ -221,7 +222,7 @@ static long check_tile_size(const Case& c, const GemmView& v)
 
 // ---- the 32/64-bit kernels: V rows per 16-byte vector, K tiles of BK, NLW loads per wave and operand; tiles of
 // ROWS x ROWS whose four waves share the stages (ROWS = 64), or load all of them each (ROWS = 32: the waves split K) ----
-template <int V, int ROWS>
+template <int V, int ROWS, bool KF>
 static void check_wide_operand(const char* what, const Case& c, const GemmView& v, bool is_x, int r0, int BK, int NLW,
                                const std::vector<int>& origins)
 {
@@ -239,22 +240,35 @@ static void check_wide_operand(const char* what, const Case& c, const GemmView& 
             for(int i = 0; i < NLW; i++)
             {
                 const int    s  = ((WK ? 0 : wave * NLW) + i) * 64 + lane;
-                const HdSlot sl = wd_slot<V, ROWS>(s);
-                CHECK(sl.row >= 0 && sl.row + V <= ROWS && sl.row % V == 0 && sl.k >= 0 && sl.k < BK, "%s %s slot %d -> row %d k %d", c.name.c_str(),
-                      what, s, sl.row, sl.k);
-                // the LDS bytes 16 s .. 16 s + 15 of a stage laid out [k][ROWS] are exactly these V rows at this k
-                CHECK((int64_t)16 * s == ((int64_t)sl.k * ROWS + sl.row) * es, "%s %s slot %d is not where the readers look", c.name.c_str(), what, s);
-                seen[(size_t)(sl.k * (ROWS / V) + sl.row / V)]++;
+                const HdSlot sl = KF ? wd_slot_kf<V, ROWS>(s) : wd_slot<V, ROWS>(s);
+                if(KF)
+                {
+                    CHECK(sl.row >= 0 && sl.row < ROWS && sl.k >= 0 && sl.k + V <= BK && sl.k % V == 0, "%s %s slot %d -> row %d k %d", c.name.c_str(),
+                          what, s, sl.row, sl.k);
+                    // the LDS bytes 16 s .. 16 s + 15 of a stage laid out [k / V][ROWS][V] are exactly these V k of this row
+                    CHECK((int64_t)16 * s == (((int64_t)sl.k / V) * ROWS + sl.row) * 16, "%s %s slot %d is not where the readers look", c.name.c_str(), what, s);
+                    seen[(size_t)((sl.k / V) * ROWS + sl.row)]++;
+                }
+                else
+                {
+                    CHECK(sl.row >= 0 && sl.row + V <= ROWS && sl.row % V == 0 && sl.k >= 0 && sl.k < BK, "%s %s slot %d -> row %d k %d", c.name.c_str(),
+                          what, s, sl.row, sl.k);
+                    // the LDS bytes 16 s .. 16 s + 15 of a stage laid out [k][ROWS] are exactly these V rows at this k
+                    CHECK((int64_t)16 * s == ((int64_t)sl.k * ROWS + sl.row) * es, "%s %s slot %d is not where the readers look", c.name.c_str(), what, s);
+                    seen[(size_t)(sl.k * (ROWS / V) + sl.row / V)]++;
+                }
                 CHECK((size_t)(r0 + sl.row) < rtab.size(), "%s %s row table index %d of %zu", c.name.c_str(), what, r0 + sl.row, rtab.size());
                 const int64_t rowpart = rtab[(size_t)(r0 + sl.row)];
-                for(int j = 1; j < V && r0 + sl.row + j < nrows; j++)
+                for(int j = 1; !KF && j < V && r0 + sl.row + j < nrows; j++)
                     CHECK(rtab[(size_t)(r0 + sl.row + j)] - rowpart == j, "%s %s row run broken at %d", c.name.c_str(), what, r0 + sl.row);
                 // the lane's part of the address, as the kernel computes it in 32 bits
                 const uint64_t lanepart = (uint64_t)es * ((uint64_t)rowpart + (uint64_t)sl.k * (uint64_t)kstride);
                 CHECK(lanepart <= 0xFFFFFFFFull, "%s %s lane offset overflows 32 bits", c.name.c_str(), what);
                 for(int o : origins)
                 {
-                    CHECK(o >= 0 && o + sl.k < v.K, "%s %s k %d of %lld", c.name.c_str(), what, o + sl.k, (long long)v.K);
+                    CHECK(o >= 0 && o + sl.k + (KF ? V - 1 : 0) < v.K, "%s %s k %d of %lld", c.name.c_str(), what, o + sl.k, (long long)v.K);
+                    for(int j = 1; KF && j < V; j++)
+                        CHECK(ktab[(size_t)(o + sl.k + j)] - ktab[(size_t)(o + sl.k)] == j, "%s %s k run broken at %d", c.name.c_str(), what, o + sl.k);
                     const uint64_t origin = (uint64_t)es * (uint64_t)o * (uint64_t)kstride;
                     CHECK(origin <= 0xFFFFFFFFull, "%s %s origin overflows 32 bits", c.name.c_str(), what);
                     const int64_t off = rowpart + (int64_t)(o + sl.k) * kstride;
@@ -270,7 +284,7 @@ static void check_wide_operand(const char* what, const Case& c, const GemmView& 
         CHECK(seen[i] == (WK ? 4 : 1), "%s %s vector %zu filled %d times", c.name.c_str(), what, i, seen[i]);
 }
 
-template <int V, int ROWS>
+template <int V, int ROWS, bool KF>
 static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
 {
     constexpr bool WK = ROWS == 32;
@@ -326,8 +340,8 @@ static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
         for(int tp : {0, tiles_p / 2, tiles_p - 1})
             for(int tq : {0, tiles_q / 2, tiles_q - 1})
             {
-                check_wide_operand<V, ROWS>("X", c, v, true, tp * ROWS, BK, NLW, origins);
-                check_wide_operand<V, ROWS>("Y", c, v, false, tq * ROWS, BK, NLW, origins);
+                check_wide_operand<V, ROWS, KF>("X", c, v, true, tp * ROWS, BK, NLW, origins);
+                check_wide_operand<V, ROWS, KF>("Y", c, v, false, tq * ROWS, BK, NLW, origins);
                 walked += (long)origins.size() * 2 * BK * ROWS / V;
             }
         if(want > 1 && split == 1)
@@ -442,10 +456,12 @@ int main()
     rank4("cfg4", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 32, 32, 32, 32, 32, 16);
     rank4("k8_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 40, 9, 24, 13, 8, 1);
     rank4("k24_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 42, 9, 25, 13, 8, 3);
+    // odd row counts under k-contiguous operands: tiles overhang, C / D may ask for moved-back tiles, which these kernels do not do
+    rank4("ragged_kfast", {20, 21, 0, 1}, {20, 21, 10, 11}, {10, 11, 0, 1}, 15, 19, 17, 21, 16, 9);
     rank4("big_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 8192, 16, 64, 1, 64, 64);
     const WideTile wide[] = {{"f32", 0, 4, 4, 2, 16, 64}, {"f64", 1, 16, 8, 2, 8, 64}, {"c32", 4, 2048, 8, 2, 8, 64},
                              {"f32", 0, 4, 4, 3, 16, 32}, {"f64", 1, 16, 8, 3, 8, 32}, {"c32", 4, 2048, 8, 3, 8, 32}};
-    int offered_wide = 0, refused_big = 0;
+    int offered_wide = 0, refused_big = 0, offered_kf = 0;
     for(const WideTile& w : wide)
         for(const Case& c : cases)
         {
@@ -481,17 +497,26 @@ int main()
             if(!avail)
                 continue;
             const int V = 16 / w.elem_bytes;
-            CHECK(v.x_vec == V && v.y_vec == V && (V == 1 || (!v.x_kfast && !v.y_kfast)) && v.k_affine && v.K % w.bk == 0 && v.xy_aligned && !v.shift_p
-                      && !v.shift_q,
+            CHECK(v.x_vec == V && v.y_vec == V && v.x_kfast == v.y_kfast && v.k_affine && v.K % w.bk == 0 && v.xy_aligned
+                      && (v.x_kfast || (!v.shift_p && !v.shift_q)),
                   "%s %s offered outside its restrictions", w.type, c.name.c_str());
             offered_wide++;
             const int nlw = w.bk * w.rows * w.elem_bytes / (w.rows == 32 ? 1024 : 4096);
-            if(w.rows == 64)
-                walked += V == 4 ? check_wide_tile<4, 64>(c, v, w.bk, nlw) : check_wide_tile<2, 64>(c, v, w.bk, nlw);
+            if(v.x_kfast)
+            {
+                offered_kf++;
+                if(w.rows == 64)
+                    walked += V == 4 ? check_wide_tile<4, 64, true>(c, v, w.bk, nlw) : check_wide_tile<2, 64, true>(c, v, w.bk, nlw);
+                else
+                    walked += V == 4 ? check_wide_tile<4, 32, true>(c, v, w.bk, nlw) : check_wide_tile<2, 32, true>(c, v, w.bk, nlw);
+            }
+            else if(w.rows == 64)
+                walked += V == 4 ? check_wide_tile<4, 64, false>(c, v, w.bk, nlw) : check_wide_tile<2, 64, false>(c, v, w.bk, nlw);
             else
-                walked += V == 4 ? check_wide_tile<4, 32>(c, v, w.bk, nlw) : check_wide_tile<2, 32>(c, v, w.bk, nlw);
+                walked += V == 4 ? check_wide_tile<4, 32, false>(c, v, w.bk, nlw) : check_wide_tile<2, 32, false>(c, v, w.bk, nlw);
         }
     g_dtype = 2;
+    CHECK(offered_kf >= 30, "only %d k-contiguous (case, type, tile) triples were offered a 32/64-bit direct-load kernel", offered_kf);
     CHECK(offered_wide >= 60, "only %d (case, type, tile) triples were offered a 32/64-bit direct-load kernel", offered_wide);
     CHECK(refused_big >= 2, "the tensor past 2^32 bytes was not exercised (%d)", refused_big);
     std::printf("%s: %d + %d problems x tiles, %ld requests walked, %d failures\n", g_fail ? "FAILED" : "ok", offered, offered_wide, walked,
