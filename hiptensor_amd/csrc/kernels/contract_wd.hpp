@@ -1,8 +1,10 @@
 // 32/64-bit (f32, f64, complex f32) contraction kernel for gfx950 whose operand tiles go from global
-// memory straight into LDS (global_load_lds_dwordx4), for the layout in which both operands are
-// contiguous along their row index (packed column-major: every benchmark configuration of these
-// types).  (Complex f64 is not instantiated: two K tiles of its operands do not fit the registers,
-// and without them it measured 8 % behind the eight-wave tile of contract_w.hpp.)
+// memory straight into LDS (global_load_lds_dwordx4), for the two layouts in which both operands
+// are contiguous along the same kind of index: their row index (packed column-major: every benchmark
+// configuration of these types; described below) or k (packed row-major: what NULL strides mean; the
+// differences are at wd_slot_kf in hd_addr.hpp and at read_k).  (Complex f64 is not instantiated: two K
+// tiles of its operands do not fit the registers, and without them it measured 8 % behind the
+// eight-wave tile of contract_w.hpp.)
 //
 // Same MFMA use, complex product and epilogue as contract_w.hpp; what differs is how a tile gets
 // into LDS and from there into registers.  There, a gather passes through registers and has one K
@@ -25,8 +27,8 @@
 //     spare LDS behind the ring, so every wait sees the same number of younger loads.
 //
 // Restrictions (the dispatcher checks them): both operands gathered in 16-byte vectors along their
-// row index, on 16-byte boundaries; one K stride per operand; K a multiple of BK; byte offsets inside
-// each operand below 2^32.
+// row index, or both along k, on 16-byte boundaries; one K stride per operand; K a multiple of BK;
+// byte offsets inside each operand below 2^32.
 #pragma once
 #include <utility>
 
