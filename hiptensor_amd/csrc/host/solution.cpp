@@ -213,7 +213,11 @@ namespace hipta
             // operands.  k-contiguous operands, 2048^2 x 1024 on 64 x 64: f32 74.8 us, f64 132.2, c32 244.3; on
             // 32 x 32 a wave's runs are 64 bytes a row and K tile: 1024^2 x 2048 f64 125 against 70.7 us)
             case HIPTK_F32: r = big ? (kf ? TileRate{0.75, 0.78} : TileRate{0.81, 0.89}) : (kf ? TileRate{0.55, 0.60} : TileRate{0.65, 0.70}); break;
-            case HIPTK_F64: r = big ? (kf ? TileRate{0.80, 0.84} : TileRate{0.82, 0.90}) : (kf ? TileRate{0.45, 0.50} : TileRate{0.82, 0.90}); break;
+            // (one operand k-contiguous, 1024^2 x 2048 f64 on 32 x 32: 82.9 against 70.8 us)
+            case HIPTK_F64:
+                r = big ? (kf ? TileRate{0.80, 0.84} : TileRate{0.82, 0.90})
+                        : (kf ? TileRate{0.45, 0.50} : (v.x_kfast || v.y_kfast) ? TileRate{0.62, 0.66} : TileRate{0.82, 0.90});
+                break;
             case HIPTK_C32: r = big ? (kf ? TileRate{0.88, 0.90} : TileRate{0.90, 0.91}) : (kf ? TileRate{0.85, 0.88} : TileRate{0.90, 0.91}); break;
             default: break;
             }
@@ -223,7 +227,7 @@ namespace hipta
             // slice shorter than the ring has less in flight to wait for); the 32 x 32 tile adds its partial
             // tiles through LDS (640^2 x 64 f32: 8.4 us against 6.3 on 64 x 64 tiles)
             // (k-contiguous: 8.6 against 6.5 us)
-            round_extra_us = 2.0 * std::min(1.0, kper / s.bk / 16.0) + (big ? 0.0 : kf ? 2.5 : 1.0);
+            round_extra_us = 2.0 * std::min(1.0, kper / s.bk / 16.0) + (big ? 0.0 : (v.x_kfast || v.y_kfast) ? 2.5 : 1.0);
         }
         if(class_max_vec(v.cls) > 1)
         {

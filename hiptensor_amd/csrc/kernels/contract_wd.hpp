@@ -1,8 +1,8 @@
 // 32/64-bit (f32, f64, complex f32) contraction kernel for gfx950 whose operand tiles go from global
-// memory straight into LDS (global_load_lds_dwordx4), for the two layouts in which both operands
-// are contiguous along the same kind of index: their row index (packed column-major: every benchmark
-// configuration of these types; described below) or k (packed row-major: what NULL strides mean; the
-// differences are at wd_slot_kf in hd_addr.hpp and at read_k).  (Complex f64 is not instantiated: two K
+// memory straight into LDS (global_load_lds_dwordx4), for operands that are each contiguous along
+// their row index (both: packed column-major, every benchmark configuration of these types; described
+// below) or along k (both: packed row-major, what NULL strides mean; the differences are at wd_slot_kf
+// in hd_addr.hpp and at read_op).  (Complex f64 is not instantiated: two K
 // tiles of its operands do not fit the registers, and without them it measured 8 % behind the
 // eight-wave tile of contract_w.hpp.)
 //
@@ -26,8 +26,8 @@
 //     Tiles requested beyond the K range are not branched around: they re-read the last tile into
 //     spare LDS behind the ring, so every wait sees the same number of younger loads.
 //
-// Restrictions (the dispatcher checks them): both operands gathered in 16-byte vectors along their
-// row index, or both along k, on 16-byte boundaries; one K stride per operand; K a multiple of BK;
+// Restrictions (the dispatcher checks them): both operands gathered in 16-byte vectors, along their
+// row index or along k, on 16-byte boundaries; one K stride per operand; K a multiple of BK;
 // byte offsets inside each operand below 2^32.
 #pragma once
 #include <utility>
@@ -54,7 +54,7 @@ namespace hiptk
     // multiplies all of it over its own quarter of the K range out of a ring of its own (no barrier in the
     // loop), and the four partial tiles are added through LDS at the end: for outputs too small to fill the
     // device with 64 x 64 tiles, in one launch.
-    template <typename Tr, int BK, int NS, bool WK, bool KF = false>
+    template <typename Tr, int BK, int NS, bool WK, bool XKF = false, bool YKF = false>
     struct WdGeom
     {
         static constexpr int ROWS = WK ? 32 : 64; // rows of an operand tile
@@ -74,7 +74,7 @@ namespace hiptk
         static_assert(!WK || RING >= (32 / Tr::TILE) * (32 / Tr::TILE) * Tr::NREG * 64 * (int)sizeof(typename Tr::O),
                       "a wave's partial tile is handed over in its own ring");
         static_assert(LDS_BYTES <= 160 * 1024, "LDS of one CU");
-        static_assert(!KF || (BK / Tr::KM) % V == 0, "a k-contiguous vector feeds whole k-steps");
+        static_assert(!(XKF || YKF) || (BK / Tr::KM) % V == 0, "a k-contiguous vector feeds whole k-steps");
     };
 
     __device__ __forceinline__ float   wd_add(float x, float y) { return __fadd_rn(x, y); }
@@ -184,10 +184,12 @@ namespace hiptk
         }
     }
 
-    template <typename Tr, int BK, int NS, bool WK, bool KF>
+    template <typename Tr, int BK, int NS, bool WK, bool XKF, bool YKF>
     __global__ void __launch_bounds__(256, 2) contract_wd_kernel(const KArgs a)
     {
-        typedef WdGeom<Tr, BK, NS, WK, KF> G;
+        typedef WdGeom<Tr, BK, NS, WK, XKF, YKF> G;
+        // with a k-contiguous operand the k-slots of one k-step are V apart in k (see wd_slot_kf), for both operands
+        constexpr bool VAPART = XKF || YKF;
         typedef typename Tr::S     S;
         constexpr int              TILE = Tr::TILE;
         constexpr int              TP = 32 / TILE, TQ = 32 / TILE;
@@ -231,9 +233,10 @@ namespace hiptk
         for(int i = 0; i < NLW; i++)
         {
             const int    s_ = ((WK ? 0 : wave * NLW) + i) * 64 + lane;
-            const HdSlot sl = KF ? wd_slot_kf<G::V, ROWS>(s_) : wd_slot<G::V, ROWS>(s_);
-            xv[i]           = (uint32_t)ES * ((uint32_t)a.xp[p0 + sl.row] + (uint32_t)sl.k * (uint32_t)a.xk_stride);
-            yv[i]           = (uint32_t)ES * ((uint32_t)a.yq[q0 + sl.row] + (uint32_t)sl.k * (uint32_t)a.yk_stride);
+            const HdSlot sx = XKF ? wd_slot_kf<G::V, ROWS>(s_) : wd_slot<G::V, ROWS>(s_);
+            const HdSlot sy = YKF ? wd_slot_kf<G::V, ROWS>(s_) : wd_slot<G::V, ROWS>(s_);
+            xv[i]           = (uint32_t)ES * ((uint32_t)a.xp[p0 + sx.row] + (uint32_t)sx.k * (uint32_t)a.xk_stride);
+            yv[i]           = (uint32_t)ES * ((uint32_t)a.yq[q0 + sy.row] + (uint32_t)sy.k * (uint32_t)a.yk_stride);
         }
         // k origin of the next tile to be requested (tiles beyond the slice's last one repeat it), as a
         // 32-bit byte offset from the operand's base, kept in scalar registers
@@ -296,14 +299,16 @@ namespace hiptk
 
         const int row   = lane & (TILE - 1);
         const int kslot = Tr::kslot(lane);
-        const int xfo   = kslot * ROWS + wp * 32 + row;
-        const int yfo   = kslot * ROWS + wq * 32 + row;
+        // (a k-contiguous operand's stage is indexed in 16-byte vectors, [k / V][ROWS]; a row-contiguous one's in
+        // elements, [k][ROWS], where the k-slots of a k-step are 1 or V rows of the stage apart)
+        const int xfo = kslot * (!XKF && VAPART ? G::V : 1) * ROWS + wp * 32 + row;
+        const int yfo = kslot * (!YKF && VAPART ? G::V : 1) * ROWS + wq * 32 + row;
 
         // This wave's operands of one K tile, in registers: tile t + 1 is read from LDS while tile t
         // is multiplied, so that a wave alone on its SIMD does not wait for LDS either.
         struct Frags
         {
-            S x[KS][TP], y[KS][TQ];
+            S x[KS][TP], y[KS][TP];
         };
         Frags fr[2];
         // the operands of k-step ks of the tile in ring stage ST (k-contiguous operands: of the V k-steps from
@@ -312,42 +317,37 @@ namespace hiptk
         {
             S e[G::V];
         };
-        auto read_k = [&](auto st_c, Frags& f, int ks) {
-            constexpr int ST = decltype(st_c)::value;
-            if constexpr(KF)
+        // one operand's part of it: KF: a vector of V k-steps' elements when ks is the first of them; else one
+        // element, at k-slot distance 1 or (next to a k-contiguous operand) V
+        auto read_op = [&](auto kf_c, const unsigned char* base, int fo, S (&dst)[KS][TP], int ks) {
+            static_assert(TP == TQ, "one reader for both operands");
+            if constexpr(decltype(kf_c)::value)
             {
                 if(ks % G::V != 0)
                     return;
-                const SVec* lx = (const SVec*)(ring + ST * G::STAGE_BYTES);
-                const SVec* ly = (const SVec*)(ring + ST * G::STAGE_BYTES + G::OP_BYTES);
+                const SVec* l = (const SVec*)base;
 #pragma unroll
                 for(int i = 0; i < TP; i++)
                 {
-                    const SVec v = lx[xfo + (ks / G::V) * Tr::KM * ROWS + i * TILE];
+                    const SVec v = l[fo + (ks / G::V) * Tr::KM * ROWS + i * TILE];
 #pragma unroll
                     for(int j = 0; j < G::V; j++)
-                        f.x[ks + j][i] = v.e[j];
-                }
-#pragma unroll
-                for(int j2 = 0; j2 < TQ; j2++)
-                {
-                    const SVec v = ly[yfo + (ks / G::V) * Tr::KM * ROWS + j2 * TILE];
-#pragma unroll
-                    for(int j = 0; j < G::V; j++)
-                        f.y[ks + j][j2] = v.e[j];
+                        dst[ks + j][i] = v.e[j];
                 }
             }
             else
             {
-                const S* lx = (const S*)(ring + ST * G::STAGE_BYTES);
-                const S* ly = (const S*)(ring + ST * G::STAGE_BYTES + G::OP_BYTES);
+                const S*  l  = (const S*)base;
+                const int k0 = VAPART ? ((ks / G::V) * Tr::KM * G::V + ks % G::V) : ks * Tr::KM;
 #pragma unroll
                 for(int i = 0; i < TP; i++)
-                    f.x[ks][i] = lx[xfo + ks * Tr::KM * ROWS + i * TILE];
-#pragma unroll
-                for(int j = 0; j < TQ; j++)
-                    f.y[ks][j] = ly[yfo + ks * Tr::KM * ROWS + j * TILE];
+                    dst[ks][i] = l[fo + k0 * ROWS + i * TILE];
             }
+        };
+        auto read_k = [&](auto st_c, Frags& f, int ks) {
+            constexpr int ST = decltype(st_c)::value;
+            read_op(std::integral_constant<bool, XKF>{}, ring + ST * G::STAGE_BYTES, xfo, f.x, ks);
+            read_op(std::integral_constant<bool, YKF>{}, ring + ST * G::STAGE_BYTES + G::OP_BYTES, yfo, f.y, ks);
         };
         auto read_tile = [&](auto st_c, Frags& f) {
 #pragma unroll
@@ -462,16 +462,16 @@ namespace hiptk
         }
     }
 
-    template <typename Tr, int BK, int NS, bool WK, bool KF>
+    template <typename Tr, int BK, int NS, bool WK, bool XKF, bool YKF>
     int launch_wd(const KArgs& a, hipStream_t stream)
     {
-        typedef WdGeom<Tr, BK, NS, WK, KF> G;
+        typedef WdGeom<Tr, BK, NS, WK, XKF, YKF> G;
         // (a tile is never moved back here.  Row-contiguous operands that would need it are not offered this
         // kernel; with k-contiguous ones the flag can only come from C / D's vectors, which the element-wise
         // epilogue does not use: an overhanging tile reads the row tables' padding and stores nothing there)
-        if(a.K < BK || a.K % BK != 0 || (!KF && (a.shift_p || a.shift_q)))
+        if(a.K < BK || a.K % BK != 0 || (!XKF && a.shift_p) || (!YKF && a.shift_q))
             return (int)hipErrorInvalidValue;
-        auto                    kern = contract_wd_kernel<Tr, BK, NS, WK, KF>;
+        auto                    kern = contract_wd_kernel<Tr, BK, NS, WK, XKF, YKF>;
         static const hipError_t attr = hipFuncSetAttribute(
             (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
         if(attr != hipSuccess)
@@ -490,7 +490,7 @@ namespace hiptk
         hiptk::TR::CLS, ID, hiptk::TR::VMAX == 1, hiptk::TR::VMAX == 1, hiptk::TR::VMAX,            \
             hiptk::TR::VMAX, 1, 64, 64, BK, 256,                                                    \
             hiptk::WdGeom<hiptk::TR, BK, NS, false>::LDS_BYTES, #TR "_64x64x" #BK "_direct" #NS,\
-            &hiptk::launch_wd<hiptk::TR, BK, NS, false, false>, BK                                         \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, false, false, false>, BK                                         \
     }
 
 // ... and of the 32 x 32 tile whose four waves split the K range between them.
@@ -499,19 +499,21 @@ namespace hiptk
         hiptk::TR::CLS, ID, hiptk::TR::VMAX == 1, hiptk::TR::VMAX == 1, hiptk::TR::VMAX,            \
             hiptk::TR::VMAX, 1, 32, 32, BK, 256,                                                    \
             hiptk::WdGeom<hiptk::TR, BK, NS, true>::LDS_BYTES, #TR "_32x32x" #BK "_direct" #NS "k4", \
-            &hiptk::launch_wd<hiptk::TR, BK, NS, true, false>, BK                                        \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, true, false, false>, BK                                        \
     }
 
-// ... and of both for operands that are contiguous along k (16-byte vectors of k, one K stride).
-#define HIPTK_WD_ENTRY_KF(TR, ID, BK, NS)                                                           \
+// ... and of both where X (XKF) and / or Y (YKF) are contiguous along k instead (16-byte vectors of k, one K stride).
+#define HIPTK_WD_ENTRY_KF(TR, ID, BK, NS, XKF, YKF)                                                 \
     {                                                                                               \
-        hiptk::TR::CLS, ID, 1, 1, hiptk::TR::VMAX, hiptk::TR::VMAX, 1, 64, 64, BK, 256,             \
-            hiptk::WdGeom<hiptk::TR, BK, NS, false, true>::LDS_BYTES, #TR "_64x64x" #BK "_direct" #NS "kf", \
-            &hiptk::launch_wd<hiptk::TR, BK, NS, false, true>, BK                                   \
+        hiptk::TR::CLS, ID, XKF, YKF, hiptk::TR::VMAX, hiptk::TR::VMAX, 1, 64, 64, BK, 256,         \
+            hiptk::WdGeom<hiptk::TR, BK, NS, false, XKF != 0, YKF != 0>::LDS_BYTES,                 \
+            #TR "_64x64x" #BK "_direct" #NS "kf" #XKF #YKF,                                         \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, false, XKF != 0, YKF != 0>, BK                     \
     }
-#define HIPTK_WK_ENTRY_KF(TR, ID, BK, NS)                                                           \
+#define HIPTK_WK_ENTRY_KF(TR, ID, BK, NS, XKF, YKF)                                                 \
     {                                                                                               \
-        hiptk::TR::CLS, ID, 1, 1, hiptk::TR::VMAX, hiptk::TR::VMAX, 1, 32, 32, BK, 256,             \
-            hiptk::WdGeom<hiptk::TR, BK, NS, true, true>::LDS_BYTES, #TR "_32x32x" #BK "_direct" #NS "k4kf", \
-            &hiptk::launch_wd<hiptk::TR, BK, NS, true, true>, BK                                    \
+        hiptk::TR::CLS, ID, XKF, YKF, hiptk::TR::VMAX, hiptk::TR::VMAX, 1, 32, 32, BK, 256,         \
+            hiptk::WdGeom<hiptk::TR, BK, NS, true, XKF != 0, YKF != 0>::LDS_BYTES,                  \
+            #TR "_32x32x" #BK "_direct" #NS "k4kf" #XKF #YKF,                                       \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, true, XKF != 0, YKF != 0>, BK                      \
     }

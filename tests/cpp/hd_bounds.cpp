@@ -284,7 +284,7 @@ static void check_wide_operand(const char* what, const Case& c, const GemmView& 
         CHECK(seen[i] == (WK ? 4 : 1), "%s %s vector %zu filled %d times", c.name.c_str(), what, i, seen[i]);
 }
 
-template <int V, int ROWS, bool KF>
+template <int V, int ROWS>
 static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
 {
     constexpr bool WK = ROWS == 32;
@@ -340,8 +340,14 @@ static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
         for(int tp : {0, tiles_p / 2, tiles_p - 1})
             for(int tq : {0, tiles_q / 2, tiles_q - 1})
             {
-                check_wide_operand<V, ROWS, KF>("X", c, v, true, tp * ROWS, BK, NLW, origins);
-                check_wide_operand<V, ROWS, KF>("Y", c, v, false, tq * ROWS, BK, NLW, origins);
+                if(v.x_kfast)
+                    check_wide_operand<V, ROWS, true>("X", c, v, true, tp * ROWS, BK, NLW, origins);
+                else
+                    check_wide_operand<V, ROWS, false>("X", c, v, true, tp * ROWS, BK, NLW, origins);
+                if(v.y_kfast)
+                    check_wide_operand<V, ROWS, true>("Y", c, v, false, tq * ROWS, BK, NLW, origins);
+                else
+                    check_wide_operand<V, ROWS, false>("Y", c, v, false, tq * ROWS, BK, NLW, origins);
                 walked += (long)origins.size() * 2 * BK * ROWS / V;
             }
         if(want > 1 && split == 1)
@@ -461,7 +467,7 @@ int main()
     rank4("big_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 8192, 16, 64, 1, 64, 64);
     const WideTile wide[] = {{"f32", 0, 4, 4, 2, 16, 64}, {"f64", 1, 16, 8, 2, 8, 64}, {"c32", 4, 2048, 8, 2, 8, 64},
                              {"f32", 0, 4, 4, 3, 16, 32}, {"f64", 1, 16, 8, 3, 8, 32}, {"c32", 4, 2048, 8, 3, 8, 32}};
-    int offered_wide = 0, refused_big = 0, offered_kf = 0;
+    int offered_wide = 0, refused_big = 0, offered_kf = 0, offered_mixed = 0;
     for(const WideTile& w : wide)
         for(const Case& c : cases)
         {
@@ -497,25 +503,20 @@ int main()
             if(!avail)
                 continue;
             const int V = 16 / w.elem_bytes;
-            CHECK(v.x_vec == V && v.y_vec == V && v.x_kfast == v.y_kfast && v.k_affine && v.K % w.bk == 0 && v.xy_aligned
-                      && (v.x_kfast || (!v.shift_p && !v.shift_q)),
+            CHECK(v.x_vec == V && v.y_vec == V && v.k_affine && v.K % w.bk == 0 && v.xy_aligned && (v.x_kfast || !v.shift_p)
+                      && (v.y_kfast || !v.shift_q),
                   "%s %s offered outside its restrictions", w.type, c.name.c_str());
             offered_wide++;
             const int nlw = w.bk * w.rows * w.elem_bytes / (w.rows == 32 ? 1024 : 4096);
-            if(v.x_kfast)
-            {
-                offered_kf++;
-                if(w.rows == 64)
-                    walked += V == 4 ? check_wide_tile<4, 64, true>(c, v, w.bk, nlw) : check_wide_tile<2, 64, true>(c, v, w.bk, nlw);
-                else
-                    walked += V == 4 ? check_wide_tile<4, 32, true>(c, v, w.bk, nlw) : check_wide_tile<2, 32, true>(c, v, w.bk, nlw);
-            }
-            else if(w.rows == 64)
-                walked += V == 4 ? check_wide_tile<4, 64, false>(c, v, w.bk, nlw) : check_wide_tile<2, 64, false>(c, v, w.bk, nlw);
+            offered_kf += (v.x_kfast || v.y_kfast) ? 1 : 0;
+            offered_mixed += (v.x_kfast != v.y_kfast) ? 1 : 0;
+            if(w.rows == 64)
+                walked += V == 4 ? check_wide_tile<4, 64>(c, v, w.bk, nlw) : check_wide_tile<2, 64>(c, v, w.bk, nlw);
             else
-                walked += V == 4 ? check_wide_tile<4, 32, false>(c, v, w.bk, nlw) : check_wide_tile<2, 32, false>(c, v, w.bk, nlw);
+                walked += V == 4 ? check_wide_tile<4, 32>(c, v, w.bk, nlw) : check_wide_tile<2, 32>(c, v, w.bk, nlw);
         }
     g_dtype = 2;
+    CHECK(offered_mixed >= 30, "only %d mixed (case, type, tile) triples were offered a 32/64-bit direct-load kernel", offered_mixed);
     CHECK(offered_kf >= 30, "only %d k-contiguous (case, type, tile) triples were offered a 32/64-bit direct-load kernel", offered_kf);
     CHECK(offered_wide >= 60, "only %d (case, type, tile) triples were offered a 32/64-bit direct-load kernel", offered_wide);
     CHECK(refused_big >= 2, "the tensor past 2^32 bytes was not exercised (%d)", refused_big);
