@@ -5,6 +5,8 @@ default selection exercises only a few tiles; this covers the rest, including th
 state (K spans several K tiles), K tails and partial tiles in M and N."""
 import os
 
+import numpy as np
+
 import pytest
 
 import cases
@@ -178,3 +180,56 @@ def _tile_exists(cls, tile):
 
     ti = TileInfo()
     return lib.hiptk_tile_info(cls, tile, ctypes.byref(ti)) == 0
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64", "c32"])
+def test_direct_load_tiles_on_random_layouts(gpu_handle, oracle_mod, dtype):
+    """The 32/64-bit kernels that load operand tiles straight into LDS, on seeded random problems: two or
+    three modes per group with extents from a small set, every operand packed with either its row modes or
+    its k modes fastest (all four combinations occur), D packed in a random mode order, K a multiple of 16,
+    scale and bilinear, complex scalars for complex data.  Each problem runs the default selection and both
+    direct-load tile ids (64 x 64; 32 x 32 with the waves splitting K), the latter also with split-K 2, and
+    is held against the oracle; a problem a tile is not offered for is skipped for that tile, and every
+    (tile, operand layout) pair must have run at least once."""
+    rng = np.random.default_rng({"f32": 11, "f64": 12, "c32": 13}[dtype])
+    ran = set()
+    try:
+        for n in range(16):
+            nm, nn, nk = (int(rng.integers(1, 3)) for _ in range(3))
+            ext = {}
+            for base, cnt in ((0, nm), (10, nn)):
+                for i in range(cnt):
+                    ext[base + i] = int(rng.choice([4, 8, 12, 20])) if i == 0 else int(rng.choice([3, 5, 6, 9]))
+            for i in range(nk):
+                ext[20 + i] = 16 if i == 0 else int(rng.choice([1, 2, 3, 5]))
+            ms, ns, ks = ([b + i for i in range(c)] for b, c in ((0, nm), (10, nn), (20, nk)))
+            a_kfast, b_kfast = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+            mA = ks + ms if a_kfast else ms + ks  # make_workload packs the first listed mode fastest
+            mB = ks + ns if b_kfast else ns + ks
+            mD = ms + ns if rng.integers(0, 2) else ns + ms
+            if dtype == "c32":
+                alpha, beta = complex(rng.uniform(-2, 2), rng.uniform(-2, 2)), (None if n % 3 == 0 else complex(rng.uniform(-2, 2), rng.uniform(-2, 2)))
+            else:
+                alpha, beta = float(rng.uniform(-2, 2)), (None if n % 3 == 0 else float(rng.uniform(-2, 2)))
+            w = wl.make_workload(dtype, cases.COMPUTE[dtype], mA, mB, mD, ext, alpha, beta,
+                                 name=f"random_{dtype}_{n}_{'k' if a_kfast else 'r'}{'k' if b_kfast else 'r'}")
+            inp = wl.host_inputs(w)
+            exp = cases.logical_view(w, oracle_mod.contract(w, inp["A"], inp["B"], inp["C"]))
+            for force in (None, "2,1", "3,1", "3,2"):
+                if force:
+                    os.environ["HIPTENSOR_AMD_FORCE_KERNEL"] = force
+                else:
+                    os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
+                print(f"[case] {w['name']} ext={ext} mD={mD} force={force}", flush=True)
+                try:
+                    got, info = gpu_util.run_gpu(gpu_handle, w, inp, pref=api.HIPTENSOR_WORKSPACE_MAX, return_info=True)
+                except api.HiptensorError as e:
+                    assert force and e.status == api.HIPTENSOR_STATUS_EXECUTION_FAILED, e
+                    continue
+                cases.assert_parity(w, cases.logical_view(w, got), exp, info["kernel_name"])
+                if force and "direct" in info["kernel_name"]:
+                    ran.add((force, info["x_kfast"], info["y_kfast"]))
+    finally:
+        os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
+    print("ran:", sorted(ran), flush=True)
+    assert len({r[0] for r in ran}) == 3 and len({(r[1], r[2]) for r in ran}) >= 3, sorted(ran)
