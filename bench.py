@@ -41,6 +41,7 @@ MEASURED_TRAFFIC_KIB = {
     # profiles/contract_hd_kernel_4096cubed.md
     ("cfg2_f16_scale_4096", "TraitsF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (100080.0, 34560.0),
     ("cfg2_f16_bilinear_4096", "TraitsF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (116540.0, 34591.0),
+    ("cfg2_bf16_scale_4096", "TraitsBF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (98747.0, 32768.0),
     ("cfg2_bf16_bilinear_4096", "TraitsBF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (115910.0, 32770.0),
     # profiles/contract_kernels_configs_1_3_4_5_counters.md (split-K: contraction kernel + reduction kernel)
     ("cfg1_f32_bilinear_256", "WTraitsF32_64x64x16_00"): (823.0 + 1187.5, 2048.0 + 256.0),
