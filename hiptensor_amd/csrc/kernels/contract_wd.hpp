@@ -27,8 +27,9 @@
 //     spare LDS behind the ring, so every wait sees the same number of younger loads.
 //
 // Restrictions (the dispatcher checks them): both operands gathered in 16-byte vectors, along their
-// row index or along k, on 16-byte boundaries; one K stride per operand; K a multiple of BK;
-// byte offsets inside each operand below 2^32.
+// row index or along k, on 16-byte boundaries; one K stride per operand; K at least BK (a last tile
+// shorter than BK loads the vectors beyond K from zeros), and a multiple of the vector where an operand
+// is contiguous along k; byte offsets inside each operand below 2^32.
 #pragma once
 #include <utility>
 
@@ -76,6 +77,9 @@ namespace hiptk
         static_assert(LDS_BYTES <= 160 * 1024, "LDS of one CU");
         static_assert(!(XKF || YKF) || (BK / Tr::KM) % V == 0, "a k-contiguous vector feeds whole k-steps");
     };
+
+    // what the vectors of a short last K tile that lie beyond K are loaded from
+    static __device__ __attribute__((aligned(16))) const unsigned char wd_zero16[16] = {0};
 
     __device__ __forceinline__ float   wd_add(float x, float y) { return __fadd_rn(x, y); }
     __device__ __forceinline__ double  wd_add(double x, double y) { return __dadd_rn(x, y); }
@@ -215,7 +219,7 @@ namespace hiptk
 
         int       kt_begin = blockIdx.z * a.ktiles_per_split;
         int       kt_end   = kt_begin + a.ktiles_per_split;
-        const int kt_all   = a.K / BK; // K is a multiple of BK
+        const int kt_all   = (a.K + BK - 1) / BK; // the last tile may hold fewer than BK k
         if(kt_end > kt_all)
             kt_end = kt_all;
         if(WK)
@@ -227,8 +231,12 @@ namespace hiptk
         }
         const int nt = kt_end - kt_begin;
 
-        // this lane's 16 bytes of each of its loads, as byte offsets from the tile's k origin
-        uint32_t xv[NLW], yv[NLW];
+        // this lane's 16 bytes of each of its loads, as byte offsets from the tile's k origin; and, bit i,
+        // whether load i of a short last tile lies inside K
+        const int tail_k      = a.K % BK;
+        const int tail_origin = tail_k ? (kt_all - 1) * BK : -1;
+        uint32_t  xin = 0, yin = 0;
+        uint32_t  xv[NLW], yv[NLW];
 #pragma unroll
         for(int i = 0; i < NLW; i++)
         {
@@ -237,6 +245,8 @@ namespace hiptk
             const HdSlot sy = YKF ? wd_slot_kf<G::V, ROWS>(s_) : wd_slot<G::V, ROWS>(s_);
             xv[i]           = (uint32_t)ES * ((uint32_t)a.xp[p0 + sx.row] + (uint32_t)sx.k * (uint32_t)a.xk_stride);
             yv[i]           = (uint32_t)ES * ((uint32_t)a.yq[q0 + sy.row] + (uint32_t)sy.k * (uint32_t)a.yk_stride);
+            xin |= wd_tail_inside(XKF, sx.k, G::V, tail_k) ? 1u << i : 0u;
+            yin |= wd_tail_inside(YKF, sy.k, G::V, tail_k) ? 1u << i : 0u;
         }
         // k origin of the next tile to be requested (tiles beyond the slice's last one repeat it), as a
         // 32-bit byte offset from the operand's base, kept in scalar registers
@@ -262,17 +272,37 @@ namespace hiptk
             const bool     real = lu < nt;
             const uint32_t dx   = real ? wdx + ST * G::STAGE_BYTES : wspare;
             const uint32_t dy   = real ? wdy + ST * G::STAGE_BYTES : wspare;
-#pragma unroll
-            for(int i = 0; i < NLW; i++)
+            if(ko == tail_origin)
             {
-                dma_dst_at(dx, i * 1024);
-                dma_load(xv[i], xsrc);
+                // the short last tile (or a repeat of it): the same number of loads, each lane from where its
+                // vector lies if that is inside K, else from zeros: the tile then multiplies as a whole one
+#pragma unroll
+                for(int i = 0; i < NLW; i++)
+                {
+                    dma_dst_at(dx, i * 1024);
+                    dma_load_at((xin >> i) & 1u ? (const void*)(xsrc + xv[i]) : (const void*)wd_zero16);
+                }
+#pragma unroll
+                for(int i = 0; i < NLW; i++)
+                {
+                    dma_dst_at(dy, i * 1024);
+                    dma_load_at((yin >> i) & 1u ? (const void*)(ysrc + yv[i]) : (const void*)wd_zero16);
+                }
             }
-#pragma unroll
-            for(int i = 0; i < NLW; i++)
+            else
             {
-                dma_dst_at(dy, i * 1024);
-                dma_load(yv[i], ysrc);
+#pragma unroll
+                for(int i = 0; i < NLW; i++)
+                {
+                    dma_dst_at(dx, i * 1024);
+                    dma_load(xv[i], xsrc);
+                }
+#pragma unroll
+                for(int i = 0; i < NLW; i++)
+                {
+                    dma_dst_at(dy, i * 1024);
+                    dma_load(yv[i], ysrc);
+                }
             }
             lu++;
             ko   = wd_next_origin(ko, klast, BK);
@@ -469,7 +499,7 @@ namespace hiptk
         // (a tile is never moved back here.  Row-contiguous operands that would need it are not offered this
         // kernel; with k-contiguous ones the flag can only come from C / D's vectors, which the element-wise
         // epilogue does not use: an overhanging tile reads the row tables' padding and stores nothing there)
-        if(a.K < BK || a.K % BK != 0 || (!XKF && a.shift_p) || (!YKF && a.shift_q))
+        if(a.K < BK || ((XKF || YKF) && a.K % G::V != 0) || (!XKF && a.shift_p) || (!YKF && a.shift_q))
             return (int)hipErrorInvalidValue;
         auto                    kern = contract_wd_kernel<Tr, BK, NS, WK, XKF, YKF>;
         static const hipError_t attr = hipFuncSetAttribute(
@@ -482,7 +512,7 @@ namespace hiptk
     }
 }
 
-// Registry line of a direct-load tile: both operands in row-index vectors, one K stride, K a multiple of BK.
+// Registry line of a direct-load tile: both operands in row-index vectors, one K stride, any K from BK on.
 // (A class whose element fills the 16 bytes would have no vectors: every problem of it is described
 // as "scalar, k-fast", and any row table would do.)
 #define HIPTK_WD_ENTRY(TR, ID, BK, NS)                                                              \
@@ -490,7 +520,7 @@ namespace hiptk
         hiptk::TR::CLS, ID, hiptk::TR::VMAX == 1, hiptk::TR::VMAX == 1, hiptk::TR::VMAX,            \
             hiptk::TR::VMAX, 1, 64, 64, BK, 256,                                                    \
             hiptk::WdGeom<hiptk::TR, BK, NS, false>::LDS_BYTES, #TR "_64x64x" #BK "_direct" #NS,\
-            &hiptk::launch_wd<hiptk::TR, BK, NS, false, false, false>, BK                                         \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, false, false, false>, 1                                         \
     }
 
 // ... and of the 32 x 32 tile whose four waves split the K range between them.
@@ -499,7 +529,7 @@ namespace hiptk
         hiptk::TR::CLS, ID, hiptk::TR::VMAX == 1, hiptk::TR::VMAX == 1, hiptk::TR::VMAX,            \
             hiptk::TR::VMAX, 1, 32, 32, BK, 256,                                                    \
             hiptk::WdGeom<hiptk::TR, BK, NS, true>::LDS_BYTES, #TR "_32x32x" #BK "_direct" #NS "k4", \
-            &hiptk::launch_wd<hiptk::TR, BK, NS, true, false, false>, BK                                        \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, true, false, false>, 1                                        \
     }
 
 // ... and of both where X (XKF) and / or Y (YKF) are contiguous along k instead (16-byte vectors of k, one K stride).
@@ -508,12 +538,12 @@ namespace hiptk
         hiptk::TR::CLS, ID, XKF, YKF, hiptk::TR::VMAX, hiptk::TR::VMAX, 1, 64, 64, BK, 256,         \
             hiptk::WdGeom<hiptk::TR, BK, NS, false, XKF != 0, YKF != 0>::LDS_BYTES,                 \
             #TR "_64x64x" #BK "_direct" #NS "kf" #XKF #YKF,                                         \
-            &hiptk::launch_wd<hiptk::TR, BK, NS, false, XKF != 0, YKF != 0>, BK                     \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, false, XKF != 0, YKF != 0>, hiptk::TR::VMAX                     \
     }
 #define HIPTK_WK_ENTRY_KF(TR, ID, BK, NS, XKF, YKF)                                                 \
     {                                                                                               \
         hiptk::TR::CLS, ID, XKF, YKF, hiptk::TR::VMAX, hiptk::TR::VMAX, 1, 32, 32, BK, 256,         \
             hiptk::WdGeom<hiptk::TR, BK, NS, true, XKF != 0, YKF != 0>::LDS_BYTES,                  \
             #TR "_32x32x" #BK "_direct" #NS "k4kf" #XKF #YKF,                                       \
-            &hiptk::launch_wd<hiptk::TR, BK, NS, true, XKF != 0, YKF != 0>, BK                      \
+            &hiptk::launch_wd<hiptk::TR, BK, NS, true, XKF != 0, YKF != 0>, hiptk::TR::VMAX                     \
     }

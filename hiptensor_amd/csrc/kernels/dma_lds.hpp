@@ -43,6 +43,11 @@ namespace hiptk
     {
         asm volatile("s_nop 4\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
     }
+    // ... with a full address per lane (no scalar base): for loads some lanes of which must look elsewhere
+    __device__ __forceinline__ void dma_load_at(const void* lane_address)
+    {
+        asm volatile("s_nop 4\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(lane_address) : "memory");
+    }
     __device__ __forceinline__ void dma_load1(uint32_t voff, const void* base)
     {
         asm volatile("s_nop 4\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");

@@ -91,6 +91,14 @@ namespace hiptk
         return o;
     }
 
+    // A last K tile that holds only tail_k (< BK) k: does the vector at k-position `k` of the tile (V
+    // consecutive k of a row if kf, else V rows at that k) lie inside K?  The others are loaded from 16
+    // bytes of zeros instead, so the tile multiplies as a whole one.
+    HIPTK_HD_FN bool wd_tail_inside(bool kf, int k, int v, int tail_k)
+    {
+        return kf ? k + v <= tail_k : k < tail_k;
+    }
+
     // ... and where the four waves of a workgroup split a slice of n K tiles between them: wave w takes
     // `count` tiles from `first` on (none, for the last waves of a short slice).
     struct WdChunk

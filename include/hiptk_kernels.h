@@ -62,8 +62,8 @@ typedef struct hiptk_tile_info
     int32_t lds_bytes;  /* static LDS                                        */
     char    name[64];
     int32_t k_multiple; /* 0: operand tiles staged through registers, any K.  Otherwise the tile loads
-                           them straight into LDS: K must be a multiple of this and at least bk, and the
-                           problem xy_aligned                                  */
+                           them straight into LDS: K must be a multiple of this (1: any) and at least bk,
+                           and the problem xy_aligned                          */
 } hiptk_tile_info_t;
 
 typedef struct hiptk_problem

@@ -29,6 +29,7 @@ using hiptk::HdSlot;
 using hiptk::wd_next_origin;
 using hiptk::wd_slot;
 using hiptk::wd_slot_kf;
+using hiptk::wd_tail_inside;
 using hiptk::wd_wave_chunk;
 using hiptk::WdChunk;
 
@@ -266,6 +267,16 @@ static void check_wide_operand(const char* what, const Case& c, const GemmView& 
                 CHECK(lanepart <= 0xFFFFFFFFull, "%s %s lane offset overflows 32 bits", c.name.c_str(), what);
                 for(int o : origins)
                 {
+                    const int tail_k = (int)(v.K % BK);
+                    if(tail_k && o == (int)(v.K / BK) * BK)
+                    {
+                        // the short last tile: a vector is requested only if it lies inside K (else 16 bytes of zeros are)
+                        const bool in = wd_tail_inside(KF, sl.k, V, tail_k);
+                        CHECK(in == (o + sl.k + (KF ? V - 1 : 0) < v.K), "%s %s short tile: slot k %d of %d kept %d", c.name.c_str(), what, sl.k, tail_k, (int)in);
+                        CHECK(KF || !in || o + sl.k < v.K, "%s %s short tile row beyond K", c.name.c_str(), what);
+                        if(!in)
+                            continue;
+                    }
                     CHECK(o >= 0 && o + sl.k + (KF ? V - 1 : 0) < v.K, "%s %s k %d of %lld", c.name.c_str(), what, o + sl.k, (long long)v.K);
                     for(int j = 1; KF && j < V; j++)
                         CHECK(ktab[(size_t)(o + sl.k + j)] - ktab[(size_t)(o + sl.k)] == j, "%s %s k run broken at %d", c.name.c_str(), what, o + sl.k);
@@ -291,8 +302,8 @@ static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
     long      walked = 0;
     const int K      = (int)v.K;
     const int tiles_p = (int)((v.P + ROWS - 1) / ROWS), tiles_q = (int)((v.Q + ROWS - 1) / ROWS);
-    const int ktiles  = K / BK;
-    CHECK(K % BK == 0 && K >= BK, "%s K %d offered to K tiles of %d", c.name.c_str(), K, BK);
+    const int ktiles  = (K + BK - 1) / BK; // the last one may be short
+    CHECK(K >= BK, "%s K %d offered to K tiles of %d", c.name.c_str(), K, BK);
     for(int want = 1; want <= 7; want++)
     {
         int split = std::min(want, ktiles);
@@ -320,11 +331,11 @@ static long check_wide_tile(const Case& c, const GemmView& v, int BK, int NLW)
             int       ko    = kt_begin * BK;
             for(int u = 0; u < nt + 12; u++)
             {
-                CHECK(ko >= 0 && ko + BK <= K, "%s origin %d out of range", c.name.c_str(), ko);
+                CHECK(ko >= 0 && ko < K && (ko + BK <= K || ko == (K / BK) * BK), "%s origin %d out of range", c.name.c_str(), ko);
                 if(u < nt)
                 {
                     CHECK(ko == (kt_begin + u) * BK, "%s tile %d origin %d", c.name.c_str(), u, ko);
-                    for(int k = 0; k < BK; k++)
+                    for(int k = 0; k < BK && ko + k < K; k++)
                         covered[(size_t)(ko + k)]++;
                 }
                 else
@@ -464,6 +475,12 @@ int main()
     rank4("k24_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 42, 9, 25, 13, 8, 3);
     // odd row counts under k-contiguous operands: tiles overhang, C / D may ask for moved-back tiles, which these kernels do not do
     rank4("ragged_kfast", {20, 21, 0, 1}, {20, 21, 10, 11}, {10, 11, 0, 1}, 15, 19, 17, 21, 16, 9);
+    // K that ends inside a K tile: 100 = 6 x 16 + 4 = 12 x 8 + 4, 42 (not even a multiple of the f32 vector: row-contiguous only)
+    rank4("k100_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 40, 9, 24, 13, 20, 5);
+    rank4("k100_kfast", {20, 21, 0, 1}, {20, 21, 10, 11}, {10, 11, 0, 1}, 40, 9, 24, 13, 20, 5);
+    rank4("k100_mixed", {0, 1, 20, 21}, {20, 21, 10, 11}, {10, 11, 0, 1}, 40, 9, 24, 13, 20, 5);
+    rank4("k42_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 40, 9, 24, 13, 6, 7);
+    rank4("k42_kfast", {20, 21, 0, 1}, {20, 21, 10, 11}, {10, 11, 0, 1}, 40, 9, 24, 13, 6, 7);
     rank4("big_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 8192, 16, 64, 1, 64, 64);
     const WideTile wide[] = {{"f32", 0, 4, 4, 2, 16, 64}, {"f64", 1, 16, 8, 2, 8, 64}, {"c32", 4, 2048, 8, 2, 8, 64},
                              {"f32", 0, 4, 4, 3, 16, 32}, {"f64", 1, 16, 8, 3, 8, 32}, {"c32", 4, 2048, 8, 3, 8, 32}};
@@ -503,8 +520,8 @@ int main()
             if(!avail)
                 continue;
             const int V = 16 / w.elem_bytes;
-            CHECK(v.x_vec == V && v.y_vec == V && v.k_affine && v.K % w.bk == 0 && v.xy_aligned && (v.x_kfast || !v.shift_p)
-                      && (v.y_kfast || !v.shift_q),
+            CHECK(v.x_vec == V && v.y_vec == V && v.k_affine && v.K >= w.bk && (!(v.x_kfast || v.y_kfast) || v.K % V == 0) && v.xy_aligned
+                      && (v.x_kfast || !v.shift_p) && (v.y_kfast || !v.shift_q),
                   "%s %s offered outside its restrictions", w.type, c.name.c_str());
             offered_wide++;
             const int nlw = w.bk * w.rows * w.elem_bytes / (w.rows == 32 ? 1024 : 4096);

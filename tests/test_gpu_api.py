@@ -33,11 +33,11 @@ def test_patient_selection_matches_oracle(gpu_handle, oracle_mod):
 def test_split_k_and_workspace_contract(gpu_handle, oracle_mod):
     import torch
 
-    # small output, K = 248 (no multiple of the direct-load kernels' K tile, which run such sizes in one launch
-    # with the waves splitting K): the recommended plan splits K and needs workspace
-    ext = {0: 16, 1: 16, 10: 16, 11: 16, 20: 8, 21: 31}
-    w = wl.make_workload("f32", cases.COMPUTE["f32"], [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], ext, 1.5, 0.75,
-                         name="splitk_f32_256x256x248_kfast")
+    # small output, long K, complex f64 (a class without a single-launch kernel whose waves split K): the
+    # recommended plan splits K and needs workspace
+    ext = {0: 16, 1: 16, 10: 16, 11: 16, 20: 16, 21: 16}
+    w = wl.make_workload("c64", cases.COMPUTE["c64"], [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.5 + 0.5j, 0.75 - 0.25j,
+                         name="splitk_c64_256")
     inp = wl.host_inputs(w)
     exp = oracle_mod.contract(w, inp["A"], inp["B"], inp["C"])
     c = wl.Contraction(gpu_handle, w, pref=api.HIPTENSOR_WORKSPACE_RECOMMENDED)
@@ -51,10 +51,10 @@ def test_split_k_and_workspace_contract(gpu_handle, oracle_mod):
     st = c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(), None, workspace_bytes=0)
     assert st == api.HIPTENSOR_STATUS_INSUFFICIENT_WORKSPACE
     torch.cuda.synchronize()
-    assert np.all(np.isnan(D.cpu().numpy().view(np.float32)))
+    assert np.all(np.isnan(D.cpu().numpy().view(np.float64)))
     assert c.run(A.data_ptr(), B.data_ptr(), Cd.data_ptr(), D.data_ptr(), ws.data_ptr()) == 0
     torch.cuda.synchronize()
-    cases.assert_parity(w, D.cpu().numpy().view(np.float32), exp, "split-K")
+    cases.assert_parity(w, D.cpu().numpy().view(wl.NP_STORE[w["dtype"]]), exp, "split-K")
     c.close()
     # a plan made with no workspace runs single-pass and gives the same answer
     got, info = gpu_util.run_gpu(gpu_handle, w, inp, pref=api.HIPTENSOR_WORKSPACE_MIN, return_info=True)
@@ -153,10 +153,10 @@ def test_contraction_inside_a_hip_graph(gpu_handle, oracle_mod):
     # (the last two pin the kernels that load operand tiles straight into LDS: one K stride, single pass;
     # K offsets from tables with split-K)
     e3 = {0: 40, 1: 9, 10: 24, 11: 13, 20: 16, 21: 3, 22: 5}
-    k248 = {0: 16, 1: 16, 10: 16, 11: 16, 20: 8, 21: 31}
+    k16 = {0: 16, 1: 16, 10: 16, 11: 16, 20: 16, 21: 16}
     todo = [(wl.config1(), None),  # one launch: 32 x 32 tiles whose waves split K
-            (wl.make_workload("f32", cases.COMPUTE["f32"], [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], k248, 1.5, 0.75,
-                              name="graph_f32_256x256x248_kfast"), None),  # split-K by default: two kernels + workspace
+            (wl.make_workload("c64", cases.COMPUTE["c64"], [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], k16, 1.5 + 0.5j, 0.75 - 0.25j,
+                              name="graph_c64_256"), None),  # split-K by default: two kernels + workspace
             (wl._rank4("f16", cases.COMPUTE["f16"], (16, 12), (8, 20), (8, 24), 1.0, 0.5, "graph_f16"), None),
             (wl._rank4("f16", cases.COMPUTE["f16"], (40, 9), (24, 13), (16, 13), 1.0, 0.5, "graph_f16_direct"), "9,1"),
             (wl.make_workload("bf16", cases.COMPUTE["bf16"], [0, 1, 20, 21, 22], [20, 22, 21, 10, 11], [10, 11, 0, 1], e3, 1.5, 0.75,

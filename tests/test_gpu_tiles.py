@@ -112,8 +112,8 @@ def layouts(dtype, compute, big):
             out.append(wl.config5(extents=(32, 2, 8, 24, 2, 16, 5, 8, 10)))
             out.append(wl.config5(extents=(32, 2, 8, 24, 2, 16, 4, 8, 10)))
     if not big and compute == cases.COMPUTE[dtype]:
-        # The 32/64-bit kernels that load their operand tiles straight into LDS (row-fast operands in
-        # 16-byte vectors, one K stride, K a multiple of their K tile of 8 or 16; a ring of 4 or 8 tiles):
+        # The 32/64-bit kernels that load their operand tiles straight into LDS (operands in 16-byte vectors,
+        # one K stride, K tiles of 8 or 16; a ring of 4 or 8 tiles):
         # a single K tile, fewer tiles than the ring holds, exactly one ring, several rings with a
         # remainder; partial and whole 64 x 64 output tiles (complex f64 has no such kernel)
         for kk in ((8, 1), (16, 1), (16, 3), (16, 8), (16, 13), (16, 17)):
@@ -121,6 +121,21 @@ def layouts(dtype, compute, big):
             tag = f"k{kk[0] * kk[1]}"
             out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, b,
                                         name=f"tiles_{tag}_rowfast_{dtype}"))
+        # K that ends inside a K tile (the vectors of the last tile that lie beyond K are loaded from zeros):
+        # 100 on every operand layout, 42 and 17 (one k into the second tile of 16) on row-contiguous operands
+        dk = {0: 40, 1: 5, 10: 24, 11: 7, 20: 20, 21: 5}
+        out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, b,
+                                    name=f"tiles_k100_rowfast_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [20, 21, 0, 1], [20, 21, 10, 11], [10, 11, 0, 1], dk, a, None,
+                                    name=f"tiles_k100_kfast_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], dk, a, b,
+                                    name=f"tiles_k100_mixed_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [20, 21, 0, 1], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, b,
+                                    name=f"tiles_k100_mixed2_{dtype}"))
+        for kk in ((6, 7), (17, 1)):
+            dk = {0: 40, 1: 5, 10: 24, 11: 7, 20: kk[0], 21: kk[1]}
+            out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, b,
+                                        name=f"tiles_k{kk[0] * kk[1]}_rowfast_{dtype}"))
         dk = {0: 64, 1: 2, 10: 64, 11: 3, 20: 16, 21: 5}
         out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, None,
                                     name=f"tiles_k80_whole_tiles_{dtype}"))
@@ -186,8 +201,8 @@ def _tile_exists(cls, tile):
 def test_direct_load_tiles_on_random_layouts(gpu_handle, oracle_mod, dtype):
     """The 32/64-bit kernels that load operand tiles straight into LDS, on seeded random problems: two or
     three modes per group with extents from a small set, every operand packed with either its row modes or
-    its k modes fastest (all four combinations occur), D packed in a random mode order, K a multiple of 16,
-    scale and bilinear, complex scalars for complex data.  Each problem runs the default selection and both
+    its k modes fastest (all four combinations occur), D packed in a random mode order, K a multiple of 4 from
+    12 on (whole K tiles or not), scale and bilinear, complex scalars for complex data.  Each problem runs the default selection and both
     direct-load tile ids (64 x 64; 32 x 32 with the waves splitting K), the latter also with split-K 2, and
     is held against the oracle; a problem a tile is not offered for is skipped for that tile, and every
     (tile, operand layout) pair must have run at least once."""
@@ -201,7 +216,7 @@ def test_direct_load_tiles_on_random_layouts(gpu_handle, oracle_mod, dtype):
                 for i in range(cnt):
                     ext[base + i] = int(rng.choice([4, 8, 12, 20])) if i == 0 else int(rng.choice([3, 5, 6, 9]))
             for i in range(nk):
-                ext[20 + i] = 16 if i == 0 else int(rng.choice([1, 2, 3, 5]))
+                ext[20 + i] = int(rng.choice([16, 16, 20, 12])) if i == 0 else int(rng.choice([1, 2, 3, 5]))
             ms, ns, ks = ([b + i for i in range(c)] for b, c in ((0, nm), (10, nn), (20, nk)))
             a_kfast, b_kfast = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
             mA = ks + ms if a_kfast else ms + ks  # make_workload packs the first listed mode fastest
