@@ -1,5 +1,5 @@
 // complex f64 kernels (two v_mfma_f64_16x16x4_f64 per two complex k).
-#include "contract_w.hpp"
+#include "contract_wd.hpp"
 
 namespace hiptk
 {
@@ -9,6 +9,9 @@ namespace hiptk
         HIPTK_W_TILE(WTraitsC64, 0, 64, 64, 16, 4, 2),
         HIPTK_W_TILE(WTraitsC64, 1, 32, 32, 8, 2, 2),
         HIPTK_W_TILE(WTraitsC64, 2, 32, 32, 16, 2, 2),
+        // (one element per 16-byte vector: every layout with one K stride is "k-contiguous, vectors of one")
+        HIPTK_WD_ENTRY_KF(WTraitsC64, 3, 8, 4, 1, 1),
+        HIPTK_WK_ENTRY_KF(WTraitsC64, 4, 8, 4, 1, 1),
     };
 
     const KernelEntry* entries_c64(int* count)

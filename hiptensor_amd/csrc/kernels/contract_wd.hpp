@@ -1,10 +1,9 @@
-// 32/64-bit (f32, f64, complex f32) contraction kernel for gfx950 whose operand tiles go from global
+// 32/64-bit (f32, f64, complex f32, complex f64) contraction kernel for gfx950 whose operand tiles go from global
 // memory straight into LDS (global_load_lds_dwordx4), for operands that are each contiguous along
 // their row index (both: packed column-major, every benchmark configuration of these types; described
 // below) or along k (both: packed row-major, what NULL strides mean; the differences are at wd_slot_kf
-// in hd_addr.hpp and at read_op).  (Complex f64 is not instantiated: two K
-// tiles of its operands do not fit the registers, and without them it measured 8 % behind the
-// eight-wave tile of contract_w.hpp.)
+// in hd_addr.hpp and at read_op).  (Complex f64, one element per 16-byte
+// vector, runs the k-contiguous form on any layout with one K stride.)
 //
 // Same MFMA use, complex product and epilogue as contract_w.hpp; what differs is how a tile gets
 // into LDS and from there into registers.  There, a gather passes through registers and has one K
@@ -312,8 +311,10 @@ namespace hiptk
 
         // C and the C / D offsets of the wave tile this wave will store (with waves that split K: wave 0,
         // all of the tile), unless the launch is a split-K slice, which stores partial sums
+        // (complex f64 has no registers for it: 64 for its C elements beside 96 of accumulators and 64 of operands)
+        constexpr bool EARLY_C = TP * TQ * Tr::NREG * sizeof(typename Tr::E) <= 128;
         WdEpilogue<Tr, TP, TQ> epi;
-        const bool             whole_k = a.split_k == 1;
+        const bool             whole_k = EARLY_C && a.split_k == 1;
         const bool             storer  = !WK || wave == 0;
         if(whole_k && storer)
             epi.fetch(a, p0 + wp * 32, q0 + wq * 32 + Tr::q_of(lane), p0, q0, lane);

@@ -483,7 +483,8 @@ int main()
     rank4("k42_kfast", {20, 21, 0, 1}, {20, 21, 10, 11}, {10, 11, 0, 1}, 40, 9, 24, 13, 6, 7);
     rank4("big_rowfast", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 8192, 16, 64, 1, 64, 64);
     const WideTile wide[] = {{"f32", 0, 4, 4, 2, 16, 64}, {"f64", 1, 16, 8, 2, 8, 64}, {"c32", 4, 2048, 8, 2, 8, 64},
-                             {"f32", 0, 4, 4, 3, 16, 32}, {"f64", 1, 16, 8, 3, 8, 32}, {"c32", 4, 2048, 8, 3, 8, 32}};
+                             {"f32", 0, 4, 4, 3, 16, 32}, {"f64", 1, 16, 8, 3, 8, 32}, {"c32", 4, 2048, 8, 3, 8, 32},
+                             {"c64", 5, 4096, 16, 3, 8, 64}, {"c64", 5, 4096, 16, 4, 8, 32}};
     int offered_wide = 0, refused_big = 0, offered_kf = 0, offered_mixed = 0;
     for(const WideTile& w : wide)
         for(const Case& c : cases)
@@ -528,9 +529,13 @@ int main()
             offered_kf += (v.x_kfast || v.y_kfast) ? 1 : 0;
             offered_mixed += (v.x_kfast != v.y_kfast) ? 1 : 0;
             if(w.rows == 64)
-                walked += V == 4 ? check_wide_tile<4, 64>(c, v, w.bk, nlw) : check_wide_tile<2, 64>(c, v, w.bk, nlw);
+                walked += V == 4   ? check_wide_tile<4, 64>(c, v, w.bk, nlw)
+                          : V == 2 ? check_wide_tile<2, 64>(c, v, w.bk, nlw)
+                                   : check_wide_tile<1, 64>(c, v, w.bk, nlw);
             else
-                walked += V == 4 ? check_wide_tile<4, 32>(c, v, w.bk, nlw) : check_wide_tile<2, 32>(c, v, w.bk, nlw);
+                walked += V == 4   ? check_wide_tile<4, 32>(c, v, w.bk, nlw)
+                          : V == 2 ? check_wide_tile<2, 32>(c, v, w.bk, nlw)
+                                   : check_wide_tile<1, 32>(c, v, w.bk, nlw);
         }
     g_dtype = 2;
     CHECK(offered_mixed >= 30, "only %d mixed (case, type, tile) triples were offered a 32/64-bit direct-load kernel", offered_mixed);
