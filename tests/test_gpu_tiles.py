@@ -197,7 +197,7 @@ def _tile_exists(cls, tile):
     return lib.hiptk_tile_info(cls, tile, ctypes.byref(ti)) == 0
 
 
-@pytest.mark.parametrize("dtype", ["f32", "f64", "c32"])
+@pytest.mark.parametrize("dtype", ["f32", "f64", "c32", "c64"])
 def test_direct_load_tiles_on_random_layouts(gpu_handle, oracle_mod, dtype):
     """The 32/64-bit kernels that load operand tiles straight into LDS, on seeded random problems: two or
     three modes per group with extents from a small set, every operand packed with either its row modes or
@@ -205,8 +205,10 @@ def test_direct_load_tiles_on_random_layouts(gpu_handle, oracle_mod, dtype):
     12 on (whole K tiles or not), scale and bilinear, complex scalars for complex data.  Each problem runs the default selection and both
     direct-load tile ids (64 x 64; 32 x 32 with the waves splitting K), the latter also with split-K 2, and
     is held against the oracle; a problem a tile is not offered for is skipped for that tile, and every
-    (tile, operand layout) pair must have run at least once."""
-    rng = np.random.default_rng({"f32": 11, "f64": 12, "c32": 13}[dtype])
+    (tile, operand layout) pair must have run at least once (complex f64, one element per vector, is described as
+    k-contiguous on every layout; its direct-load tiles are ids 3 and 4)."""
+    rng = np.random.default_rng({"f32": 11, "f64": 12, "c32": 13, "c64": 14}[dtype])
+    forces = ("3,1", "4,1", "4,2") if dtype == "c64" else ("2,1", "3,1", "3,2")
     ran = set()
     try:
         for n in range(16):
@@ -222,7 +224,7 @@ def test_direct_load_tiles_on_random_layouts(gpu_handle, oracle_mod, dtype):
             mA = ks + ms if a_kfast else ms + ks  # make_workload packs the first listed mode fastest
             mB = ks + ns if b_kfast else ns + ks
             mD = ms + ns if rng.integers(0, 2) else ns + ms
-            if dtype == "c32":
+            if dtype in ("c32", "c64"):
                 alpha, beta = complex(rng.uniform(-2, 2), rng.uniform(-2, 2)), (None if n % 3 == 0 else complex(rng.uniform(-2, 2), rng.uniform(-2, 2)))
             else:
                 alpha, beta = float(rng.uniform(-2, 2)), (None if n % 3 == 0 else float(rng.uniform(-2, 2)))
@@ -230,7 +232,7 @@ def test_direct_load_tiles_on_random_layouts(gpu_handle, oracle_mod, dtype):
                                  name=f"random_{dtype}_{n}_{'k' if a_kfast else 'r'}{'k' if b_kfast else 'r'}")
             inp = wl.host_inputs(w)
             exp = cases.logical_view(w, oracle_mod.contract(w, inp["A"], inp["B"], inp["C"]))
-            for force in (None, "2,1", "3,1", "3,2"):
+            for force in (None,) + forces:
                 if force:
                     os.environ["HIPTENSOR_AMD_FORCE_KERNEL"] = force
                 else:
@@ -247,4 +249,4 @@ def test_direct_load_tiles_on_random_layouts(gpu_handle, oracle_mod, dtype):
     finally:
         os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
     print("ran:", sorted(ran), flush=True)
-    assert len({r[0] for r in ran}) == 3 and len({(r[1], r[2]) for r in ran}) >= 3, sorted(ran)
+    assert len({r[0] for r in ran}) == 3 and len({(r[1], r[2]) for r in ran}) >= (1 if dtype == "c64" else 3), sorted(ran)
