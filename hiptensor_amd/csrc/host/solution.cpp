@@ -150,7 +150,8 @@ namespace hipta
             case HIPTK_C64:
                 // (2048^2 x 1024: 527 us on either tile; 1920^2 x 768: 406 us on 900 tiles of 64 x 64, 375 us on
                 // 3600 of 32 x 32; 512^3, one tile per CU: 74.8 us on 64 of the one, 26.6 us on 256 of the other)
-                return area >= 4096 ? TileRate{0.70, 0.82} : TileRate{0.50, 0.82};
+                // (1024^2 x 512, four 32 x 32 tiles per CU: 75.2 us; 512^3 in two slices 28.7)
+                return area >= 4096 ? TileRate{0.70, 0.82} : TileRate{0.50, 0.78};
             // (128 x 128 on 4096 x 4096 x 512, four tiles per CU: complex f32 535 us, f32 140.5 us; complex f32 on
             // 64 x 64: 1024^2 x 512 in one pass 50.7 us, 3072 x 1024 x 1024 203.6 us)
             case HIPTK_C32: return area >= 16384 ? TileRate{0.84, 0.86} : TileRate{0.62, 0.82};
@@ -220,8 +221,9 @@ namespace hipta
                 break;
             case HIPTK_C32: r = big ? (kf ? TileRate{0.88, 0.90} : TileRate{0.90, 0.91}) : (kf ? TileRate{0.85, 0.88} : TileRate{0.90, 0.91}); break;
             // (complex f64, one element per vector: 2048^2 x 1024 478 us on 64 x 64 against 525 staged, 1024^2 x 512 71.9;
-            // on 32 x 32 tiles 512^3 24.9 us, 1024^2 x 512 92.7)
-            case HIPTK_C64: r = big ? TileRate{0.85, 0.91} : TileRate{0.50, 0.55}; break;
+            // on 32 x 32 tiles 512^3, one workgroup per CU, 24.0 us (28.7 on the staged tile in two slices); 1024^2 x 512,
+            // four per CU, 92.7)
+            case HIPTK_C64: r = big ? TileRate{0.85, 0.91} : TileRate{0.85, 0.70}; break;
             default: break;
             }
             // ... whose prologue (tables, then the first tiles' flight) and epilogue nothing overlaps when a
@@ -230,7 +232,9 @@ namespace hipta
             // slice shorter than the ring has less in flight to wait for); the 32 x 32 tile adds its partial
             // tiles through LDS (640^2 x 64 f32: 8.4 us against 6.3 on 64 x 64 tiles)
             // (k-contiguous: 8.6 against 6.5 us)
-            round_extra_us = 2.0 * std::min(1.0, kper / s.bk / 16.0) + (big ? 0.0 : (v.x_kfast || v.y_kfast) ? 2.5 : 1.0);
+            // (complex f64 is "k-contiguous" on every layout: one element per vector)
+            const bool short_runs = (v.x_kfast || v.y_kfast) && v.cls != HIPTK_C64;
+            round_extra_us        = 2.0 * std::min(1.0, kper / s.bk / 16.0) + (big ? 0.0 : short_runs ? 2.5 : 1.0);
         }
         if(class_max_vec(v.cls) > 1)
         {
@@ -244,7 +248,9 @@ namespace hipta
             r.alone *= f;
             r.full *= f;
         }
-        const double frac     = std::min(sharing * r.alone, r.full);
+        // (a workgroup that has its CU to itself runs at `alone`, which for waves that never meet at a barrier can
+        // be above what two such workgroups reach together)
+        const double frac     = sharing <= 1.0 ? r.alone : std::min(sharing * r.alone, r.full);
         const double flops_wg = class_flops_per_mac(v.cls) * (double)s.bp * s.bq * kper;
         const double cu_rate  = class_flops_per_clk_cu(v.cls) * dev.clock_ghz * 1e3; // flop / us
         double       us       = per_cu * flops_wg / (frac * cu_rate);
