@@ -146,7 +146,10 @@ namespace hipta
             case HIPTK_F64:
                 // (the 64 x 64 tile runs on eight waves, 16 x 32 outputs each: alone on a CU it reaches 0.64 of
                 // nominal on 1024^3 f64 against 0.53 on four waves; 1920^2 x 768: 104.9 against 108.1 us)
-                return area >= 16384 ? TileRate{0.76, 0.76} : TileRate{0.60, 0.78};
+                // (many short tiles per CU, 4096^2 x 512: 128 x 128 258-265 us on k-contiguous operands, 296-314 on
+                // row-contiguous ones (estimate_us), 64 x 64 269-273, where the direct-load 64 x 64 tile, whose prologue
+                // nothing overlaps, needs 280-294)
+                return area >= 16384 ? TileRate{0.83, 0.83} : TileRate{0.60, 0.80};
             case HIPTK_C64:
                 // (2048^2 x 1024: 527 us on either tile; 1920^2 x 768: 406 us on 900 tiles of 64 x 64, 375 us on
                 // 3600 of 32 x 32; 512^3, one tile per CU: 74.8 us on 64 of the one, 26.6 us on 256 of the other)
@@ -174,6 +177,8 @@ namespace hipta
         const double sharing = std::min<double>(resident, per_cu);
         TileRate     r       = tile_rate(v.cls, s.bp * s.bq);
         double round_extra_us = 0.0;
+        if(v.cls == HIPTK_F64 && s.bp * s.bq >= 16384 && !(v.x_kfast && v.y_kfast))
+            r = TileRate{0.74, 0.74};
         if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152 && s.bk == 32)
         {
             // The 256 x 256 and 256 x 192 tiles whose operand tiles are loaded straight into LDS (four waves,
@@ -216,7 +221,7 @@ namespace hipta
             case HIPTK_F32: r = big ? (kf ? TileRate{0.75, 0.78} : TileRate{0.81, 0.89}) : (kf ? TileRate{0.55, 0.60} : TileRate{0.65, 0.70}); break;
             // (one operand k-contiguous, 1024^2 x 2048 f64 on 32 x 32: 82.9 against 70.8 us)
             case HIPTK_F64:
-                r = big ? (kf ? TileRate{0.80, 0.84} : TileRate{0.82, 0.90})
+                r = big ? (kf ? TileRate{0.84, 0.88} : TileRate{0.82, 0.90})
                         : (kf ? TileRate{0.45, 0.50} : (v.x_kfast || v.y_kfast) ? TileRate{0.62, 0.66} : TileRate{0.82, 0.90});
                 break;
             case HIPTK_C32: r = big ? (kf ? TileRate{0.88, 0.90} : TileRate{0.90, 0.91}) : (kf ? TileRate{0.85, 0.88} : TileRate{0.90, 0.91}); break;

@@ -24,6 +24,12 @@
 //     readers each wave waits until only the loads of the NS - 2 tiles after it are outstanding.
 //     Tiles requested beyond the K range are not branched around: they re-read the last tile into
 //     spare LDS behind the ring, so every wait sees the same number of younger loads.
+//   * Nothing but MFMAs, loads, LDS reads and scalar instructions in a step: a vector instruction between
+//     the MFMAs waits for the matrix pipe, and a branch cuts the step into blocks.  So the LDS address of
+//     every read is a register that was set before the loop plus an offset that fits the instruction
+//     (`xat`, `yat`), and each kernel is instantiated twice: for K a multiple of BK, and with the test for
+//     a short last K tile in its steps (launch_wd picks).  With the address additions in the loop
+//     1920 x 1920 x 768 f64 took 107.7 us, without them 100.5, without the test 98.0.
 //
 // Restrictions (the dispatcher checks them): both operands gathered in 16-byte vectors, along their
 // row index or along k, on 16-byte boundaries; one K stride per operand; K at least BK (a last tile
@@ -79,6 +85,18 @@ namespace hiptk
 
     // what the vectors of a short last K tile that lie beyond K are loaded from
     static __device__ __attribute__((aligned(16))) const unsigned char wd_zero16[16] = {0};
+
+    // sizeof(T) = 4, 8 or 16 bytes of LDS at byte address `at` (a multiple of that size)
+    template <typename T>
+    __device__ __forceinline__ T lds_read(uint32_t at)
+    {
+        typedef uint32_t __attribute__((ext_vector_type(sizeof(T) / 4))) R;
+        typedef __attribute__((address_space(3))) R                      RL;
+        const R r = *(const RL*)(uintptr_t)at;
+        T       t;
+        __builtin_memcpy(&t, &r, sizeof(T));
+        return t;
+    }
 
     __device__ __forceinline__ float   wd_add(float x, float y) { return __fadd_rn(x, y); }
     __device__ __forceinline__ double  wd_add(double x, double y) { return __dadd_rn(x, y); }
@@ -187,7 +205,9 @@ namespace hiptk
         }
     }
 
-    template <typename Tr, int BK, int NS, bool WK, bool XKF, bool YKF>
+    // TAIL: K need not be a multiple of BK.  (The test for the short last tile is a branch in every step of the
+    // main loop, which costs 2-5 %: problems without such a tile run the instantiation without it.)
+    template <typename Tr, int BK, int NS, bool WK, bool XKF, bool YKF, bool TAIL>
     __global__ void __launch_bounds__(256, 2) contract_wd_kernel(const KArgs a)
     {
         typedef WdGeom<Tr, BK, NS, WK, XKF, YKF> G;
@@ -232,7 +252,7 @@ namespace hiptk
 
         // this lane's 16 bytes of each of its loads, as byte offsets from the tile's k origin; and, bit i,
         // whether load i of a short last tile lies inside K
-        const int tail_k      = a.K % BK;
+        const int tail_k      = TAIL ? a.K % BK : 0;
         const int tail_origin = tail_k ? (kt_all - 1) * BK : -1;
         uint32_t  xin = 0, yin = 0;
         uint32_t  xv[NLW], yv[NLW];
@@ -271,7 +291,7 @@ namespace hiptk
             const bool     real = lu < nt;
             const uint32_t dx   = real ? wdx + ST * G::STAGE_BYTES : wspare;
             const uint32_t dy   = real ? wdy + ST * G::STAGE_BYTES : wspare;
-            if(ko == tail_origin)
+            if(TAIL && ko == tail_origin)
             {
                 // the short last tile (or a repeat of it): the same number of loads, each lane from where its
                 // vector lies if that is inside K, else from zeros: the tile then multiplies as a whole one
@@ -350,17 +370,28 @@ namespace hiptk
         };
         // one operand's part of it: KF: a vector of V k-steps' elements when ks is the first of them; else one
         // element, at k-slot distance 1 or (next to a k-contiguous operand) V
-        auto read_op = [&](auto kf_c, const unsigned char* base, int fo, S (&dst)[KS][TP], int ks) {
+        // (`at`: the LDS byte address of this lane's first element of the operand's stage, and the addresses every
+        // PIN_BYTES behind it)
+        // (2048: what the offset field of a paired 8-byte read spans; complex f64 has no registers for them)
+        constexpr bool PINNED    = sizeof(S) < 16;
+        constexpr int  PIN_BYTES = PINNED ? 2048 : (1 << 30);
+        constexpr int  PINS      = G::OP_BYTES > PIN_BYTES ? G::OP_BYTES / PIN_BYTES : 1;
+        // (not PINNED: `base`, the operand's stage, and `fo`, the lane's first element in it)
+        auto read_op = [&](auto kf_c, const uint32_t (&at)[PINS], const unsigned char* base, int fo, S (&dst)[KS][TP], int ks) {
             static_assert(TP == TQ, "one reader for both operands");
             if constexpr(decltype(kf_c)::value)
             {
                 if(ks % G::V != 0)
                     return;
-                const SVec* l = (const SVec*)base;
 #pragma unroll
                 for(int i = 0; i < TP; i++)
                 {
-                    const SVec v = l[fo + (ks / G::V) * Tr::KM * ROWS + i * TILE];
+                    const int off = ((ks / G::V) * Tr::KM * ROWS + i * TILE) * (int)sizeof(SVec);
+                    SVec      v;
+                    if constexpr(PINNED)
+                        v = lds_read<SVec>(at[off / PIN_BYTES] + (uint32_t)(off % PIN_BYTES));
+                    else
+                        v = ((const SVec*)base)[fo + (ks / G::V) * Tr::KM * ROWS + i * TILE];
 #pragma unroll
                     for(int j = 0; j < G::V; j++)
                         dst[ks + j][i] = v.e[j];
@@ -368,17 +399,38 @@ namespace hiptk
             }
             else
             {
-                const S*  l  = (const S*)base;
                 const int k0 = VAPART ? ((ks / G::V) * Tr::KM * G::V + ks % G::V) : ks * Tr::KM;
 #pragma unroll
                 for(int i = 0; i < TP; i++)
-                    dst[ks][i] = l[fo + k0 * ROWS + i * TILE];
+                {
+                    const int off = (k0 * ROWS + i * TILE) * (int)sizeof(S);
+                    if constexpr(PINNED)
+                        dst[ks][i] = lds_read<S>(at[off / PIN_BYTES] + (uint32_t)(off % PIN_BYTES));
+                    else
+                        dst[ks][i] = ((const S*)base)[fo + k0 * ROWS + i * TILE];
+                }
             }
         };
+        // Those addresses, per ring stage, in registers of their own that the compiler cannot tell apart from
+        // any other value: it would otherwise add the stage's offset before every read, and a vector
+        // instruction between the MFMAs waits for the matrix pipe.  Every read is then one of them plus an offset
+        // that fits the instruction.
+        uint32_t xat[NS][PINS], yat[NS][PINS];
+#pragma unroll
+        for(int st = 0; st < NS; st++)
+#pragma unroll
+            for(int pin = 0; pin < PINS; pin++)
+            {
+                const uint32_t stage = (uint32_t)(uintptr_t)(lds_u8_ptr)ring + st * G::STAGE_BYTES + pin * PIN_BYTES;
+                xat[st][pin]         = stage + (uint32_t)xfo * (uint32_t)(XKF ? sizeof(SVec) : sizeof(S));
+                yat[st][pin]         = stage + G::OP_BYTES + (uint32_t)yfo * (uint32_t)(YKF ? sizeof(SVec) : sizeof(S));
+                if constexpr(PINNED)
+                    asm volatile("" : "+v"(xat[st][pin]), "+v"(yat[st][pin]));
+            }
         auto read_k = [&](auto st_c, Frags& f, int ks) {
             constexpr int ST = decltype(st_c)::value;
-            read_op(std::integral_constant<bool, XKF>{}, ring + ST * G::STAGE_BYTES, xfo, f.x, ks);
-            read_op(std::integral_constant<bool, YKF>{}, ring + ST * G::STAGE_BYTES + G::OP_BYTES, yfo, f.y, ks);
+            read_op(std::integral_constant<bool, XKF>{}, xat[ST], ring + ST * G::STAGE_BYTES, xfo, f.x, ks);
+            read_op(std::integral_constant<bool, YKF>{}, yat[ST], ring + ST * G::STAGE_BYTES + G::OP_BYTES, yfo, f.y, ks);
         };
         auto read_tile = [&](auto st_c, Frags& f) {
 #pragma unroll
@@ -502,13 +554,16 @@ namespace hiptk
         // epilogue does not use: an overhanging tile reads the row tables' padding and stores nothing there)
         if(a.K < BK || ((XKF || YKF) && a.K % G::V != 0) || (!XKF && a.shift_p) || (!YKF && a.shift_q))
             return (int)hipErrorInvalidValue;
-        auto                    kern = contract_wd_kernel<Tr, BK, NS, WK, XKF, YKF>;
-        static const hipError_t attr = hipFuncSetAttribute(
-            (const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
-        if(attr != hipSuccess)
-            return (int)attr;
+        auto whole = contract_wd_kernel<Tr, BK, NS, WK, XKF, YKF, false>;
+        auto tail  = contract_wd_kernel<Tr, BK, NS, WK, XKF, YKF, true>;
+        static const hipError_t attr_whole = hipFuncSetAttribute(
+            (const void*)whole, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
+        static const hipError_t attr_tail = hipFuncSetAttribute(
+            (const void*)tail, hipFuncAttributeMaxDynamicSharedMemorySize, G::LDS_BYTES);
+        if(attr_whole != hipSuccess || attr_tail != hipSuccess)
+            return (int)(attr_whole != hipSuccess ? attr_whole : attr_tail);
         dim3 grid(a.tiles_p * a.tiles_q, 1, a.split_k);
-        hipLaunchKernelGGL(kern, grid, dim3(256), G::LDS_BYTES, stream, a);
+        hipLaunchKernelGGL(a.K % BK == 0 ? whole : tail, grid, dim3(256), G::LDS_BYTES, stream, a);
         return (int)hipGetLastError();
     }
 }
