@@ -1,0 +1,79 @@
+"""What the compiler made of the hand-ordered main loops of the direct-load kernels (no GPU needed).
+
+A step of those loops is meant to hold nothing but MFMAs, direct loads, LDS reads, waits, the barrier and
+scalar instructions: a vector instruction between f64 MFMAs waits for the matrix pipe, and a branch cuts the
+step into blocks the MFMAs do not overlap.  Neither shows in a parity test, and both have happened (LDS read
+addresses recomputed before every read; the test for a short last K tile in every step): configuration 3
+took 107.7 instead of 98 us.  So the device assembly of the instantiations the benchmark configurations run
+is checked here: the loop that holds the MFMAs of a whole ring of K tiles has no vector ALU instruction and
+no branch but its own."""
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+KDIR = os.path.join(ROOT, "hiptensor_amd", "csrc", "kernels")
+
+
+def device_asm(unit, tmp_path):
+    out = tmp_path / (unit + ".s")
+    subprocess.run(["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+                    "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-option-ignored",
+                    "-I" + os.path.join(ROOT, "include"), "-I" + KDIR, "--cuda-device-only", "-S", "-o", str(out),
+                    os.path.join(KDIR, unit + ".hip")], check=True, capture_output=True)
+    return out.read_text().split("\n")
+
+
+def kernel_body(lines, symbol):
+    start = next(i for i, l in enumerate(lines) if l.startswith(symbol + ":"))
+    end = next(i for i in range(start, len(lines)) if "s_endpgm" in lines[i])
+    return lines[start:end]
+
+
+def main_loops(body, min_mfma):
+    """(first, last) line of every loop (label ... backward conditional branch to it) with at least min_mfma MFMAs
+    that holds no other such loop."""
+    labels = {m.group(1): i for i, l in enumerate(body) if (m := re.match(r"^(\.LBB\d+_\d+):", l))}
+    loops = []
+    for i, l in enumerate(body):
+        m = re.search(r"s_cbranch_\w+\s+(\.LBB\d+_\d+)", l)
+        if m and labels.get(m.group(1), i) < i:
+            a = labels[m.group(1)]
+            if sum("v_mfma" in x for x in body[a:i]) >= min_mfma:
+                loops.append((a, i))
+    return [(a, b) for a, b in loops if not any((c, d) != (a, b) and a <= c and d <= b for c, d in loops)]
+
+
+def opcodes(body, a, b):
+    ops = []
+    for l in body[a:b]:
+        t = l.strip().split()
+        if t and not t[0].startswith((";", ".", "#")) and not t[0].endswith(":"):
+            ops.append(t[0])
+    return ops
+
+
+CASES = [
+    # configuration 3: f64, 64 x 64 tile, K tiles of 8, ring of 8, row-contiguous operands, K a multiple of the K tile
+    ("contract_f64", "_ZN5hiptk18contract_wd_kernelINS_10WTraitsF64ELi8ELi8ELb0ELb0ELb0ELb0EEEvNS_5KArgsE", 8 * 8),
+    # configuration 4: complex f32, the same geometry (four k-steps a tile, four MFMAs per complex product)
+    ("contract_c32", "_ZN5hiptk18contract_wd_kernelINS_10WTraitsC32ELi8ELi8ELb0ELb0ELb0ELb0EEEvNS_5KArgsE", 8 * 4 * 4),
+    # configuration 2: f16, 256 x 256 tile, both operands row-contiguous, one K stride
+    ("contract_f16_hd", "_ZN5hiptk18contract_hd_kernelINS_9TraitsF16ELb0ELb0ELi256ELb1EEEvNS_5KArgsE", 128),
+]
+
+
+@pytest.mark.parametrize("unit,symbol,mfmas", CASES, ids=[c[0] for c in CASES])
+def test_main_loop_is_mfma_loads_and_scalar_only(tmp_path, unit, symbol, mfmas):
+    body = kernel_body(device_asm(unit, tmp_path), symbol)
+    loops = main_loops(body, mfmas)
+    assert loops, "no loop with %d MFMAs found: the ring is no longer unrolled as one loop" % mfmas
+    for a, b in loops:
+        ops = opcodes(body, a, b)
+        assert sum(o.startswith("v_mfma") for o in ops) == mfmas, (a, b, sum(o.startswith("v_mfma") for o in ops))
+        valu = sorted({o for o in ops if o.startswith("v_") and not o.startswith("v_mfma")})
+        assert not valu, f"vector ALU instructions in the main loop of {symbol}: {valu}"
+        assert not any(o.startswith(("s_cbranch", "s_branch")) for o in ops), "a branch inside the main loop"
+        assert not any(o.startswith(("scratch_", "buffer_store", "global_store")) for o in ops), "stores or spills in the main loop"
