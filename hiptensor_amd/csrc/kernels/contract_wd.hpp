@@ -371,13 +371,10 @@ namespace hiptk
         // one operand's part of it: KF: a vector of V k-steps' elements when ks is the first of them; else one
         // element, at k-slot distance 1 or (next to a k-contiguous operand) V
         // (`at`: the LDS byte address of this lane's first element of the operand's stage, and the addresses every
-        // PIN_BYTES behind it)
-        // (2048: what the offset field of a paired 8-byte read spans; complex f64 has no registers for them)
-        constexpr bool PINNED    = sizeof(S) < 16;
-        constexpr int  PIN_BYTES = PINNED ? 2048 : (1 << 30);
-        constexpr int  PINS      = G::OP_BYTES > PIN_BYTES ? G::OP_BYTES / PIN_BYTES : 1;
-        // (not PINNED: `base`, the operand's stage, and `fo`, the lane's first element in it)
-        auto read_op = [&](auto kf_c, const uint32_t (&at)[PINS], const unsigned char* base, int fo, S (&dst)[KS][TP], int ks) {
+        // PIN_BYTES behind it: what the offset field of a paired 8-byte read spans)
+        constexpr int PIN_BYTES = 2048;
+        constexpr int PINS      = G::OP_BYTES > PIN_BYTES ? G::OP_BYTES / PIN_BYTES : 1;
+        auto read_op = [&](auto kf_c, const uint32_t (&at)[PINS], S (&dst)[KS][TP], int ks) {
             static_assert(TP == TQ, "one reader for both operands");
             if constexpr(decltype(kf_c)::value)
             {
@@ -386,12 +383,8 @@ namespace hiptk
 #pragma unroll
                 for(int i = 0; i < TP; i++)
                 {
-                    const int off = ((ks / G::V) * Tr::KM * ROWS + i * TILE) * (int)sizeof(SVec);
-                    SVec      v;
-                    if constexpr(PINNED)
-                        v = lds_read<SVec>(at[off / PIN_BYTES] + (uint32_t)(off % PIN_BYTES));
-                    else
-                        v = ((const SVec*)base)[fo + (ks / G::V) * Tr::KM * ROWS + i * TILE];
+                    const int  off = ((ks / G::V) * Tr::KM * ROWS + i * TILE) * (int)sizeof(SVec);
+                    const SVec v   = lds_read<SVec>(at[off / PIN_BYTES] + (uint32_t)(off % PIN_BYTES));
 #pragma unroll
                     for(int j = 0; j < G::V; j++)
                         dst[ks + j][i] = v.e[j];
@@ -404,10 +397,7 @@ namespace hiptk
                 for(int i = 0; i < TP; i++)
                 {
                     const int off = (k0 * ROWS + i * TILE) * (int)sizeof(S);
-                    if constexpr(PINNED)
-                        dst[ks][i] = lds_read<S>(at[off / PIN_BYTES] + (uint32_t)(off % PIN_BYTES));
-                    else
-                        dst[ks][i] = ((const S*)base)[fo + k0 * ROWS + i * TILE];
+                    dst[ks][i]    = lds_read<S>(at[off / PIN_BYTES] + (uint32_t)(off % PIN_BYTES));
                 }
             }
         };
@@ -424,13 +414,12 @@ namespace hiptk
                 const uint32_t stage = (uint32_t)(uintptr_t)(lds_u8_ptr)ring + st * G::STAGE_BYTES + pin * PIN_BYTES;
                 xat[st][pin]         = stage + (uint32_t)xfo * (uint32_t)(XKF ? sizeof(SVec) : sizeof(S));
                 yat[st][pin]         = stage + G::OP_BYTES + (uint32_t)yfo * (uint32_t)(YKF ? sizeof(SVec) : sizeof(S));
-                if constexpr(PINNED)
-                    asm volatile("" : "+v"(xat[st][pin]), "+v"(yat[st][pin]));
+                asm volatile("" : "+v"(xat[st][pin]), "+v"(yat[st][pin]));
             }
         auto read_k = [&](auto st_c, Frags& f, int ks) {
             constexpr int ST = decltype(st_c)::value;
-            read_op(std::integral_constant<bool, XKF>{}, xat[ST], ring + ST * G::STAGE_BYTES, xfo, f.x, ks);
-            read_op(std::integral_constant<bool, YKF>{}, yat[ST], ring + ST * G::STAGE_BYTES + G::OP_BYTES, yfo, f.y, ks);
+            read_op(std::integral_constant<bool, XKF>{}, xat[ST], f.x, ks);
+            read_op(std::integral_constant<bool, YKF>{}, yat[ST], f.y, ks);
         };
         auto read_tile = [&](auto st_c, Frags& f) {
 #pragma unroll
