@@ -56,6 +56,7 @@ MEASURED_TRAFFIC_KIB = {
     # profiles/contract_bandwidth_bound_shapes.md
     ("skinny_f16_scale_8192x16x8192", "TraitsF16_64x64x64_xfalse8_yfalse8_kafftrue"): (66629.0 + 1060.0, 2048.0 + 256.0),
     ("longk_f16_scale_256x256x65536", "TraitsF16_64x64x64_xfalse8_yfalse8_kafftrue"): (98695.0 + 4123.5, 8192.0 + 128.0),
+    ("longk_f16_scale_256x256x65536", "TraitsF16_128x128x64_xfalse8_yfalse8_kafftrue_pipe2x4"): (65597.5 + 4123.5, 8192.0 + 128.0),
     ("skinny_f32_scale_8192x16x8192", "WTraitsF32_64x64x16_00"): (133440.0 + 1060.0, 2048.0 + 512.0),
     ("longk_f32_scale_256x256x65536", "WTraitsF32_128x128x16_00"): (132190.0 + 8219.5, 16384.0 + 256.0),
     ("skinny_f32_scale_8192x16x8192", "WTraitsF32_64x64x16_direct8"): (133200.0 + 1060.0, 2048.0 + 512.0),

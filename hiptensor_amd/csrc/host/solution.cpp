@@ -141,7 +141,7 @@ namespace hipta
                 return area >= 65536   ? TileRate{0.44, 0.44}
                        : area >= 49152 ? TileRate{0.40, 0.40}
                        : area >= 32768 ? TileRate{0.38, 0.38}
-                       : area >= 16384 ? TileRate{0.265, 0.315}
+                       : area >= 16384 ? TileRate{0.34, 0.315}
                                        : TileRate{0.107, 0.21};
             case HIPTK_F64:
                 // (the 64 x 64 tile runs on eight waves, 16 x 32 outputs each: alone on a CU it reaches 0.64 of
@@ -263,6 +263,11 @@ namespace hipta
         const double bytes = ((double)v.P * v.K + (double)v.Q * v.K + (double)v.P * v.Q * (v.bilinear ? 2 : 1))
                              * v.elem_bytes;
         us = std::max(us, bytes / (dev.hbm_gbs * 1e3 * 0.6));
+        // split-K slices of different tiles share nothing in time: every workgroup's operand panels come through
+        // the fabric (256 x 256 x 65536 f16 in 32 slices: 16 tiles of 64 x 64 move 2.7e8 B for 6.7e7 algorithmic
+        // and take 40.5 us, 4 tiles of 128 x 128 move half of that and take 33.4)
+        if(split > 1)
+            us = std::max(us, tiles * (double)(s.bp + s.bq) * (double)v.K * v.elem_bytes / (dev.hbm_gbs * 1e3 * 1.4));
         // launch, and prologue + epilogue of every round of workgroups on a CU
         // (a workgroup's epilogue moves its output tile, and C, at about 30 GB/s per CU)
         const double tile_io = (double)s.bp * s.bq * v.elem_bytes * (v.bilinear ? 2.0 : 1.0) / 30e3;
