@@ -17,7 +17,16 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 KDIR = os.path.join(ROOT, "hiptensor_amd", "csrc", "kernels")
 
 
+_ASM = {}
+
+
 def device_asm(unit, tmp_path):
+    if unit not in _ASM:
+        _ASM[unit] = _compile(unit, tmp_path)
+    return _ASM[unit]
+
+
+def _compile(unit, tmp_path):
     out = tmp_path / (unit + ".s")
     subprocess.run(["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
                     "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-option-ignored",
@@ -77,3 +86,21 @@ def test_main_loop_is_mfma_loads_and_scalar_only(tmp_path, unit, symbol, mfmas):
         assert not valu, f"vector ALU instructions in the main loop of {symbol}: {valu}"
         assert not any(o.startswith(("s_cbranch", "s_branch")) for o in ops), "a branch inside the main loop"
         assert not any(o.startswith(("scratch_", "buffer_store", "global_store")) for o in ops), "stores or spills in the main loop"
+
+
+@pytest.mark.parametrize("unit", ["contract_f32", "contract_f64", "contract_c32", "contract_c64"])
+def test_every_32_64_bit_direct_load_instantiation(tmp_path, unit):
+    """... and the same for every instantiation of the 32/64-bit direct-load kernel for K a multiple of the K tile
+    (64 x 64 and 32 x 32 tiles, row- and k-contiguous operands): each has its ring unrolled as one clean loop."""
+    lines = device_asm(unit, tmp_path)
+    symbols = [l.split(":")[0] for l in lines if re.match(r"^_ZN5hiptk18contract_wd_kernel.*ELb0EEEvNS_5KArgsE:", l)]
+    assert len(symbols) >= 2, symbols
+    for symbol in symbols:
+        body = kernel_body(lines, symbol)
+        loops = main_loops(body, 16)
+        assert loops, f"{symbol}: no main loop found"
+        for a, b in loops:
+            ops = opcodes(body, a, b)
+            valu = sorted({o for o in ops if o.startswith("v_") and not o.startswith("v_mfma")})
+            assert not valu, f"vector ALU instructions in the main loop of {symbol}: {valu}"
+            assert not any(o.startswith(("s_cbranch", "s_branch", "scratch_")) for o in ops), symbol
