@@ -45,12 +45,11 @@ MEASURED_TRAFFIC_KIB = {
     ("cfg2_bf16_bilinear_4096", "TraitsBF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (115910.0, 32770.0),
     # profiles/contract_kernels_configs_1_3_4_5_counters.md (split-K: contraction kernel + reduction kernel)
     ("cfg1_f32_bilinear_256", "WTraitsF32_64x64x16_00"): (823.0 + 1187.5, 2048.0 + 256.0),
-    ("cfg1_f32_bilinear_256", "WTraitsF32_64x64x16_direct8"): (830.5 + 675.5, 1024.0 + 256.0),
     ("cfg1_f32_bilinear_256", "WTraitsF32_32x32x16_direct4k4"): (979.0, 256.0),
     ("cfg3_f64_bilinear_1920x1920x768", "WTraitsF64_64x64x16_00"): (74014.4, 28800.0),
-    ("cfg3_f64_bilinear_1920x1920x768", "WTraitsF64_64x64x8_direct8"): (85919.0, 28800.0),
+    ("cfg3_f64_bilinear_1920x1920x768", "WTraitsF64_64x64x8_direct4"): (84483.0, 28800.0),
     ("cfg4_c32_bilinear_1024x1024x512", "WTraitsC32_64x64x8_00"): (12368.0 + 12348.0, 16384.0 + 8192.0),
-    ("cfg4_c32_bilinear_1024x1024x512", "WTraitsC32_64x64x8_direct8"): (16483.0, 8192.0),
+    ("cfg4_c32_bilinear_1024x1024x512", "WTraitsC32_64x64x8_direct4"): (16476.0, 8192.0),
     ("cfg5_f16_bilinear_rank6_permuted", "TraitsF16_256x192x64_xfalse8_ytrue8_kafffalse_pipe4x2"): (325638.6, 102232.8),
     ("cfg5_f16_bilinear_rank6_permuted", "TraitsF16_256x192x32_xfalse8_ytrue8_kafffalse_direct2x2"): (327800.0, 102000.0),
     # profiles/contract_bandwidth_bound_shapes.md
@@ -59,9 +58,8 @@ MEASURED_TRAFFIC_KIB = {
     ("longk_f16_scale_256x256x65536", "TraitsF16_128x128x64_xfalse8_yfalse8_kafftrue_pipe2x4"): (65597.5 + 4123.5, 8192.0 + 128.0),
     ("skinny_f32_scale_8192x16x8192", "WTraitsF32_64x64x16_00"): (133440.0 + 1060.0, 2048.0 + 512.0),
     ("longk_f32_scale_256x256x65536", "WTraitsF32_128x128x16_00"): (132190.0 + 8219.5, 16384.0 + 256.0),
-    ("skinny_f32_scale_8192x16x8192", "WTraitsF32_64x64x16_direct8"): (133200.0 + 1060.0, 2048.0 + 512.0),
     ("skinny_f32_scale_8192x16x8192", "WTraitsF32_32x32x16_direct4k4"): (133220.0, 512.0),
-    ("longk_f32_scale_256x256x65536", "WTraitsF32_64x64x16_direct8"): (196670.0 + 4123.5, 8192.0 + 256.0),
+    ("longk_f32_scale_256x256x65536", "WTraitsF32_64x64x16_direct4"): (196670.0 + 4123.5, 8192.0 + 256.0),
     # profiles/permute_kernels_1GiB_tensors.md
     ("perm_f32_512x64x128x64_2031", "permute_tiled_f32_128x128_r4_w4"): (524329.9, 1049097.7),
 }

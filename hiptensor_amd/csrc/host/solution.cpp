@@ -208,8 +208,8 @@ namespace hipta
         }
         if(s.direct && class_flops_per_clk_cu(v.cls) != 4096.0)
         {
-            // The 32/64-bit 64 x 64 tiles whose operand tiles are loaded straight into LDS (four waves, two
-            // workgroups per CU): slopes of 1024 x 1024 x K (one workgroup per CU) and 2048 x 2048 x K scans
+            // The 32/64-bit 64 x 64 tiles whose operand tiles are loaded straight into LDS (four waves, three to
+            // four workgroups per CU): slopes of 1024 x 1024 x K (one workgroup per CU) and 2048 x 2048 x K scans
             const bool big = s.bp * s.bq >= 4096; // 64 x 64, or 32 x 32 with the waves splitting K
             const bool kf  = v.x_kfast && v.y_kfast; // 16-byte vectors of k: shorter runs in memory
             switch(v.cls)

@@ -113,10 +113,10 @@ def layouts(dtype, compute, big):
             out.append(wl.config5(extents=(32, 2, 8, 24, 2, 16, 4, 8, 10)))
     if not big and compute == cases.COMPUTE[dtype]:
         # The 32/64-bit kernels that load their operand tiles straight into LDS (operands in 16-byte vectors,
-        # one K stride, K tiles of 8 or 16; a ring of 4 or 8 tiles):
-        # a single K tile, fewer tiles than the ring holds, exactly one ring, several rings with a
-        # remainder; partial and whole 64 x 64 output tiles (complex f64 has no such kernel)
-        for kk in ((8, 1), (16, 1), (16, 3), (16, 8), (16, 13), (16, 17)):
+        # one K stride, K tiles of 8 or 16; a ring of 4 tiles):
+        # a single K tile, fewer tiles than the ring holds, exactly one ring (K = 32 or 64), several rings with a
+        # remainder; partial and whole 64 x 64 output tiles
+        for kk in ((8, 1), (16, 1), (16, 2), (16, 3), (16, 4), (16, 8), (16, 13), (16, 17)):
             dk = {0: 40, 1: 5, 10: 24, 11: 7, 20: kk[0], 21: kk[1]}
             tag = f"k{kk[0] * kk[1]}"
             out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], dk, a, b,
