@@ -49,7 +49,7 @@ MEASURED_TRAFFIC_KIB = {
     ("cfg3_f64_bilinear_1920x1920x768", "WTraitsF64_64x64x16_00"): (74014.4, 28800.0),
     ("cfg3_f64_bilinear_1920x1920x768", "WTraitsF64_64x64x8_direct4"): (84483.0, 28800.0),
     ("cfg4_c32_bilinear_1024x1024x512", "WTraitsC32_64x64x8_00"): (12368.0 + 12348.0, 16384.0 + 8192.0),
-    ("cfg4_c32_bilinear_1024x1024x512", "WTraitsC32_64x64x8_direct4"): (16476.0, 8192.0),
+    ("cfg4_c32_bilinear_1024x1024x512", "WTraitsC32_64x64x8_direct8"): (16483.0, 8192.0),
     ("cfg5_f16_bilinear_rank6_permuted", "TraitsF16_256x192x64_xfalse8_ytrue8_kafffalse_pipe4x2"): (325638.6, 102232.8),
     ("cfg5_f16_bilinear_rank6_permuted", "TraitsF16_256x192x32_xfalse8_ytrue8_kafffalse_direct2x2"): (327800.0, 102000.0),
     # profiles/contract_bandwidth_bound_shapes.md

@@ -68,7 +68,7 @@ CASES = [
     # configuration 3: f64, 64 x 64 tile, K tiles of 8, ring of 4, row-contiguous operands, K a multiple of the K tile
     ("contract_f64", "_ZN5hiptk18contract_wd_kernelINS_10WTraitsF64ELi8ELi4ELb0ELb0ELb0ELb0EEEvNS_5KArgsE", 4 * 8),
     # configuration 4: complex f32, the same geometry (four k-steps a tile, four MFMAs per complex product)
-    ("contract_c32", "_ZN5hiptk18contract_wd_kernelINS_10WTraitsC32ELi8ELi4ELb0ELb0ELb0ELb0EEEvNS_5KArgsE", 4 * 4 * 4),
+    ("contract_c32", "_ZN5hiptk18contract_wd_kernelINS_10WTraitsC32ELi8ELi8ELb0ELb0ELb0ELb0EEEvNS_5KArgsE", 8 * 4 * 4),
     # configuration 2: f16, 256 x 256 tile, both operands row-contiguous, one K stride
     ("contract_f16_hd", "_ZN5hiptk18contract_hd_kernelINS_9TraitsF16ELb0ELb0ELi256ELb1EEEvNS_5KArgsE", 128),
 ]
