@@ -14,7 +14,9 @@ for its kernel (average launch duration measured with HIP events on the launch s
 `cpu_baseline` object (the reference's own CPU contraction, or the oracle port, timed on a
 bounded slab of the same workload on this host), a `target` object (the same problem as a
 bilinear contraction in f16 and in bf16: kernel time, TFLOP/s, fraction of the nominal peak and
-of the MFMA-only sustained rate), a short `permutation` object (GB/s of one
+of the MFMA-only sustained rate; the same in packed row-major layout), an `others` object (the other
+configurations, per element type: kernel time, TFLOP/s, fraction of the type's peak), a `parity` object per
+timed workload (its D buffer against the oracle; the run exits non-zero beyond the tolerance), a short `permutation` object (GB/s of one
 hiptensorPermutation workload; --permutation gives that operation its own full line) and, with
 --all, the other configurations.
 """
@@ -87,8 +89,38 @@ def mfma_ceiling(dtype, random_operands):
     return tf.value if _CALIB.hiptk_mfma_ceiling(kcls[dtype], 1 if random_operands else 0, ctypes.byref(tf)) == 0 else None
 
 
-def measure(handle, w, steps, warmup, settle_s=0.25):
-    """Returns dict(ms_per_step wall, kernel_ms from HIP events, info)."""
+def measured_parity(w, inp, D_host, rows=8, samples=4096):
+    """The D buffer the timed steps wrote, against the CPU oracle (the checker; outside every timed region) on
+    `rows` whole rows of the flattened output and a prime-strided sample of all of it: the two metrics of
+    tests/cases.py (relative error against the contract's tolerance for the type, the reference harness's
+    element-wise metric against its own bound)."""
+    import numpy as np
+
+    import cases
+    import oracle
+    from hiptensor_amd import workloads as wl
+
+    M, N, K = wl.dims(w)
+    total = M * N
+    step = max(2, total // samples)
+    while any(step % d == 0 for d in range(2, int(step ** 0.5) + 1)):
+        step += 1
+    b0 = (total // 2 // N) * N
+    exp = wl.nan_buffer(w["dtype"], inp["spanD"])
+    oracle.contract(w, inp["A"], inp["B"], inp["C"], D=exp, begin=b0, end=min(total, b0 + rows * N))
+    oracle.contract(w, inp["A"], inp["B"], inp["C"], D=exp, begin=0, end=-1, step=step)
+    el, gl = cases.logical_view(w, exp), cases.logical_view(w, D_host)
+    f = wl.to_float(w["dtype"], el)
+    sel = ~np.isnan(f.real if np.iscomplexobj(f) else f)
+    rel = cases.relative_error(w["dtype"], gl[sel], el[sel])
+    elt = cases.error_metric(w["dtype"], gl[sel], el[sel])
+    return {"measured_rel": rel, "tolerance": cases.contract_tolerance(w), "measured_elt": elt,
+            "elt_bound": cases.harness_tolerance(w), "outputs_checked": int(sel.sum()),
+            "ok": bool(rel <= cases.contract_tolerance(w) and elt <= cases.harness_tolerance(w))}
+
+
+def measure(handle, w, steps, warmup, settle_s=0.25, check=True):
+    """Returns dict(ms_per_step wall, kernel_ms from HIP events, info, parity of the timed D buffer)."""
     import torch
 
     from hiptensor_amd import workloads as wl
@@ -100,6 +132,7 @@ def measure(handle, w, steps, warmup, settle_s=0.25):
     A, B = gpu_util.to_device(inp["A"]), gpu_util.to_device(inp["B"])
     Cd = gpu_util.to_device(inp["C"]) if inp["C"] is not None else None
     D = torch.empty(inp["spanD"] * wl.ELEM_BYTES[w["dtype"]], dtype=torch.uint8, device="cuda")
+    D.fill_(0xFF)  # (NaN in every floating type here: an element the timed steps do not write fails the check below)
     c = wl.Contraction(handle, w)
     ws = torch.empty(max(int(c.workspace_bytes), 16), dtype=torch.uint8, device="cuda")
     stream = torch.cuda.current_stream()
@@ -125,6 +158,11 @@ def measure(handle, w, steps, warmup, settle_s=0.25):
     t1 = time.perf_counter()
     assert st == 0
     out = {"ms_per_step": (t1 - t0) * 1e3 / steps, "kernel_ms": e0.elapsed_time(e1) / steps, "info": dict(c.info)}
+    if check:
+        import numpy as np
+
+        D_host = D.cpu().numpy().view(wl.NP_STORE[w["dtype"]])
+        out["parity"] = measured_parity(w, inp, D_host)
     c.close()
     return out
 
@@ -300,6 +338,7 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time every other configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-target", action="store_true", help="skip the bilinear f16 / bf16 rows of the default line")
+    ap.add_argument("--no-others", action="store_true", help="skip the other configurations in the default line")
     ap.add_argument("--permutation", action="store_true",
                     help="time hiptensorPermutation instead (workload: a name of workloads.permutation_configs(), "
                          "default perm_f32_rank4); the JSON line then carries GB/s against the HBM roofline")
@@ -372,39 +411,52 @@ def main():
     out["roofline"]["mfma_only_sustained_tflops"] = ceil
     if ceil.get("random_operands"):
         out["roofline"]["frac_of_sustained"] = tflops / ceil["random_operands"]
-    out["parity"] = {"oracle": "CPU restatement of the reference's contraction, pinned bit-for-bit to the reference's compiled CPU path",
-                     "tolerance": {"f16": 1e-2, "bf16": 1e-2, "f32": 1e-5, "c32": 1e-5, "f64": 1e-12, "c64": 1e-12}[w["dtype"]],
-                     "tolerance_metric": "max|d - r| / max|r| over the checked outputs (tests/cases.py); the reference "
-                                         "harness's element-wise |d - r| / (|d| + |r| + 1) is held to its own bound 2 K eps beside it"}
+    # measured on the D buffer the timed steps wrote (8 whole rows and a prime-strided sample of all of D)
+    out["parity"] = dict(r.get("parity", {}),
+                         oracle="CPU restatement of the reference's contraction, pinned bit-for-bit to the reference's compiled CPU path",
+                         tolerance_metric="measured_rel = max|d - r| / max|r| over the checked outputs of the timed buffer, against "
+                                          "`tolerance`; measured_elt = the reference harness's element-wise |d - r| / (|d| + |r| + 1), "
+                                          "against its own bound 2 K eps (+ 16-bit terms)")
+    failed = [] if out["parity"].get("ok", True) else [w["name"]]
     # The same 4096^3 problem as a bilinear contraction (beta = 1, C read), f16 and bf16: the
     # operation and types the throughput target is stated on.
     if a.workload == "cfg2_f16_scale" and not a.no_target:
         target = {}
-        for tname in ("cfg2_f16_bilinear", "cfg2_bf16_bilinear"):
-            tw = cfgs[tname]
+        rm = wl.row_major_configs()
+        # ... and in the layout NULL strides give (packed row-major: both operands contiguous along k)
+        for tname in ("cfg2_f16_bilinear", "cfg2_bf16_bilinear", "rowmajor_f16_bilinear", "rowmajor_bf16_bilinear"):
+            tw = cfgs[tname] if tname in cfgs else rm[tname]
             tr = measure(handle, tw, a.steps, a.warmup, a.settle)
             ttf = wl.flops(tw) / (tr["kernel_ms"] * 1e-3) / 1e12
             sustained = mfma_ceiling(tw["dtype"], 1)
             target[tname] = {"kernel_ms": tr["kernel_ms"], "tflops": ttf, "frac": ttf / PEAK_TFLOPS[tw["dtype"]],
                              "mfma_only_sustained_tflops": sustained,
                              "frac_of_sustained": ttf / sustained if sustained else None,
-                             "kernel": tr["info"]["kernel_name"], "op": "bilinear", "dtype": tw["dtype"]}
+                             "kernel": tr["info"]["kernel_name"], "op": "bilinear", "dtype": tw["dtype"],
+                             "parity": tr["parity"]}
+            if not tr["parity"]["ok"]:
+                failed.append(tname)
         out["target"] = target
-    if a.all:
+    if a.workload == "cfg2_f16_scale" and not a.no_others or a.all:
+        # the other configurations, per element type (GPU only, fewer steps; --all adds the reference's CPU
+        # contraction beside each)
         others = {}
         for name, cw in cfgs.items():
-            if name == a.workload:
+            if name == a.workload or (not a.all and name in ("cfg2_f16_bilinear", "cfg2_bf16_bilinear")):
                 continue
-            steps = max(5, a.steps // 2)
-            rr = measure(handle, cw, steps, a.warmup, a.settle)
+            steps = max(5, a.steps // 4)
+            rr = measure(handle, cw, steps, max(2, a.warmup // 2), min(a.settle, 0.1))
             tf = wl.flops(cw) / (rr["kernel_ms"] * 1e-3) / 1e12
-            sustained = mfma_ceiling(cw["dtype"], 1)
             others[name] = {"kernel_ms": rr["kernel_ms"], "tflops": tf, "frac_peak": tf / PEAK_TFLOPS[cw["dtype"]],
-                            "mfma_only_sustained_tflops": sustained,
                             "hbm_GBs_algorithmic": wl.algorithmic_bytes(cw) / (rr["kernel_ms"] * 1e-3) / 1e9,
                             "traffic": measured_traffic(cw["name"], rr["info"]["kernel_name"]),
-                            "kernel": rr["info"]["kernel_name"], "split_k": rr["info"]["split_k"], "dtype": cw["dtype"]}
-        if not a.no_cpu:
+                            "kernel": rr["info"]["kernel_name"], "split_k": rr["info"]["split_k"], "dtype": cw["dtype"],
+                            "parity": rr["parity"]}
+            if not rr["parity"]["ok"]:
+                failed.append(name)
+            if a.all:
+                others[name]["mfma_only_sustained_tflops"] = mfma_ceiling(cw["dtype"], 1)
+        if a.all and not a.no_cpu:
             # the reference's CPU contraction beside the other configurations too: in full where
             # that takes seconds, on a slab for the rank-6 problem
             for name in ("cfg1", "cfg3", "cfg4", "cfg5"):
@@ -466,6 +518,9 @@ def main():
         out["cpu_baseline"] = cpu_baseline(w)
     api.hiptensorDestroy(handle)
     print(json.dumps(out))
+    if failed:
+        print("bench.py: the timed results of %s differ from the oracle beyond the tolerance" % ", ".join(failed), file=sys.stderr)
+        sys.exit(1)
 
 
 if __name__ == "__main__":

@@ -90,6 +90,7 @@ _SIGS = {
     "hiptensorAmdPlanInfo": (C.c_int, [vp, C.POINTER(PlanInfo)]),
     "hiptensorAmdPlanTable": (C.c_int64, [vp, C.c_int, i32p, C.c_int64]),
     "hiptensorAmdPlanCacheInfo": (C.c_int, [vp, i64p, i64p]),
+    "hiptensorAmdPlanRetain": (C.c_int, [vp]),
     "hiptk_tile_count": (C.c_int, [C.c_int]),
     "hiptk_tile_info": (C.c_int, [C.c_int, C.c_int, vp]),
     "hiptk_fill_pattern": (C.c_int, [vp, C.c_uint64, C.c_int, vp]),

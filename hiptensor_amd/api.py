@@ -252,6 +252,11 @@ def planInfo(plan):
     return out
 
 
+def planRetain(plan):
+    """Keeps the plan's state until hiptensorDestroy (the cache never retires it); status code."""
+    return lib.hiptensorAmdPlanRetain(plan)
+
+
 def planCacheInfo(handle):
     """(plan states, planning requests) the handle's cache holds."""
     a, b = C.c_int64(0), C.c_int64(0)

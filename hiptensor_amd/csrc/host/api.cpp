@@ -835,6 +835,7 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         p.y_max_off = (int32_t)v.y_max_off;
         p.xk_stride            = (int32_t)v.xk_stride;
         p.yk_stride            = (int32_t)v.yk_stride;
+        (void)hiptk_resolve(&p); // the registry is searched here, once, not at every launch
         fresh->kernel_name     = hiptk_kernel_name(&p);
         if(!h->hostOnly())
             if(auto e = uploadTables(*fresh); e != HIPTENSOR_STATUS_SUCCESS)
@@ -990,12 +991,22 @@ hiptensorStatus_t contractionImpl(const char*                       fn,
     {
         // (retired states stay allocated for the life of the process, so this read is safe)
         log.errorf(fn,
-                   "This plan is no longer valid: its handle was destroyed, or the handle's plan cache retired it; "
-                   "create the plan again (%s)",
+                   "This plan is no longer valid: its handle was destroyed, or the handle's plan cache retired it "
+                   "before it was ever executed; create the plan again (%s)",
                    hiptensorGetErrorString(HIPTENSOR_STATUS_INTERNAL_ERROR));
         return HIPTENSOR_STATUS_INTERNAL_ERROR;
     }
     const PlanState* st = hipta::planState(plan);
+    // from its first execution on a state is never retired by the cache (the device may hold its
+    // table addresses beyond this call); a state the cache retired a moment ago is refused here
+    if(st && !Handle::pin(st))
+    {
+        log.errorf(fn,
+                   "This plan is no longer valid: the handle's plan cache retired it before it was ever executed; "
+                   "create the plan again (%s)",
+                   hiptensorGetErrorString(HIPTENSOR_STATUS_INTERNAL_ERROR));
+        return HIPTENSOR_STATUS_INTERNAL_ERROR;
+    }
     if(st)
         st->last_use.store(hipta::next_use_tick(), std::memory_order_relaxed);
     if(!st || st->device != h->device() || !st->dev_block)
@@ -1123,7 +1134,9 @@ hiptensorStatus_t contractionImpl(const char*                       fn,
                      sizeof(msg),
                      "KernelId: %lu KernelName: %s, %0.3f ms, %0.3f TFlops, %0.3f GB/s%s",
                      (unsigned long)st->sol->uid,
-                     st->kernel_name.c_str(),
+                     // (the kernel that ran: the plan's, or its register-staged stand-in for operands
+                     // that are not 16-byte aligned)
+                     hiptk_kernel_name_at(&st->prob, X, Y),
                      ms,
                      flops / 1e9 / ms,
                      bytes / 1e6 / ms,

@@ -350,6 +350,16 @@ extern "C" int hiptensorAmdPlanInfo(const void* plan, hiptensorAmdPlanInfo_t* ou
     return 0;
 }
 
+extern "C" int hiptensorAmdPlanRetain(const void* plan)
+{
+    if(!plan)
+        return (int)HIPTENSOR_STATUS_NOT_INITIALIZED;
+    const hipta::PlanState* st = (const hipta::PlanState*)((const hiptensorContractionPlan_t*)plan)->mSolution;
+    if(!st)
+        return (int)HIPTENSOR_STATUS_NOT_INITIALIZED;
+    return hipta::Handle::pin(st) ? 0 : (int)HIPTENSOR_STATUS_INTERNAL_ERROR;
+}
+
 extern "C" int hiptensorAmdPlanCacheInfo(const void* handle, int64_t* states, int64_t* requests)
 {
     if(!handle)

@@ -133,23 +133,54 @@ namespace hipta
             }
             if(mPlans.size() >= mMaxPlans)
             {
-                // retire the least recently planned-or-executed state
-                auto lru = mPlans.begin();
+                // retire the least recently planned state among those that were never executed (an
+                // executed state's tables may still be read by the device: a captured graph, a launch
+                // in another thread); if every state has been executed the cache grows instead
+                auto lru = mPlans.end();
                 for(auto jt = mPlans.begin(); jt != mPlans.end(); ++jt)
-                    if(jt->second->last_use.load(std::memory_order_relaxed) < lru->second->last_use.load(std::memory_order_relaxed))
+                {
+                    if(jt->second->launched.load(std::memory_order_acquire))
+                        continue;
+                    if(lru == mPlans.end()
+                       || jt->second->last_use.load(std::memory_order_relaxed) < lru->second->last_use.load(std::memory_order_relaxed))
                         lru = jt;
-                for(auto at = mAlias.begin(); at != mAlias.end();)
-                    at = at->second == lru->second.get() ? mAlias.erase(at) : std::next(at);
-                victim = std::move(lru->second);
-                mPlans.erase(lru);
+                }
+                if(lru != mPlans.end())
+                {
+                    for(auto at = mAlias.begin(); at != mAlias.end();)
+                        at = at->second == lru->second.get() ? mAlias.erase(at) : std::next(at);
+                    victim        = std::move(lru->second);
+                    victim->magic = PlanState::RETIRED; // under the lock: pin() refuses it from here on
+                    mPlans.erase(lru);
+                }
             }
-            raw = fresh.get();
+            raw        = fresh.get();
+            raw->owner = this;
             raw->last_use.store(next_use_tick(), std::memory_order_relaxed);
             mPlans.emplace(decision, std::move(fresh));
             alias(request, raw);
         }
         retire(std::move(victim));
         return raw;
+    }
+
+    bool Handle::pin(const PlanState* st)
+    {
+        // (retired states stay allocated for the life of the process, so these reads are safe)
+        if(!st || st->magic != PlanState::MAGIC)
+            return false;
+        if(st->launched.load(std::memory_order_acquire))
+            return true;
+        Handle* o = st->owner;
+        if(!o)
+            return false;
+        // the cache retires states under this lock: either it has retired this one already, or it
+        // sees the mark and leaves it alone
+        std::lock_guard<std::mutex> g(o->mLock);
+        if(st->magic != PlanState::MAGIC)
+            return false;
+        st->launched.store(true, std::memory_order_release);
+        return true;
     }
 
     size_t Handle::planCount()

@@ -39,6 +39,13 @@ namespace hipta
         // last planning or execution that touched this state (a process-wide tick): the handle's
         // cache retires the least recently used state when it is full
         mutable std::atomic<uint64_t> last_use{0};
+        // Set, under the owning handle's lock, by the first execution of a plan made from this state.
+        // From then on the device may hold the table addresses beyond the call (a captured graph
+        // replays them, another thread may be between its checks and its launch), so the cache never
+        // retires such a state: it lives until hiptensorDestroy.  Only states that were planned and
+        // never executed are candidates for retirement.
+        mutable std::atomic<bool> launched{false};
+        class Handle*             owner = nullptr;
         static constexpr uint64_t MAGIC   = 0x504c414e68697074ull;
         // a state whose device tables were released: its handle was destroyed, or the handle's cache
         // retired it.  The (small) object itself stays allocated until the process ends, so a plan
@@ -74,9 +81,15 @@ namespace hipta
         // Adopts `fresh` under `decision` (or returns the state another thread adopted first, freeing
         // fresh's device block) and remembers `request` as an alias of it.
         PlanState* intern(const std::string& request, const std::string& decision, std::unique_ptr<PlanState> fresh);
+        // To be called by every execution before it uses `st`: false if the state was retired (its
+        // handle destroyed, or the cache dropped it before any execution); otherwise the state is
+        // marked as launched and stays valid until its handle is destroyed.
+        static bool pin(const PlanState* st);
         size_t     planCount();
         size_t     aliasCount();
-        // most states / aliases a handle keeps (HIPTENSOR_AMD_PLAN_CACHE=<states> overrides the first)
+        // most states / aliases a handle keeps (HIPTENSOR_AMD_PLAN_CACHE=<states> overrides the first);
+        // states that have been executed do not count as removable, so a handle that executes more
+        // distinct plans than this keeps them all
         static constexpr size_t MAX_PLANS   = 4096;
         static constexpr size_t MAX_ALIASES = 16384;
 

@@ -179,7 +179,19 @@ namespace hipta
         double round_extra_us = 0.0;
         if(v.cls == HIPTK_F64 && s.bp * s.bq >= 16384 && !(v.x_kfast && v.y_kfast))
             r = TileRate{0.74, 0.74};
-        if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152 && s.bk == 32)
+        if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.direct && s.bk == 64)
+        {
+            // The 256 x 256 tile on 16 x 16 x 32 MFMAs whose operand tiles are loaded straight into LDS in K tiles of
+            // 64 (four waves).  4096^3 f16 scale, one device: both operands k-contiguous 98.5 us (main loop 84.2,
+            // prologue 1.5, epilogue 7.9) against 108.8 on the same loop with 32 x 32 x 16 MFMAs and 121.0 on the
+            // eight-wave staged tile; both row-contiguous 105.5 against 114.7 on the 32 x 32 x 16 direct-load tile of
+            // K tiles of 32 (bf16 bilinear 99.2 against 107.0).
+            const double f = (v.x_kfast && v.y_kfast) ? 1.33 : (v.x_kfast || v.y_kfast) ? 1.28 : 1.235;
+            r.alone *= f;
+            r.full *= f;
+            round_extra_us = 6.5;
+        }
+        else if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152 && s.bk == 32)
         {
             // The 256 x 256 and 256 x 192 tiles whose operand tiles are loaded straight into LDS (four waves,
             // K in steps of 32): a faster main loop, but one workgroup has the CU to itself, so nothing

@@ -1,0 +1,16 @@
+// f16 kernels on v_mfma_f32_16x16x32 with operand tiles loaded straight into LDS in K tiles of 64: 256 x 256 tile, X row-contiguous.
+#include "contract_hk.hpp"
+
+namespace hiptk
+{
+    static const KernelEntry k_entries[] = {
+        HIPTK_HK_ENTRY(TraitsF16, 11, 256, false, true, 2, 2, 2),
+        HIPTK_HK_ENTRY(TraitsF16, 11, 256, false, false, 2, 2, 2),
+    };
+
+    const KernelEntry* entries_f16_hk_rx(int* count)
+    {
+        *count = (int)(sizeof(k_entries) / sizeof(k_entries[0]));
+        return k_entries;
+    }
+}

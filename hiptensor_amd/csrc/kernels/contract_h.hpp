@@ -395,6 +395,33 @@ namespace hiptk
         }
     }
 
+    // Where a lane's accumulators of one 32-row slab of its wave tile lie, for the epilogue: as QUADS
+    // groups of 4 consecutive rows at one column, quad q = c * NRQ + g being the g-th of the lane's
+    // NRQ row groups at its c-th of NCOL columns.
+    //   row0(q, lane): first of the quad's rows within the slab;  col(q, lane): its column within the wave tile;
+    //   get(i, q, e):  the accumulator of row row0 + e of slab i.
+    // v_mfma_f32_32x32x16: blocks of 32 x 32, 16 registers per lane (register r: row 8 (r / 4) + 4 (lane / 32) + r % 4,
+    // column lane % 32)
+    template <int TP, int TQ>
+    struct Acc32
+    {
+        f32x16_t (&a)[TP][TQ];
+        static constexpr int NCOL = TQ, NRQ = 4, QUADS = NCOL * NRQ;
+        __device__ static inline int row0(int q, int lane) { return 8 * (q & 3) + 4 * (lane >> 5); }
+        __device__ static inline int col(int q, int lane) { return 32 * (q >> 2) + (lane & 31); }
+        __device__ inline float      get(int i, int q, int e) const { return a[i][q >> 2][4 * (q & 3) + e]; }
+    };
+    // v_mfma_f32_16x16x32: blocks of 16 x 16, 4 registers per lane (register r: row 4 (lane / 16) + r, column lane % 16)
+    template <int TP, int TQ>
+    struct Acc16
+    {
+        f32x4_t (&a)[2 * TP][2 * TQ];
+        static constexpr int NCOL = 2 * TQ, NRQ = 2, QUADS = NCOL * NRQ;
+        __device__ static inline int row0(int q, int lane) { return 16 * (q & 1) + 4 * (lane >> 4); }
+        __device__ static inline int col(int q, int lane) { return 16 * (q >> 1) + (lane & 15); }
+        __device__ inline float      get(int i, int q, int e) const { return a[2 * i + (q & 1)][q >> 1][e]; }
+    };
+
     // Epilogue of the 16-bit kernels: D = alpha * acc (+ beta * C) for the wave tiles of one
     // workgroup tile.  `lds` is the workgroup's whole LDS allocation of LDSCAP bytes, free by
     // now (every wave has passed the main loop's last barrier); p0 / q0 are the first row / column
@@ -402,9 +429,10 @@ namespace hiptk
     // back to end at P / Q).
     // DEEP: two slabs of C in flight also for the 128-wide wave tiles (for kernels whose main loop
     // leaves the registers for it).
-    template <typename Tr, int WP, int WQ, int TP, int TQ, int LDSCAP, bool DEEP = false>
-    __device__ __forceinline__ void epilogue_h(const KArgs& a, f32x16_t (&acc)[TP][TQ], uint16_t* lds, int p0, int q0, int p_own, int q_own)
+    template <typename Tr, int WP, int WQ, int TP, int TQ, int LDSCAP, bool DEEP, typename Acc>
+    __device__ __forceinline__ void epilogue_acc(const KArgs& a, const Acc acc, uint16_t* lds, int p0, int q0, int p_own, int q_own)
     {
+        constexpr int QUADS = Acc::QUADS;
         constexpr int WTP = TP * 32, WTQ = TQ * 32;
         const int     tid  = threadIdx.x;
         const int     lane = tid & 63;
@@ -420,23 +448,21 @@ namespace hiptk
         const float beta  = (float)a.beta[0];
         if(a.split_k > 1)
         {
-            const int pw = p0 + wp * WTP + 4 * (lane >> 5);
-            const int qw = q0 + wq * WTQ + (lane & 31);
-            float*    ws = (float*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
+            float* ws = (float*)a.ws + (size_t)blockIdx.z * (size_t)a.P * (size_t)a.Q;
 #pragma unroll
-            for(int j = 0; j < TQ; j++)
+            for(int u = 0; u < QUADS; u++)
             {
-                const int q = qw + j * 32;
+                const int q = q0 + wq * WTQ + Acc::col(u, lane);
                 if(!q_in(q))
                     continue;
 #pragma unroll
                 for(int i = 0; i < TP; i++)
 #pragma unroll
-                    for(int r = 0; r < 16; r++)
+                    for(int e = 0; e < 4; e++)
                     {
-                        const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
+                        const int p = p0 + wp * WTP + i * 32 + Acc::row0(u, lane) + e;
                         if(p_in(p))
-                            ws[(size_t)p * a.Q + q] = acc[i][j][r];
+                            ws[(size_t)p * a.Q + q] = acc.get(i, u, e);
                     }
             }
             return;
@@ -492,15 +518,13 @@ namespace hiptk
             };
             auto write_slab = [&](int i, uint16_t* dst) {
 #pragma unroll
-                for(int j = 0; j < TQ; j++)
-#pragma unroll
-                    for(int g = 0; g < 4; g++)
-                    {
-                        u32x2_t w;
-                        w[0] = (uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g]) | ((uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 1]) << 16);
-                        w[1] = (uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 2]) | ((uint32_t)Tr::from_f32(alpha * acc[i][j][4 * g + 3]) << 16);
-                        *(u32x2_t*)(dst + (j * 32 + (lane & 31)) * PH + 8 * g + 4 * (lane >> 5)) = w;
-                    }
+                for(int u = 0; u < QUADS; u++)
+                {
+                    u32x2_t w;
+                    w[0] = (uint32_t)Tr::from_f32(alpha * acc.get(i, u, 0)) | ((uint32_t)Tr::from_f32(alpha * acc.get(i, u, 1)) << 16);
+                    w[1] = (uint32_t)Tr::from_f32(alpha * acc.get(i, u, 2)) | ((uint32_t)Tr::from_f32(alpha * acc.get(i, u, 3)) << 16);
+                    *(u32x2_t*)(dst + Acc::col(u, lane) * PH + Acc::row0(u, lane)) = w;
+                }
             };
             offsets(0, doff[0]);
             write_slab(0, st0);
@@ -633,10 +657,10 @@ namespace hiptk
             float* const   st0 = (float*)lds + wave * ((DB ? 2 : 1) * 32 * EP);
             auto write_slab = [&](int i, float* dst) {
 #pragma unroll
-                for(int j = 0; j < TQ; j++)
+                for(int u = 0; u < QUADS; u++)
 #pragma unroll
-                    for(int r = 0; r < 16; r++)
-                        dst[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
+                    for(int e = 0; e < 4; e++)
+                        dst[(Acc::row0(u, lane) + e) * EP + Acc::col(u, lane)] = acc.get(i, u, e);
             };
             prefetch(0, sl[0]);
             if constexpr(DB)
@@ -777,10 +801,10 @@ namespace hiptk
             float* const   st0 = (float*)lds + wave * ((DB ? 2 : 1) * 32 * EP);
             auto write_slab = [&](int i, float* dst) {
 #pragma unroll
-                for(int j = 0; j < TQ; j++)
+                for(int u = 0; u < QUADS; u++)
 #pragma unroll
-                    for(int r = 0; r < 16; r++)
-                        dst[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * EP + j * 32 + (lane & 31)] = acc[i][j][r];
+                    for(int e = 0; e < 4; e++)
+                        dst[(Acc::row0(u, lane) + e) * EP + Acc::col(u, lane)] = acc.get(i, u, e);
             };
             // (all look-ups of the first two slabs before their first C load: one wait, not two)
             prepare(0, off[0]);
@@ -889,15 +913,16 @@ namespace hiptk
             // compiler knows, the tables), so it would fetch one offset, one C element and store
             // one D element at a time; the offsets of a slab's 16 rows are therefore fetched once,
             // ahead of the columns, and the 16 C elements of a column before the first store.
-            const int pw = p0 + wp * WTP + 4 * (lane >> 5);
-            const int qw = q0 + wq * WTQ + (lane & 31);
-            const bool bil = a.bilinear != 0;
-            uint32_t   dqo[TQ], cqo[TQ];
-            bool       qok[TQ];
+            constexpr int NCOL = Acc::NCOL, NRQ = Acc::NRQ, NROW = 4 * NRQ; // a lane's columns, and its rows per slab
+            const int     pw = p0 + wp * WTP;
+            const int     qw = q0 + wq * WTQ;
+            const bool    bil = a.bilinear != 0;
+            uint32_t      dqo[NCOL], cqo[NCOL];
+            bool          qok[NCOL];
 #pragma unroll
-            for(int j = 0; j < TQ; j++)
+            for(int j = 0; j < NCOL; j++)
             {
-                const int q = qw + j * 32;
+                const int q = qw + Acc::col(j * NRQ, lane);
                 qok[j]      = q_in(q);
                 // (the tables are padded beyond every index a tile can reach, with the offset of
                 // index 0: loads need no guard, only the stores do)
@@ -907,38 +932,51 @@ namespace hiptk
 #pragma unroll
             for(int i = 0; i < TP; i++)
             {
-                uint32_t dpo[16], cpo[16];
-                bool     pok[16];
+                uint32_t dpo[NROW], cpo[NROW];
+                bool     pok[NROW];
 #pragma unroll
-                for(int r = 0; r < 16; r++)
+                for(int r = 0; r < NROW; r++)
                 {
-                    const int p = pw + i * 32 + 8 * (r >> 2) + (r & 3);
+                    const int p = pw + i * 32 + Acc::row0(r >> 2, lane) + (r & 3);
                     pok[r]      = p_in(p);
                     dpo[r]      = (uint32_t)a.dp[p];
                     cpo[r]      = bil ? (uint32_t)a.cp[p] : 0u;
                 }
 #pragma unroll
-                for(int j = 0; j < TQ; j++)
+                for(int j = 0; j < NCOL; j++)
                 {
                     if(!qok[j])
                         continue;
-                    float c[16];
+                    float c[NROW];
 #pragma unroll
-                    for(int r = 0; r < 16; r++)
+                    for(int r = 0; r < NROW; r++)
                         c[r] = 0.f;
                     if(bil)
                     {
 #pragma unroll
-                        for(int r = 0; r < 16; r++)
+                        for(int r = 0; r < NROW; r++)
                             c[r] = Tr::out_to_f32(Cp[cpo[r] + cqo[j]]);
                     }
 #pragma unroll
-                    for(int r = 0; r < 16; r++)
+                    for(int r = 0; r < NROW; r++)
                         if(pok[r])
-                            Dp[dpo[r] + dqo[j]] = Tr::out_from_f32(Tr::axpby(alpha, acc[i][j][r], beta, c[r], bil));
+                            Dp[dpo[r] + dqo[j]] = Tr::out_from_f32(Tr::axpby(alpha, acc.get(i, j * NRQ + (r >> 2), r & 3), beta, c[r], bil));
                 }
             }
         }
+    }
+
+    // ... for accumulators of v_mfma_f32_32x32x16 blocks
+    template <typename Tr, int WP, int WQ, int TP, int TQ, int LDSCAP, bool DEEP = false>
+    __device__ __forceinline__ void epilogue_h(const KArgs& a, f32x16_t (&acc)[TP][TQ], uint16_t* lds, int p0, int q0, int p_own, int q_own)
+    {
+        epilogue_acc<Tr, WP, WQ, TP, TQ, LDSCAP, DEEP>(a, Acc32<TP, TQ>{acc}, lds, p0, q0, p_own, q_own);
+    }
+    // ... and of v_mfma_f32_16x16x32 blocks (TP x TQ still counts blocks of 32 x 32)
+    template <typename Tr, int WP, int WQ, int TP, int TQ, int LDSCAP, bool DEEP = false>
+    __device__ __forceinline__ void epilogue_h16(const KArgs& a, f32x4_t (&acc)[2 * TP][2 * TQ], uint16_t* lds, int p0, int q0, int p_own, int q_own)
+    {
+        epilogue_acc<Tr, WP, WQ, TP, TQ, LDSCAP, DEEP>(a, Acc16<TP, TQ>{acc}, lds, p0, q0, p_own, q_own);
     }
 
     template <typename Tr,

@@ -43,6 +43,15 @@ namespace hiptk
     {
         asm volatile("s_nop 4\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
     }
+    // The same load without the wait states in front of it, for the inside of a hand-ordered main loop:
+    // an s_nop N holds the wave's issue slot for N + 1 rounds of 4 cycles, longer than a 16-cycle MFMA
+    // runs.  To be used only where (1) another instruction sits between the write of M0 and this load
+    // and (2) no VALU instruction writes a scalar register anywhere near: the loops that use it are
+    // checked for that in their device assembly (tests/test_kernel_codegen.py).
+    __device__ __forceinline__ void dma_load_in_loop(uint32_t voff, const void* base)
+    {
+        asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
+    }
     // ... with a full address per lane (no scalar base): for loads some lanes of which must look elsewhere
     __device__ __forceinline__ void dma_load_at(const void* lane_address)
     {

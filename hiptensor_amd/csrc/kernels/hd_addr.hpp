@@ -114,6 +114,84 @@ namespace hiptk
         return c;
     }
 
+    // ---- 16-bit kernel for operands that are both contiguous along k (contract_hk.hpp): K tiles of 64 ----
+    // A stage is stage[row][64 k]: 128-byte rows, so that a direct load fetches whole 128-byte lines
+    // (8 rows per KiB).  The 16-byte slot s holds the 8 k from `k` on of row `row`; the XOR puts the
+    // 16 rows that 16 consecutive lanes of a ds_read_b128 touch into 16 disjoint bank ranges.
+    constexpr int HK_BK = 64;
+
+    // position (0 .. 7) in its row's 128 bytes of the 16-byte chunk that holds k = 8 * chunk .. + 7
+    HIPTK_HD_FN int hk_chunk_pos(int row, int chunk)
+    {
+        return chunk ^ ((row >> 1) & 7);
+    }
+
+    template <int BR>
+    HIPTK_HD_FN HdSlot hk_slot(int s)
+    {
+        HdSlot o;
+        o.row = s >> 3;
+        o.k   = 8 * hk_chunk_pos(o.row, s & 7); // (the XOR is its own inverse)
+        return o;
+    }
+
+    // ... and for either kind of operand: a k-contiguous one as above, a row-contiguous one as
+    // stage[k][BR] (64 k-rows), whose slot s holds the 8 rows from `row` on at `k`
+    template <bool KF, int BR>
+    HIPTK_HD_FN HdSlot hk_stage_slot(int s)
+    {
+        if(KF)
+            return hk_slot<BR>(s);
+        HdSlot        o;
+        constexpr int cpr = BR / 8;
+        o.k               = s / cpr;
+        o.row             = 8 * ((s % cpr) ^ (2 * (o.k & 3)));
+        return o;
+    }
+
+    // The K tiles one workgroup reduces: nt whole tiles of 64, then, when the slice ends at K and K is
+    // not a multiple of 64, a tail tile of `tail` k-steps of 16: it is loaded whole from K - 64 (so
+    // that no address leaves the tensor) and only its last `tail` k-steps are multiplied.  Tiles
+    // requested beyond the last one repeat it.
+    struct HkSlice
+    {
+        int nt, tail, n_load, kmax, k00, klast;
+    };
+
+    HIPTK_HD_FN HkSlice hk_slice(int K, int kt_begin, int ktiles_per_split)
+    {
+        HkSlice   s;
+        const int kt_whole = K / HK_BK;
+        const int kt_stop  = kt_begin + ktiles_per_split;
+        s.nt               = (kt_stop < kt_whole ? kt_stop : kt_whole) - kt_begin;
+        s.tail             = ((K % HK_BK) != 0 && kt_stop > kt_whole) ? (K % HK_BK) / 16 : 0;
+        s.n_load           = s.nt + (s.tail ? 1 : 0);
+        s.kmax             = K - HK_BK;
+        s.k00              = kt_begin * HK_BK < s.kmax ? kt_begin * HK_BK : s.kmax;
+        s.klast            = s.tail ? s.kmax : (kt_begin + s.nt - 1) * HK_BK;
+        return s;
+    }
+
+    HIPTK_HD_FN int hk_next_origin(int ko, int klast)
+    {
+        return ko + HK_BK < klast ? ko + HK_BK : klast;
+    }
+
+    // The MFMA slot (0 .. 63, counted from the k-step in which a ring stage has become free) in front of
+    // which wave `wave` issues its j-th direct load of the K tile that goes into that stage: one load
+    // every `spacing` MFMAs, the waves staggered so that the texture path sees them one at a time.
+    HIPTK_HD_FN constexpr int hk_load_slot(int wave, int j, int spacing)
+    {
+        return j * spacing + wave % spacing;
+    }
+
+    // position in its k-row of stage[k][rows] (row-contiguous operand) of the element of row `row`: the
+    // 8-row chunks of a k-row are exchanged by c -> c ^ 2 (k % 4)
+    HIPTK_HD_FN int hd_row_pos(int row, int k)
+    {
+        return (((row >> 3) ^ (2 * (k & 3))) << 3) | (row & 7);
+    }
+
     template <bool KF, int BR>
     HIPTK_HD_FN HdSlot hd_slot(int s)
     {

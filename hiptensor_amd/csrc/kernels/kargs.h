@@ -61,6 +61,10 @@ namespace hiptk
     const KernelEntry* entries_bf16_hd(int* count);
     const KernelEntry* entries_bf16_hd192(int* count);
     const KernelEntry* entries_bf16_hd192_tab(int* count);
+    const KernelEntry* entries_f16_hk_kx(int* count);
+    const KernelEntry* entries_f16_hk_rx(int* count);
+    const KernelEntry* entries_bf16_hk_kx(int* count);
+    const KernelEntry* entries_bf16_hk_rx(int* count);
     const KernelEntry* entries_f16_v4(int* count);
     const KernelEntry* entries_f16_v2(int* count);
     const KernelEntry* entries_bf16_v4(int* count);

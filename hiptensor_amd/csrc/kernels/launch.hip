@@ -24,6 +24,10 @@ namespace hiptk
                                           entries_bf16_hd,
                                           entries_bf16_hd192,
                                           entries_bf16_hd192_tab,
+                                          entries_f16_hk_kx,
+                                          entries_f16_hk_rx,
+                                          entries_bf16_hk_kx,
+                                          entries_bf16_hk_rx,
                                           entries_f16_aff,
                                           entries_bf16_aff,
                                           entries_f16_vec,
@@ -228,7 +232,37 @@ namespace hiptk
             }
             return best;
         }
+
+        // The entry a launch with these operand addresses runs: the resolved one where the plan
+        // resolved it (and the problem still is the one it was resolved for), else a search.
+        const KernelEntry* entry_for(const hiptk_problem_t* p, const void* X, const void* Y)
+        {
+            const KernelEntry* e = (const KernelEntry*)p->kernel;
+            const bool         resolved = e && e->cls == p->cls && e->tile_id == p->tile_id && e->x_kfast == (p->x_kfast != 0)
+                                  && e->y_kfast == (p->y_kfast != 0) && e->x_vec == p->x_vec && e->y_vec == p->y_vec;
+            if(!resolved)
+                e = find_entry(p);
+            if(e && e->k_multiple > 0 && ((((uintptr_t)X) | ((uintptr_t)Y)) & 15) != 0)
+                e = resolved ? (const KernelEntry*)p->kernel_unaligned : staged_entry(p);
+            return e;
+        }
     }
+}
+
+extern "C" int hiptk_resolve(hiptk_problem_t* prob)
+{
+    if(!prob)
+        return HIPTK_ERR_ARG;
+    const hiptk::KernelEntry* e = hiptk::find_entry(prob);
+    prob->kernel                = e;
+    prob->kernel_unaligned      = (e && e->k_multiple > 0) ? hiptk::staged_entry(prob) : e;
+    return e ? HIPTK_OK : HIPTK_ERR_NO_KERNEL;
+}
+
+extern "C" const char* hiptk_kernel_name_at(const hiptk_problem_t* prob, const void* X, const void* Y)
+{
+    const hiptk::KernelEntry* e = prob ? hiptk::entry_for(prob, X, Y) : nullptr;
+    return e ? e->name : "";
 }
 
 extern "C" int hiptk_tile_count(int cls)
@@ -306,9 +340,7 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
     const bool bil = prob->op == HIPTK_OP_BILINEAR;
     if(bil && (!C || !beta || !prob->cp || !prob->cq))
         return HIPTK_ERR_ARG;
-    const KernelEntry* e = find_entry(prob);
-    if(e && e->k_multiple > 0 && ((((uintptr_t)X) | ((uintptr_t)Y)) & 15) != 0)
-        e = staged_entry(prob);
+    const KernelEntry* e = entry_for(prob, X, Y);
     if(!e)
         return HIPTK_ERR_NO_KERNEL;
 
@@ -341,8 +373,12 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
     a.cd_vec    = prob->cd_vec;
     a.shift_p   = prob->shift_p ? 1 : 0;
     a.shift_q   = prob->shift_q ? 1 : 0;
-    a.x_last_vec = prob->x_max_off >= 7 ? 2u * (uint32_t)(prob->x_max_off - 7) : 0u;
-    a.y_last_vec = prob->y_max_off >= 7 ? 2u * (uint32_t)(prob->y_max_off - 7) : 0u;
+    {
+        // byte offset of the last 16-byte vector of X / Y (the class's own element size)
+        const int32_t eb = operand_bytes(prob->cls), back = 16 / eb - 1;
+        a.x_last_vec     = prob->x_max_off >= back ? (uint32_t)eb * (uint32_t)(prob->x_max_off - back) : 0u;
+        a.y_last_vec     = prob->y_max_off >= back ? (uint32_t)eb * (uint32_t)(prob->y_max_off - back) : 0u;
+    }
     // A moved-back tile stores whole 8-element vectors of D that reach into its neighbour's
     // columns (same values).  When D is updated in place (C == D) the neighbour's elements must
     // not be read and written twice, so that case stores element by element.

@@ -306,13 +306,14 @@ def interleaved_configs():
     }
 
 
-def host_inputs(w, nan_gaps=True):
-    """Seeded host buffers {"A", "B", "C" (or None)} plus spans."""
-    A = fill_tensor(w["dtype"], w["lens"]["A"], w["strides"]["A"], SEED_A, nan_gaps)
-    B = fill_tensor(w["dtype"], w["lens"]["B"], w["strides"]["B"], SEED_B, nan_gaps)
+def host_inputs(w, nan_gaps=True, seed_shift=0):
+    """Seeded host buffers {"A", "B", "C" (or None)} plus spans; seed_shift moves all three seeds
+    (other draws of the same distributions)."""
+    A = fill_tensor(w["dtype"], w["lens"]["A"], w["strides"]["A"], SEED_A + seed_shift, nan_gaps)
+    B = fill_tensor(w["dtype"], w["lens"]["B"], w["strides"]["B"], SEED_B + seed_shift, nan_gaps)
     Cb = None
     if w["beta"] is not None:
-        Cb = fill_tensor(w["dtype"], w["lens"]["D"], w["strides"]["C"], SEED_C, nan_gaps)
+        Cb = fill_tensor(w["dtype"], w["lens"]["D"], w["strides"]["C"], SEED_C + seed_shift, nan_gaps)
     return {"A": A, "B": B, "C": Cb, "spanD": span_elems(w["lens"]["D"], w["strides"]["D"])}
 
 

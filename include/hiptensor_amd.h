@@ -179,10 +179,16 @@ typedef struct hiptensorAmdPlanInfo
 } hiptensorAmdPlanInfo_t;
 int hiptensorAmdPlanInfo(const void* plan, hiptensorAmdPlanInfo_t* out);
 /* Size of a handle's plan cache: `states` = plan states it holds (each owns its offset tables on the
- * device; one per distinct planning decision, at most 4096, the least recently used is retired beyond
- * that), `requests` = distinct planning requests (problem x workspace size ...) that map onto them.
+ * device; one per distinct planning decision; beyond 4096 the least recently planned one that was never
+ * executed is retired), `requests` = distinct planning requests (problem x workspace size ...) that map onto them.
  * No counterpart in the reference, whose plans point into process-wide singletons. */
 int hiptensorAmdPlanCacheInfo(const void* handle, int64_t* states, int64_t* requests);
+/* Keeps the plan's state (and its offset tables on the device) until hiptensorDestroy: the cache never
+ * retires it.  The first execution of a plan does the same by itself, since from then on a captured
+ * graph or a launch in another thread may read the tables; this call is for a caller that holds a
+ * plan for later without having executed it.  Returns HIPTENSOR_STATUS_INTERNAL_ERROR for a plan whose
+ * state was retired already.  No counterpart in the reference (its plans never expire). */
+int hiptensorAmdPlanRetain(const void* plan);
 
 /* Copies offset table `which` (0 xp, 1 xk, 2 yq, 3 yk, 4 cp, 5 cq, 6 dp, 7 dq; logical
  * length only, without padding) into out[0..cap); returns the logical length. */

@@ -109,6 +109,12 @@ typedef struct hiptk_problem
                                      themselves moved through LDS clamp every address to it, and the
                                      direct-load kernels are offered only while the byte offset of the
                                      last vector fits 32 bits */
+    /* Filled by hiptk_resolve (zero otherwise): the registry entries this problem runs, looked up once
+     * when the plan is made instead of at every launch.  `kernel` is what hiptk_kernel_name names;
+     * `kernel_unaligned` is what runs in its place when X or Y is not 16-byte aligned at the launch (the
+     * same entry, unless `kernel` loads operand tiles straight into LDS).  Both are tied to the fields
+     * above: a caller that changes any of them afterwards clears these two (or resolves again). */
+    const void *kernel, *kernel_unaligned;
 } hiptk_problem_t;
 
 /* Number of tile configurations of a class, and their description. */
@@ -119,6 +125,14 @@ int hiptk_tile_info(int cls, int tile_id, hiptk_tile_info_t* out);
  * combination; its name ("" if none). */
 int         hiptk_kernel_available(const hiptk_problem_t* prob);
 const char* hiptk_kernel_name(const hiptk_problem_t* prob);
+
+/* Looks the problem's kernels up once and stores them in prob->kernel / prob->kernel_unaligned, so
+ * that hiptk_contract does not search the registry at every launch.  HIPTK_ERR_NO_KERNEL if there is
+ * none.  Optional: hiptk_contract searches when the two fields are null. */
+int hiptk_resolve(hiptk_problem_t* prob);
+/* Name of the kernel a launch with these operand addresses runs: the resolved (or looked-up) kernel,
+ * or its register-staged stand-in when X or Y is not 16-byte aligned. */
+const char* hiptk_kernel_name_at(const hiptk_problem_t* prob, const void* X, const void* Y);
 
 /* Bytes of workspace the problem needs (0 when split_k == 1). */
 uint64_t hiptk_workspace_bytes(const hiptk_problem_t* prob);

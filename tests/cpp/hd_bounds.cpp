@@ -26,6 +26,12 @@ using hiptk::hd_slice;
 using hiptk::hd_slot;
 using hiptk::HdSlice;
 using hiptk::HdSlot;
+using hiptk::hk_chunk_pos;
+using hiptk::hk_next_origin;
+using hiptk::hk_slice;
+using hiptk::hd_row_pos;
+using hiptk::hk_stage_slot;
+using hiptk::HkSlice;
 using hiptk::wd_next_origin;
 using hiptk::wd_slot;
 using hiptk::wd_slot_kf;
@@ -221,6 +227,159 @@ static long check_tile_size(const Case& c, const GemmView& v)
     return walked;
 }
 
+// ---- the 16-bit kernels on 16 x 16 x 32 MFMAs: K tiles of 64, stage[row][64] (k-contiguous operand) or stage[k][rows]
+// (row-contiguous), 8 loads per wave and operand ----
+template <bool KF, int BR>
+static void check_hk_operand(const char* what, const Case& c, const GemmView& v, bool is_x, int r0, const std::vector<int>& origins)
+{
+    const std::vector<int32_t>& rtab    = is_x ? v.xp : v.yq;
+    const std::vector<int32_t>& ktab    = is_x ? v.xk : v.yk;
+    const int64_t               kstride = is_x ? v.xk_stride : v.yk_stride;
+    const int64_t               nrows   = is_x ? v.P : v.Q;
+    const int64_t               span    = (is_x != v.swapped) ? v.spanA : v.spanB;
+    std::vector<int>            seen(BR * 8, 0);
+    constexpr int               NL = BR / 32;
+    for(int wave = 0; wave < 4; wave++)
+        for(int lane = 0; lane < 64; lane++)
+            for(int i = 0; i < NL; i++)
+            {
+                const int    s  = (wave * NL + i) * 64 + lane;
+                const HdSlot sl = hk_stage_slot<KF, BR>(s);
+                if(KF)
+                {
+                    CHECK(sl.row >= 0 && sl.row < BR && sl.k >= 0 && sl.k + 8 <= 64 && sl.k % 8 == 0, "%s %s slot %d -> row %d k %d", c.name.c_str(), what, s,
+                          sl.row, sl.k);
+                    // the LDS bytes 16 s .. 16 s + 15 of a stage laid out [row][8 chunks] are where the readers look for this chunk
+                    CHECK(s == sl.row * 8 + hk_chunk_pos(sl.row, sl.k / 8), "%s %s slot %d is not where the readers look", c.name.c_str(), what, s);
+                    seen[(size_t)(sl.row * 8 + sl.k / 8)]++;
+                }
+                else
+                {
+                    CHECK(sl.row >= 0 && sl.row + 8 <= BR && sl.row % 8 == 0 && sl.k >= 0 && sl.k < 64, "%s %s slot %d -> row %d k %d", c.name.c_str(), what, s,
+                          sl.row, sl.k);
+                    // the LDS elements 8 s .. 8 s + 7 of a stage laid out [k][BR] are where the readers look for these 8 rows
+                    CHECK(8 * s == sl.k * BR + hd_row_pos(sl.row, sl.k), "%s %s slot %d is not where the readers look", c.name.c_str(), what, s);
+                    seen[(size_t)(sl.k * (BR / 8) + sl.row / 8)]++;
+                }
+                CHECK((size_t)(r0 + sl.row) < rtab.size(), "%s %s row table index %d of %zu", c.name.c_str(), what, r0 + sl.row, rtab.size());
+                const int64_t rowpart = rtab[(size_t)(r0 + sl.row)];
+                for(int j = 1; !KF && j < 8 && r0 + sl.row + j < nrows; j++)
+                    CHECK(rtab[(size_t)(r0 + sl.row + j)] - rowpart == j, "%s %s row run broken at %d", c.name.c_str(), what, r0 + sl.row);
+                const uint64_t lanepart = 2ull * ((uint64_t)rowpart + (uint64_t)sl.k * (uint64_t)kstride);
+                CHECK(lanepart <= 0xFFFFFFFFull, "%s %s lane offset overflows 32 bits", c.name.c_str(), what);
+                for(int o : origins)
+                {
+                    CHECK(o >= 0 && o + sl.k + (KF ? 8 : 1) <= v.K, "%s %s k %d of %lld", c.name.c_str(), what, o + sl.k, (long long)v.K);
+                    const uint64_t origin = 2ull * (uint64_t)o * (uint64_t)kstride;
+                    CHECK(origin <= 0xFFFFFFFFull, "%s %s origin overflows 32 bits", c.name.c_str(), what);
+                    const int64_t off = rowpart + (int64_t)(o + sl.k) * kstride;
+                    CHECK((uint64_t)off * 2 == lanepart + origin, "%s %s address parts", c.name.c_str(), what);
+                    CHECK(off >= 0 && off + 8 <= span, "%s %s r0 %d slot %d origin %d: elements %lld..+8 of %lld", c.name.c_str(), what, r0, s, o,
+                          (long long)off, (long long)span);
+                    CHECK(off % 8 == 0, "%s %s r0 %d slot %d origin %d: offset %lld not a multiple of 8", c.name.c_str(), what, r0, s, o, (long long)off);
+                    for(int j = 0; j < (KF ? 8 : 1); j++)
+                        CHECK(ktab[(size_t)(o + sl.k + j)] == (int64_t)(o + sl.k + j) * kstride && (!KF || j == 0 || kstride == 1), "%s %s k run broken at %d",
+                              c.name.c_str(), what, o + sl.k);
+                }
+            }
+    for(size_t i = 0; i < seen.size(); i++)
+        CHECK(seen[i] == 1, "%s %s chunk %zu filled %d times", c.name.c_str(), what, i, seen[i]);
+    if(KF)
+    {
+        // the operand reads: lane l of k-step ks reads chunk 4 ks + l / 16 of row (wave row) + 16 b + l % 16; 16 consecutive
+        // lanes must touch 16 different 16-byte bank groups (a row is 128 bytes = half of the 64 banks)
+        for(int ks = 0; ks < 2; ks++)
+            for(int g = 0; g < 4; g++)
+            {
+                int groups = 0;
+                for(int l = 16 * g; l < 16 * g + 16; l++)
+                    groups |= 1 << (((l & 15) & 1) * 8 + hk_chunk_pos(l & 15, 4 * ks + (l >> 4)));
+                CHECK(groups == 0xFFFF, "%s %s k-step %d lanes %d..: bank groups %x", c.name.c_str(), what, ks, 16 * g, groups);
+            }
+    }
+    else
+    {
+        // a transposing read: lane g of a 16-lane group points at the 4 consecutive rows 4 (g % 4) .. + 3 of k-row g / 4; they must be
+        // 8 contiguous bytes, and the group's 16 words must lie in 16 different 8-byte bank pairs (4 k-rows x 32 bytes)
+        for(int b = 0; b < BR / 32; b++)
+            for(int grp = 0; grp < 4; grp++)
+            {
+                unsigned long long pairs = 0;
+                for(int g = 0; g < 16; g++)
+                {
+                    const int k = 8 * grp + (g >> 2), r = 16 * b + 4 * (g & 3);
+                    CHECK(hd_row_pos(r + 3, k) == hd_row_pos(r, k) + 3, "%s %s rows %d..+3 at k %d are not contiguous in LDS", c.name.c_str(), what, r, k);
+                    pairs |= 1ull << (((k * BR + hd_row_pos(r, k)) / 4) % 32);
+                }
+                CHECK(__builtin_popcountll(pairs) == 16, "%s %s block %d group %d: transposing read touches %d bank pairs", c.name.c_str(), what, b, grp,
+                      __builtin_popcountll(pairs));
+            }
+    }
+}
+
+static long check_hk_tile(const Case& c, const GemmView& v)
+{
+    long      walked = 0;
+    const int K      = (int)v.K;
+    const int tiles_p = (int)((v.P + 255) / 256), tiles_q = (int)((v.Q + 255) / 256);
+    const int ktiles  = (K + 63) / 64;
+    for(int want = 1; want <= 5; want++)
+    {
+        int split = std::min(want, ktiles);
+        int per   = (ktiles + split - 1) / split;
+        split     = (ktiles + per - 1) / per;
+        std::vector<int> covered((size_t)K, 0);
+        std::vector<int> origins;
+        for(int z = 0; z < split; z++)
+        {
+            const HkSlice sl = hk_slice(K, z * per, per);
+            CHECK(sl.nt >= 0 && sl.n_load >= 1 && sl.tail >= 0 && sl.tail <= 3, "%s K %d slice %d/%d: nt %d tail %d", c.name.c_str(), K, z, split, sl.nt, sl.tail);
+            for(int u = 0; u < sl.nt; u++)
+                for(int k = 0; k < 64; k++)
+                    covered[(size_t)((z * per + u) * 64 + k)]++;
+            // the tail tile is loaded from K - 64 and its last `tail` k-steps are multiplied
+            for(int k = K - 16 * sl.tail; k < K; k++)
+                covered[(size_t)k]++;
+            int ko = sl.k00;
+            for(int u = 0; u < sl.n_load + 8; u++)
+            {
+                CHECK(ko >= 0 && ko <= K - 64, "%s origin %d out of range", c.name.c_str(), ko);
+                if(u < sl.nt)
+                    CHECK(ko == (z * per + u) * 64, "%s whole tile %d origin %d", c.name.c_str(), u, ko);
+                else if(sl.tail)
+                    CHECK(ko == K - 64, "%s tail tile origin %d", c.name.c_str(), ko);
+                else
+                    CHECK(ko == (z * per + sl.nt - 1) * 64, "%s tile %d beyond the slice at %d", c.name.c_str(), u, ko);
+                origins.push_back(ko);
+                ko = hk_next_origin(ko, sl.klast);
+            }
+        }
+        for(int k = 0; k < K; k++)
+            CHECK(covered[(size_t)k] == 1, "%s K %d split %d: k %d multiplied %d times", c.name.c_str(), K, split, k, covered[(size_t)k]);
+        std::sort(origins.begin(), origins.end());
+        origins.erase(std::unique(origins.begin(), origins.end()), origins.end());
+        for(int tp : {0, tiles_p / 2, tiles_p - 1})
+            for(int tq : {0, tiles_q / 2, tiles_q - 1})
+            {
+                const int p_own = tp * 256, q_own = tq * 256;
+                const int p0 = (v.shift_p && p_own + 256 > v.P) ? (int)v.P - 256 : p_own;
+                const int q0 = (v.shift_q && q_own + 256 > v.Q) ? (int)v.Q - 256 : q_own;
+                if(v.x_kfast)
+                    check_hk_operand<true, 256>("X", c, v, true, p0, origins);
+                else
+                    check_hk_operand<false, 256>("X", c, v, true, p0, origins);
+                if(v.y_kfast)
+                    check_hk_operand<true, 256>("Y", c, v, false, q0, origins);
+                else
+                    check_hk_operand<false, 256>("Y", c, v, false, q0, origins);
+                walked += (long)origins.size() * 512 * 8;
+            }
+        if(want > 1 && split == 1)
+            break;
+    }
+    return walked;
+}
+
 // ---- the 32/64-bit kernels: V rows per 16-byte vector, K tiles of BK, NLW loads per wave and operand; tiles of
 // ROWS x ROWS whose four waves share the stages (ROWS = 64), or load all of them each (ROWS = 32: the waves split K) ----
 template <int V, int ROWS, bool KF>
@@ -392,6 +551,14 @@ int main()
         rank4((t + "_mixed").c_str(), {0, 1, 20, 21}, {20, 21, 10, 11}, {10, 11, 0, 1}, 40, 9, 24, 13, kk.first, kk.second);
         rank4((t + "_mixed2").c_str(), {20, 21, 0, 1}, {10, 11, 20, 21}, {0, 1, 10, 11}, 40, 9, 24, 13, kk.first, kk.second);
     }
+    // K in tiles of 64 with every tail (0, 16, 32, 48 beyond a tile) and one tile only, every operand layout
+    for(auto kk : std::vector<std::pair<int, int>>{{16, 4}, {16, 5}, {16, 7}, {16, 8}, {16, 11}, {16, 14}, {16, 21}})
+    {
+        const std::string t = "k" + std::to_string(kk.first * kk.second);
+        rank4((t + "_kfast64").c_str(), {20, 21, 0, 1}, {20, 21, 10, 11}, {10, 11, 0, 1}, 40, 9, 24, 13, kk.first, kk.second);
+        rank4((t + "_rowfast64").c_str(), {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 40, 9, 24, 13, kk.first, kk.second);
+        rank4((t + "_mixed64").c_str(), {0, 1, 20, 21}, {20, 21, 10, 11}, {10, 11, 0, 1}, 40, 9, 24, 13, kk.first, kk.second);
+    }
     // 4096^3 (benchmark configuration 2) and its row-major form
     rank4("cfg2", {0, 1, 20, 21}, {10, 11, 20, 21}, {0, 1, 10, 11}, 64, 64, 64, 64, 64, 64);
     rank4("cfg2_rowmajor", {21, 20, 1, 0}, {21, 20, 11, 10}, {11, 10, 1, 0}, 64, 64, 64, 64, 64, 64);
@@ -429,7 +596,7 @@ int main()
         }
     }
     long walked = 0;
-    int  offered = 0;
+    int  offered = 0, offered_hk = 0;
     for(const Case& c : cases)
     {
         ProblemIn in;
@@ -446,8 +613,9 @@ int main()
         CHECK(st == PlanStatus::OK, "%s: %s", c.name.c_str(), why.c_str());
         if(st != PlanStatus::OK)
             continue;
-        // is a direct-load tile offered for it?  (tile ids 9: 256 x 256, 10: 256 x 192)
-        for(int tile : {9, 10})
+        // is a direct-load tile offered for it?  (tile ids 9: 256 x 256, 10: 256 x 192; 11: 256 x 256 in K tiles of 64
+        // on 16 x 16 x 32 MFMAs)
+        for(int tile : {9, 10, 11})
         {
             hiptk_problem_t p{};
             p.cls = v.cls, p.tile_id = tile, p.x_kfast = v.x_kfast, p.y_kfast = v.y_kfast, p.x_vec = v.x_vec, p.y_vec = v.y_vec;
@@ -460,11 +628,19 @@ int main()
             if(!avail)
                 continue;
             CHECK(v.x_vec == 8 && v.y_vec == 8 && v.K % 16 == 0 && v.K >= 32 && v.xy_aligned, "%s offered outside its restrictions", c.name.c_str());
+            if(tile == 11)
+            {
+                CHECK(v.k_affine && v.K >= 64, "%s offered the K-tile-of-64 kernel outside its restrictions", c.name.c_str());
+                offered_hk++;
+                walked += check_hk_tile(c, v);
+                continue;
+            }
             offered++;
             walked += tile == 9 ? check_tile_size<256>(c, v) : check_tile_size<192>(c, v);
         }
     }
     CHECK(offered >= 40, "only %d (case, tile) pairs were offered a direct-load kernel", offered);
+    CHECK(offered_hk >= 20, "only %d cases were offered the kernel with K tiles of 64", offered_hk);
 
     // ---- 32/64-bit classes ----
     // benchmark configurations 1 (256^3), 3 (1920^2 x 768), 4 (1024^2 x 512) and a tensor of 2^32 bytes and more

@@ -272,3 +272,30 @@ def test_plan_cache_retires_least_recently_used_states(monkeypatch):
     api.hiptensorDestroy(h)
     with pytest.raises(api.HiptensorError):
         api.planInfo(cs[3].plan)
+
+
+def test_plan_cache_never_retires_a_state_that_is_held(monkeypatch):
+    """A state that has been executed (or retained: the same mark, set here without a device) may still be
+    read by the device - a captured graph replays its table addresses - so the cache must skip it when it
+    looks for a state to retire, and grow when every state is held."""
+    monkeypatch.setenv("HIPTENSOR_AMD_PLAN_CACHE", "2")
+    h = api.check(api.hiptensorCreateHostOnly())
+    first = wl.Contraction(h, cases.rank_case(2, "f32", 1.0, None))
+    assert api.planRetain(first.plan) == 0
+    second = wl.Contraction(h, cases.rank_case(3, "f32", 1.0, None))
+    third = wl.Contraction(h, cases.rank_case(4, "f32", 1.0, None))  # retires `second`, the only one not held
+    assert api.planCacheInfo(h)[0] == 2
+    assert api.planInfo(first.plan)["kernel_name"]
+    with pytest.raises(api.HiptensorError):
+        api.planInfo(second.plan)
+    assert api.planRetain(second.plan) == api.HIPTENSOR_STATUS_INTERNAL_ERROR
+    assert api.planRetain(third.plan) == 0
+    fourth = wl.Contraction(h, cases.rank_case(5, "f32", 1.0, None))  # nothing to retire: the cache grows
+    assert api.planCacheInfo(h)[0] == 3
+    for c in (first, third, fourth):
+        assert api.planInfo(c.plan)["kernel_name"]
+    # re-planning the retired problem gives a fresh, valid state
+    again = wl.Contraction(h, cases.rank_case(3, "f32", 1.0, None))
+    assert api.planInfo(again.plan)["kernel_name"]
+    api.hiptensorDestroy(h)
+    assert api.planRetain(first.plan) == api.HIPTENSOR_STATUS_INTERNAL_ERROR

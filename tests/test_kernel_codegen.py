@@ -104,3 +104,45 @@ def test_every_32_64_bit_direct_load_instantiation(tmp_path, unit):
             valu = sorted({o for o in ops if o.startswith("v_") and not o.startswith("v_mfma")})
             assert not valu, f"vector ALU instructions in the main loop of {symbol}: {valu}"
             assert not any(o.startswith(("s_cbranch", "s_branch", "scratch_")) for o in ops), symbol
+
+
+@pytest.mark.parametrize("unit", ["contract_f16_hk_kx", "contract_f16_hk_rx", "contract_bf16_hk_kx", "contract_bf16_hk_rx"])
+def test_16x16x32_direct_load_loops_hold_no_wait_states(tmp_path, unit):
+    """The 16-bit kernels on v_mfma_f32_16x16x32 (K tiles of 64).  A 16-cycle MFMA leaves a single wave three issue
+    slots, and s_nop N holds N + 1 of them, so the direct loads inside the loop are issued WITHOUT the wait states the
+    load helper otherwise puts in front (they guard a scalar register written by a vector instruction, e.g. the
+    reload of a spilled SGPR, being read by the load within 5 wait states; one such read of a stale address faulted
+    the device once).  That is safe only while the loop holds no vector instruction that writes a scalar register
+    and nothing but these helpers writes M0: both are checked here, for every wave position's copy of the loop of every
+    instantiation, beside what the other main loops are held to."""
+    lines = device_asm(unit, tmp_path)
+    symbols = [l.split(":")[0] for l in lines if re.match(r"^_ZN5hiptk18contract_hk_kernel.*EvNS_5KArgsE:", l)]
+    assert len(symbols) == 2, symbols
+    for symbol in symbols:
+        body = kernel_body(lines, symbol)
+        # two K tiles of 2 x 64 MFMAs: the rings' common period (the epilogue's loops, which enclose the K tail's MFMAs, are longer)
+        loops = [(a, b) for a, b in main_loops(body, 256) if len(opcodes(body, a, b)) < 1024]
+        assert len(loops) == 4, f"{symbol}: {len(loops)} main loops (one per wave position expected)"
+        for a, b in loops:
+            ops = opcodes(body, a, b)
+            assert sum(o.startswith("v_mfma_f32_16x16x32") for o in ops) == 256, symbol
+            valu = sorted({o for o in ops if o.startswith("v_") and not o.startswith("v_mfma")})
+            assert not valu, f"vector ALU instructions in the main loop of {symbol}: {valu}"
+            assert not any(o.startswith(("s_cbranch", "s_branch", "scratch_", "buffer_store", "global_store")) for o in ops), symbol
+            # (the first load of a window keeps its wait states: one s_nop per K tile in one wave position's copy)
+            assert sum(o == "s_nop" for o in ops) <= 2, f"{symbol}: s_nop in the main loop"
+            assert sum(o == "global_load_lds_dwordx4" for o in ops) == 32, symbol
+            # M0 is written by the load helpers' s_add_u32 only, once per load, in front of the MFMA before it
+            text = [l for l in body[a:b] if "m0" in l.split(";")[0]]
+            assert len(text) == 32 and all(l.strip().startswith("s_add_u32 m0,") for l in text), text[:5]
+            # instructions beside the MFMAs: fewer than three per MFMA on average
+            assert len(ops) - 256 < 3 * 256 // 2, f"{symbol}: {len(ops) - 256} instructions beside 256 MFMAs"
+
+
+def test_direct_load_loops_leave_m0_alone(tmp_path):
+    """The 32 x 32 x 16 direct-load kernel writes M0 one MFMA ahead of the load that reads it, in separate asm
+    statements: nothing the compiler generates in between may touch M0."""
+    body = kernel_body(device_asm("contract_f16_hd", tmp_path), "_ZN5hiptk18contract_hd_kernelINS_9TraitsF16ELb0ELb0ELi256ELb1EEEvNS_5KArgsE")
+    for a, b in main_loops(body, 128):
+        text = [l for l in body[a:b] if "m0" in l.split(";")[0]]
+        assert text and all(l.strip().startswith("s_add_u32 m0,") for l in text), text[:5]
