@@ -833,6 +833,8 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         p.xy_aligned = v.xy_aligned;
         p.x_max_off = (int32_t)v.x_max_off;
         p.y_max_off = (int32_t)v.y_max_off;
+        p.x_rows_adjacent = v.x_rows_adjacent;
+        p.y_rows_adjacent = v.y_rows_adjacent;
         p.xk_stride            = (int32_t)v.xk_stride;
         p.yk_stride            = (int32_t)v.yk_stride;
         (void)hiptk_resolve(&p); // the registry is searched here, once, not at every launch

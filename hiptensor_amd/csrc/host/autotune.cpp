@@ -93,6 +93,8 @@ namespace hipta
         p.xy_aligned = v.xy_aligned;
         p.x_max_off = (int32_t)v.x_max_off;
         p.y_max_off = (int32_t)v.y_max_off;
+        p.x_rows_adjacent = v.x_rows_adjacent;
+        p.y_rows_adjacent = v.y_rows_adjacent;
         p.xk_stride = (int32_t)v.xk_stride;
         p.yk_stride = (int32_t)v.yk_stride;
         p.xp      = base + offs[0];

@@ -517,6 +517,24 @@ namespace hipta
                                : 0;
         }
 
+        // k-contiguous operand: which neighbour of a vector is its neighbour in memory too, the next row's or the next
+        // vector of its own row?
+        {
+            auto rows_adjacent = [](const std::vector<int32_t>& rows, int64_t nrows, const std::vector<int32_t>& ks, int64_t nk, bool kfast, int vec) {
+                if(!kfast || vec < 2 || nrows < 2)
+                    return 0;
+                int64_t by_row = 0, by_k = 0, k_pairs = 0;
+                for(int64_t r = 0; r + 1 < nrows; r++)
+                    by_row += (int64_t)rows[(size_t)r + 1] - rows[(size_t)r] == vec;
+                for(int64_t k = 0; k + vec < nk; k += vec, k_pairs++)
+                    by_k += (int64_t)ks[(size_t)(k + vec)] - ks[(size_t)k] == vec;
+                // (as fractions of the pairs there are)
+                return by_row * (k_pairs > 0 ? k_pairs : 1) > by_k * (nrows - 1) ? 1 : 0;
+            };
+            v.x_rows_adjacent = rows_adjacent(v.xp, v.P, v.xk, v.K, v.x_kfast != 0, v.x_vec);
+            v.y_rows_adjacent = rows_adjacent(v.yq, v.Q, v.yk, v.K, v.y_kfast != 0, v.y_vec);
+        }
+
         v.spanA = span_elems(A.len, A.stride);
         v.spanB = span_elems(B.len, B.stride);
         v.spanD = span_elems(D.len, D.stride);

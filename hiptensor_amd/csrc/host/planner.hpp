@@ -68,6 +68,9 @@ namespace hipta
         int xy_aligned = 0;
         // largest element offset of X / Y that the tables address
         int64_t x_max_off = 0, y_max_off = 0;
+        // k-contiguous operand: the vectors of consecutive rows are neighbours in memory more often than consecutive
+        // vectors of one row (a hint for the kernels' LDS layout)
+        int x_rows_adjacent = 0, y_rows_adjacent = 0;
         int elem_bytes = 0;
         // bytes each tensor spans in memory (1 + sum (len-1)*stride elements)
         int64_t spanA = 0, spanB = 0, spanC = 0, spanD = 0;

@@ -31,6 +31,7 @@ namespace hipta
                 s.threads   = ti.threads;
                 s.lds_bytes = ti.lds_bytes;
                 s.direct    = ti.k_multiple > 0;
+                s.mfma_k    = ti.mfma_k;
                 s.name      = ti.name;
                 uint64_t h  = 0x68697074656e73ull;
                 for(uint64_t x : {(uint64_t)cls, (uint64_t)t, (uint64_t)ti.bp, (uint64_t)ti.bq, (uint64_t)ti.bk})
@@ -190,6 +191,17 @@ namespace hipta
             r.alone *= f;
             r.full *= f;
             round_extra_us = 6.5;
+        }
+        else if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.direct && s.bk == 32 && s.mfma_k == 32)
+        {
+            // The 256 x 192 tile on 16 x 16 x 32 MFMAs that reads its k offsets from tables and loads K tiles of 32 into
+            // a ring of four stages.  Rank-6 benchmark layout (5376 x 6912 x 4080 f16 bilinear, three rounds of tiles,
+            // X row-contiguous in runs of 64 bytes, Y k-contiguous in runs of 16, staged chunk-major): 265 us against
+            // 300 on the 32 x 32 x 16 tile below (main loop of a round 67 against 80 us, epilogue 16 and 17.5).
+            const double f = (v.x_kfast && v.y_kfast) ? 1.085 : (v.x_kfast || v.y_kfast) ? 1.225 : 1.36;
+            r.alone *= f;
+            r.full *= f;
+            round_extra_us = 5.0;
         }
         else if(class_flops_per_clk_cu(v.cls) == 4096.0 && s.threads == 256 && s.bp * s.bq >= 49152 && s.bk == 32)
         {

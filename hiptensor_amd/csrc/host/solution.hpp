@@ -24,6 +24,7 @@ namespace hipta
         int         cls, tile_id;
         int         bp, bq, bk, threads, lds_bytes;
         bool        direct; // operand tiles go from global memory straight into LDS
+        int         mfma_k; // 32: a 16-bit tile on v_mfma_f32_16x16x32 (else 0)
         std::string name;
     };
 

@@ -4,8 +4,8 @@
 namespace hiptk
 {
     static const KernelEntry k_entries[] = {
-        HIPTK_HK_ENTRY(TraitsBF16, 11, 256, false, true, 2, 2, 2),
-        HIPTK_HK_ENTRY(TraitsBF16, 11, 256, false, false, 2, 2, 2),
+        HIPTK_HK_ENTRY(TraitsBF16, 11, 256, false, true, 2, 2, 4),
+        HIPTK_HK_ENTRY(TraitsBF16, 11, 256, false, false, 2, 2, 4),
     };
 
     const KernelEntry* entries_bf16_hk_rx(int* count)

@@ -385,7 +385,7 @@ namespace hiptk
             substep(wv_c, I0{}, cur, I1{}, std::false_type{}, s_c);
             y_next(s_c); // tile t + 4 shares tile t's stage
             // Every wave has issued its reads of tile t.  Tile t + 1 must have landed.
-            __builtin_amdgcn_s_waitcnt(waitcnt_vm(NWAIT));
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(NWAIT));
             lds_barrier();
             __builtin_amdgcn_sched_barrier(0);
             // substep 1: multiply k 16..31 of tile t, fetch k 0..15 of tile t + 1 (beyond the last

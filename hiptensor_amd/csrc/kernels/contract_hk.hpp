@@ -29,7 +29,7 @@
 //     the current one is multiplied (a whole k-step ahead: 128 registers), so every wave has issued its
 //     last read of tile t when the last k-step of tile t begins: there, after the barrier that also hands
 //     tile t + 1 to the readers, the stages of tile t are free, and the loads of tile t + NSY (Y) and
-//     t + NSX (X) are issued into them during the 128 MFMAs that follow, one every 2 SP MFMAs per wave,
+//     t + NSX (X) are issued into them during the 128 MFMAs that follow, one every SP MFMAs per wave,
 //     the operand with the shorter ring first.
 //   * Swizzles.  k-contiguous: the 16-byte chunk at position c of a row holds chunk c ^ ((row / 2) % 8)
 //     of that row (each lane picks its global source accordingly): 16 consecutive lanes of a
@@ -129,6 +129,20 @@ namespace hiptk
         }
     };
 
+    // Which block (row i, column j) of the wave tile the m-th MFMA of a k-step multiplies: the 8 x 8 blocks
+    // are walked in squares of 2 x 2, the squares row by row.  The order changes nothing in cycles but the
+    // clock the device holds (4096^3, k-contiguous operands: 101.6 us row by row or column by column, 100.8
+    // row by row in alternating directions, 99.9 in 2 x 2 squares, the same in 2 x 4 strips and along a
+    // Z curve; a loop of nothing but these MFMAs: 1741 MHz row by row, 1949 in squares).
+    constexpr int hk_block_i(int m, int nbq)
+    {
+        return 2 * ((m / 4) / (nbq / 2)) + (m % 4) / 2;
+    }
+    constexpr int hk_block_j(int m, int nbq)
+    {
+        return 2 * ((m / 4) % (nbq / 2)) + m % 2;
+    }
+
     // The MFMA of the main loop, as inline assembly that accumulates in place in AGPRs.  The compiler
     // does not know these are MFMAs, so whoever reads the accumulators afterwards waits first
     // (hk_mfma_drain).
@@ -162,7 +176,7 @@ namespace hiptk
         constexpr int BP = G::BP, NXL = G::NXL, NYL = G::NYL;
         constexpr int TP = 4, TQ = BQ / 64, WP = 2, WQ = 2; // 32 x 32 blocks of a wave tile (what the epilogue walks)
         // MFMA blocks of a wave tile, k-steps per K tile, MFMAs per k-step, MFMAs between two loads of a wave
-        constexpr int NBP = 2 * TP, NBQ = 2 * TQ, KST = 2, NM = NBP * NBQ, SPM = 2 * SP;
+        constexpr int NBP = 2 * TP, NBQ = 2 * TQ, KST = 2, NM = NBP * NBQ, SPM = SP;
         constexpr int NL = NXL + NYL; // loads per wave and K tile
         // the operand with the shorter ring is requested first in every tile's window
         constexpr bool YFIRST = NSY <= NSX;
@@ -285,8 +299,8 @@ namespace hiptk
         u32x4_t xf[2][NBP], yf[2][NBQ];
 
         // One k-step: NM MFMAs out of register set KS % 2; the operand fetches of the next k-step (k-step
-        // NKS of the stages nx / ny) into the other set, X block i in front of row i's first MFMA and Y
-        // block i in front of its fifth; and this wave's loads of the window slots G0 .. G0 + NM - 1.
+        // NKS of the stages nx / ny) into the other set, X block i in front of MFMA NBQ i and Y block j in
+        // front of MFMA NBP j + NBP / 2; and this wave's loads of the window slots G0 .. G0 + NM - 1.
         // sched_barrier(0) after every MFMA keeps the issue order as written.
         auto kstep = [&](auto wv_c, auto ks_c, const uint16_t* nx, const uint16_t* ny, auto nks_c, auto g0_c) __attribute__((always_inline)) {
             constexpr int KS   = decltype(ks_c)::value;
@@ -295,13 +309,15 @@ namespace hiptk
             constexpr int slot = KS & 1;
             hk_static_for<NM>([&](auto m_c) __attribute__((always_inline)) {
                 constexpr int m = decltype(m_c)::value;
-                constexpr int i = m / NBQ;
                 if constexpr(m % NBQ == 0)
-                    xf[slot ^ 1][i] = fx.load(nx, i, NKS);
-                if constexpr(m % NBQ == 4)
-                    yf[slot ^ 1][i] = fy.load(ny, i, NKS);
+                    xf[slot ^ 1][m / NBQ] = fx.load(nx, m / NBQ, NKS);
+                if constexpr(m % NBP == NBP / 2)
+                    yf[slot ^ 1][m / NBP] = fy.load(ny, m / NBP, NKS);
                 window_slot(wv_c, std::integral_constant<int, G0 + m>{}, std::true_type{});
-                hk_mfma16_acc(Tr{}, acc[m / NBQ][m % NBQ], xf[slot][m / NBQ], yf[slot][m % NBQ]);
+                {
+                    constexpr int bi = hk_block_i(m, NBQ), bj = hk_block_j(m, NBQ);
+                    hk_mfma16_acc(Tr{}, acc[bi][bj], xf[slot][bi], yf[slot][bj]);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             });
         };
@@ -321,7 +337,7 @@ namespace hiptk
             // k-step 0 fetches k-step 1 (the window that opened in the last k-step of the tile before goes on)
             kstep(wv_c, I0{}, cx, cy, I1{}, std::integral_constant<int, NM>{});
             // Every wave has issued its reads of tile t.  Tile t + 1 must have landed.
-            __builtin_amdgcn_s_waitcnt(waitcnt_vm(NWAIT));
+            __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(NWAIT));
             lds_barrier();
             __builtin_amdgcn_sched_barrier(0);
             // the stages of tile t are free: the window of tiles t + NSY (Y) and t + NSX (X) opens
@@ -471,7 +487,7 @@ namespace hiptk
     {                                                                                                       \
         TR::CLS, ID, XKF, YKF, 8, 8, true, 256, BQ, 64, 256, hiptk::HkGeom<BQ, NSX, NSY>::LDS_BYTES,         \
             #TR "_256x" #BQ "x64_x" #XKF "8_y" #YKF "8_kafftrue_direct2x2_m16x16x32",                       \
-            &hiptk::launch_hk<hiptk::TR, XKF, YKF, BQ, NSX, NSY, SP>, 16                                    \
+            &hiptk::launch_hk<hiptk::TR, XKF, YKF, BQ, NSX, NSY, SP>, 16, 32                                  \
     }
 #define HIPTK_HK_TILE(TR, ID, BQ, NSX, NSY, SP)                                                              \
     HIPTK_HK_ENTRY(TR, ID, BQ, true, true, NSX, NSY, SP), HIPTK_HK_ENTRY(TR, ID, BQ, true, false, NSX, NSY, SP), \

@@ -62,10 +62,24 @@ namespace hiptk
         asm volatile("s_nop 4\n\tglobal_load_lds_dword %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
     }
 
+    // The 4-byte load without wait states in front of it: under the conditions of dma_load_in_loop
+    __device__ __forceinline__ void dma_load1_bare(uint32_t voff, const void* base)
+    {
+        asm volatile("global_load_lds_dword %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
+    }
+
     // s_waitcnt immediates (gfx9 encoding): vmcnt(N) with the other counters left alone
     constexpr int waitcnt_vm(int n)
     {
         return (n & 15) | ((n >> 4) << 14) | 0x0F70;
+    }
+    // vmcnt(N) and lgkmcnt(0) in one: what a wave waits for before the barrier that hands a ring stage on (its
+    // loads of the tile the next step reads have landed; its own LDS reads of the tile just multiplied are done,
+    // so that the stage may be overwritten).  Written out because the wait the workgroup fence implies was
+    // found missing in front of the first barrier of an unrolled loop body.
+    constexpr int waitcnt_vm_lgkm0(int n)
+    {
+        return (n & 15) | ((n >> 4) << 14) | 0x0070;
     }
     // lgkmcnt(0) with the other counters left alone
     constexpr int waitcnt_lgkm0 = 0xC07F;

@@ -211,4 +211,28 @@ namespace hiptk
         }
         return o;
     }
+    // A k-contiguous operand whose runs along k are one vector long has its neighbouring vectors elsewhere: where
+    // those of consecutive rows follow one another in memory, the ring kernel (contract_hr.hpp) lays the stage out
+    // chunk-major, stage[4 chunks of 8 k][rows][8]: a direct load's 64 lanes then cover 64 consecutive rows of one
+    // chunk (4 lanes = 64 contiguous bytes, one access of the vector cache) instead of 16 rows x 4 chunks (4 lanes =
+    // 4 places), and the MFMA operand read (16 lanes = 16 consecutive rows of one chunk = 256 contiguous bytes)
+    // needs no swizzle.  `chunked` is that choice; it is a matter of speed only.
+    template <bool KF, int BR>
+    HIPTK_HD_FN HdSlot hr_slot(int s, bool chunked)
+    {
+        if(KF && chunked)
+        {
+            HdSlot o;
+            o.row = s % BR;
+            o.k   = 8 * (s / BR);
+            return o;
+        }
+        return hd_slot<KF, BR>(s);
+    }
+    // element position in a k-contiguous operand's stage of the 8 k from 8 * chunk on of row `row`
+    template <int BR>
+    HIPTK_HD_FN int hr_chunk_elem(int row, int chunk, bool chunked)
+    {
+        return chunked ? (chunk * BR + row) * 8 : row * HD_BK + ((chunk ^ ((row >> 2) & 3)) << 3);
+    }
 }

@@ -31,6 +31,9 @@ namespace hiptk
         int32_t shift_p, shift_q;
         // byte offset of the last 16-byte vector of X / Y that the tables address (direct-load kernels, table form)
         uint32_t x_last_vec, y_last_vec;
+        // 1: a k-contiguous X / Y is staged chunk-major by the kernels that can (the vectors of consecutive rows are
+        // neighbours in memory; those of consecutive k are not)
+        int32_t x_chunked, y_chunked;
         double   alpha[2], beta[2];
     };
 
@@ -46,6 +49,7 @@ namespace hiptk
         const char* name;
         launch_fn   launch;
         int32_t     k_multiple; // 0: any K; else K must be a multiple of this and at least bk
+        int32_t     mfma_k; // reduction depth of the MFMA instruction the tile is built on, where the selection tells tiles apart by it (else 0)
     };
 
     // Each kernel translation unit contributes its table.
@@ -65,6 +69,10 @@ namespace hiptk
     const KernelEntry* entries_f16_hk_rx(int* count);
     const KernelEntry* entries_bf16_hk_kx(int* count);
     const KernelEntry* entries_bf16_hk_rx(int* count);
+    const KernelEntry* entries_f16_hr192_kx(int* count);
+    const KernelEntry* entries_f16_hr192_rx(int* count);
+    const KernelEntry* entries_bf16_hr192_kx(int* count);
+    const KernelEntry* entries_bf16_hr192_rx(int* count);
     const KernelEntry* entries_f16_v4(int* count);
     const KernelEntry* entries_f16_v2(int* count);
     const KernelEntry* entries_bf16_v4(int* count);

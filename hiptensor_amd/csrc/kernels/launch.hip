@@ -28,6 +28,10 @@ namespace hiptk
                                           entries_f16_hk_rx,
                                           entries_bf16_hk_kx,
                                           entries_bf16_hk_rx,
+                                          entries_f16_hr192_kx,
+                                          entries_f16_hr192_rx,
+                                          entries_bf16_hr192_kx,
+                                          entries_bf16_hr192_rx,
                                           entries_f16_aff,
                                           entries_bf16_aff,
                                           entries_f16_vec,
@@ -289,6 +293,7 @@ extern "C" int hiptk_tile_info(int cls, int tile_id, hiptk_tile_info_t* out)
             out->threads   = e.threads;
             out->lds_bytes = e.lds_bytes;
             out->k_multiple = e.k_multiple;
+            out->mfma_k     = e.mfma_k;
             std::snprintf(out->name, sizeof(out->name), "cls%d_%dx%dx%d", cls, e.bp, e.bq, e.bk);
             return HIPTK_OK;
         }
@@ -379,6 +384,8 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
         a.x_last_vec     = prob->x_max_off >= back ? (uint32_t)eb * (uint32_t)(prob->x_max_off - back) : 0u;
         a.y_last_vec     = prob->y_max_off >= back ? (uint32_t)eb * (uint32_t)(prob->y_max_off - back) : 0u;
     }
+    a.x_chunked = (prob->x_kfast && prob->x_rows_adjacent) ? 1 : 0;
+    a.y_chunked = (prob->y_kfast && prob->y_rows_adjacent) ? 1 : 0;
     // A moved-back tile stores whole 8-element vectors of D that reach into its neighbour's
     // columns (same values).  When D is updated in place (C == D) the neighbour's elements must
     // not be read and written twice, so that case stores element by element.

@@ -64,6 +64,7 @@ typedef struct hiptk_tile_info
     int32_t k_multiple; /* 0: operand tiles staged through registers, any K.  Otherwise the tile loads
                            them straight into LDS: K must be a multiple of this (1: any) and at least bk,
                            and the problem xy_aligned                          */
+    int32_t mfma_k;     /* 32: a 16-bit tile built on v_mfma_f32_16x16x32 (else 0)   */
 } hiptk_tile_info_t;
 
 typedef struct hiptk_problem
@@ -109,6 +110,12 @@ typedef struct hiptk_problem
                                      themselves moved through LDS clamp every address to it, and the
                                      direct-load kernels are offered only while the byte offset of the
                                      last vector fits 32 bits */
+    int32_t x_rows_adjacent, y_rows_adjacent; /* a hint, for a k-contiguous operand only: 1 when the vectors of
+                                     consecutive rows follow one another in memory more often than consecutive
+                                     vectors of one row do (xp[p + 1] - xp[p] == x_vec against xk[k + x_vec] -
+                                     xk[k] == x_vec).  The kernels that load operand tiles straight into LDS and
+                                     read k offsets from the tables then stage the operand chunk-major, so that
+                                     neighbouring lanes load neighbouring memory.  Any value gives the same results */
     /* Filled by hiptk_resolve (zero otherwise): the registry entries this problem runs, looked up once
      * when the plan is made instead of at every launch.  `kernel` is what hiptk_kernel_name names;
      * `kernel_unaligned` is what runs in its place when X or Y is not 16-byte aligned at the launch (the

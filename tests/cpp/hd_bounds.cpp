@@ -31,6 +31,8 @@ using hiptk::hk_next_origin;
 using hiptk::hk_slice;
 using hiptk::hd_row_pos;
 using hiptk::hk_stage_slot;
+using hiptk::hr_chunk_elem;
+using hiptk::hr_slot;
 using hiptk::HkSlice;
 using hiptk::wd_next_origin;
 using hiptk::wd_slot;
@@ -100,8 +102,9 @@ static TensorIn tensor(const Case& c, const std::vector<int32_t>& modes, std::ve
 
 template <bool KF, int BR>
 static void check_operand(const char* what, const Case& c, const GemmView& v, bool is_x, int r0, const std::vector<int>& origins,
-                          bool affine)
+                          bool affine, bool ring = false) // ring: the kernel on 16 x 16 x 32 MFMAs (contract_hr.hpp), table form only
 {
+    const bool chunked = ring && KF && (is_x ? v.x_rows_adjacent : v.y_rows_adjacent) != 0;
     const std::vector<int32_t>& rtab    = is_x ? v.xp : v.yq;
     const std::vector<int32_t>& ktab    = is_x ? v.xk : v.yk;
     const int64_t               kstride = is_x ? v.xk_stride : v.yk_stride;
@@ -116,11 +119,14 @@ static void check_operand(const char* what, const Case& c, const GemmView& v, bo
             for(int i = 0; i < NL; i++)
             {
                 const int    s  = (wave * NL + i) * 64 + lane;
-                const HdSlot sl = hd_slot<KF, BR>(s);
+                const HdSlot sl = ring ? hr_slot<KF, BR>(s, chunked) : hd_slot<KF, BR>(s);
                 CHECK(sl.row >= 0 && sl.row + (KF ? 1 : 8) <= BR && sl.k >= 0 && sl.k + (KF ? 8 : 1) <= 32, "%s %s slot %d -> row %d k %d",
                       c.name.c_str(), what, s, sl.row, sl.k);
                 seen[KF ? sl.row * 4 + sl.k / 8 : sl.k * (BR / 8) + sl.row / 8]++;
-                if(KF)
+                if(ring) // the LDS elements 8 s .. 8 s + 7 are where the operand reads look for this vector
+                    CHECK(8 * s == (KF ? hr_chunk_elem<BR>(sl.row, sl.k / 8, chunked) : sl.k * BR + hd_row_pos(sl.row, sl.k)),
+                          "%s %s slot %d is not where the readers look", c.name.c_str(), what, s);
+                if(KF && !ring)
                 {
                     CHECK(k_first < 0 || k_first == sl.k, "%s %s lane %d: chunk differs between its loads", c.name.c_str(), what, lane);
                     k_first = sl.k;
@@ -157,10 +163,41 @@ static void check_operand(const char* what, const Case& c, const GemmView& v, bo
         }
     for(size_t i = 0; i < seen.size(); i++)
         CHECK(seen[i] == 1, "%s %s chunk %zu filled %d times", c.name.c_str(), what, i, seen[i]);
+    if(ring && KF)
+    {
+        // operand read of v_mfma_f32_16x16x32: lane l reads the 16 bytes of chunk l / 16 of row (block's first) + l % 16;
+        // 16 consecutive lanes must touch 16 different 16-byte groups of the 64 banks
+        for(int b = 0; b < BR / 16; b++)
+            for(int g = 0; g < 4; g++)
+            {
+                int groups = 0;
+                for(int l = 0; l < 16; l++)
+                    groups |= 1 << ((hr_chunk_elem<BR>(16 * b + l, g, chunked) / 8) % 16);
+                CHECK(groups == 0xFFFF, "%s %s block %d chunk %d: bank groups %x", c.name.c_str(), what, b, g, groups);
+            }
+    }
+    if(ring && !KF)
+    {
+        // a transposing read: lane g of a 16-lane group points at the rows 4 (g % 4) .. + 3 of k-row g / 4: 8 contiguous bytes,
+        // and the group's 16 words in 16 different 8-byte bank pairs
+        for(int b = 0; b < BR / 16; b++)
+            for(int grp = 0; grp < 8; grp++)
+            {
+                unsigned long long pairs = 0;
+                for(int g = 0; g < 16; g++)
+                {
+                    const int k = 8 * (grp & 3) + 4 * (grp >> 2) + (g >> 2), r = 16 * b + 4 * (g & 3);
+                    CHECK(hd_row_pos(r + 3, k) == hd_row_pos(r, k) + 3, "%s %s rows %d..+3 at k %d are not contiguous in LDS", c.name.c_str(), what, r, k);
+                    pairs |= 1ull << (((k * BR + hd_row_pos(r, k)) / 4) % 32);
+                }
+                CHECK(__builtin_popcountll(pairs) == 16, "%s %s block %d group %d: transposing read touches %d bank pairs", c.name.c_str(), what, b, grp,
+                      __builtin_popcountll(pairs));
+            }
+    }
 }
 
 template <int BQ>
-static long check_tile_size(const Case& c, const GemmView& v)
+static long check_tile_size(const Case& c, const GemmView& v, bool ring = false)
 {
     long      walked = 0;
     const int K      = (int)v.K;
@@ -211,14 +248,15 @@ static long check_tile_size(const Case& c, const GemmView& v)
                 const int p_own = tp * 256, q_own = tq * BQ;
                 const int p0 = (v.shift_p && p_own + 256 > v.P) ? (int)v.P - 256 : p_own;
                 const int q0 = (v.shift_q && q_own + BQ > v.Q) ? (int)v.Q - BQ : q_own;
+                const bool affine = !ring && v.k_affine != 0;
                 if(v.x_kfast)
-                    check_operand<true, 256>("X", c, v, true, p0, origins, v.k_affine != 0);
+                    check_operand<true, 256>("X", c, v, true, p0, origins, affine, ring);
                 else
-                    check_operand<false, 256>("X", c, v, true, p0, origins, v.k_affine != 0);
+                    check_operand<false, 256>("X", c, v, true, p0, origins, affine, ring);
                 if(v.y_kfast)
-                    check_operand<true, BQ>("Y", c, v, false, q0, origins, v.k_affine != 0);
+                    check_operand<true, BQ>("Y", c, v, false, q0, origins, affine, ring);
                 else
-                    check_operand<false, BQ>("Y", c, v, false, q0, origins, v.k_affine != 0);
+                    check_operand<false, BQ>("Y", c, v, false, q0, origins, affine, ring);
                 walked += (long)origins.size() * (256 + BQ) * 4;
             }
         if(want > 1 && split == 1)
@@ -230,7 +268,7 @@ static long check_tile_size(const Case& c, const GemmView& v)
 // ---- the 16-bit kernels on 16 x 16 x 32 MFMAs: K tiles of 64, stage[row][64] (k-contiguous operand) or stage[k][rows]
 // (row-contiguous), 8 loads per wave and operand ----
 template <bool KF, int BR>
-static void check_hk_operand(const char* what, const Case& c, const GemmView& v, bool is_x, int r0, const std::vector<int>& origins)
+static void check_hk_operand(const char* what, const Case& c, const GemmView& v, bool is_x, int r0, const std::vector<int>& origins, bool affine)
 {
     const std::vector<int32_t>& rtab    = is_x ? v.xp : v.yq;
     const std::vector<int32_t>& ktab    = is_x ? v.xk : v.yk;
@@ -265,21 +303,24 @@ static void check_hk_operand(const char* what, const Case& c, const GemmView& v,
                 const int64_t rowpart = rtab[(size_t)(r0 + sl.row)];
                 for(int j = 1; !KF && j < 8 && r0 + sl.row + j < nrows; j++)
                     CHECK(rtab[(size_t)(r0 + sl.row + j)] - rowpart == j, "%s %s row run broken at %d", c.name.c_str(), what, r0 + sl.row);
-                const uint64_t lanepart = 2ull * ((uint64_t)rowpart + (uint64_t)sl.k * (uint64_t)kstride);
+                const uint64_t lanepart = 2ull * ((uint64_t)rowpart + (affine ? (uint64_t)sl.k * (uint64_t)kstride : 0ull));
                 CHECK(lanepart <= 0xFFFFFFFFull, "%s %s lane offset overflows 32 bits", c.name.c_str(), what);
                 for(int o : origins)
                 {
                     CHECK(o >= 0 && o + sl.k + (KF ? 8 : 1) <= v.K, "%s %s k %d of %lld", c.name.c_str(), what, o + sl.k, (long long)v.K);
-                    const uint64_t origin = 2ull * (uint64_t)o * (uint64_t)kstride;
+                    // one k stride: origin in the scalar base; tables: the entry of the vector's first k, added to the row part
+                    const uint64_t origin = 2ull * (affine ? (uint64_t)o * (uint64_t)kstride : (uint64_t)ktab[(size_t)(o + sl.k)]);
                     CHECK(origin <= 0xFFFFFFFFull, "%s %s origin overflows 32 bits", c.name.c_str(), what);
-                    const int64_t off = rowpart + (int64_t)(o + sl.k) * kstride;
+                    const int64_t off = rowpart + (affine ? (int64_t)(o + sl.k) * kstride : (int64_t)ktab[(size_t)(o + sl.k)]);
                     CHECK((uint64_t)off * 2 == lanepart + origin, "%s %s address parts", c.name.c_str(), what);
+                    CHECK(off <= (is_x ? v.x_max_off : v.y_max_off) - 7, "%s %s offset %lld beyond the last vector", c.name.c_str(), what, (long long)off);
                     CHECK(off >= 0 && off + 8 <= span, "%s %s r0 %d slot %d origin %d: elements %lld..+8 of %lld", c.name.c_str(), what, r0, s, o,
                           (long long)off, (long long)span);
                     CHECK(off % 8 == 0, "%s %s r0 %d slot %d origin %d: offset %lld not a multiple of 8", c.name.c_str(), what, r0, s, o, (long long)off);
                     for(int j = 0; j < (KF ? 8 : 1); j++)
-                        CHECK(ktab[(size_t)(o + sl.k + j)] == (int64_t)(o + sl.k + j) * kstride && (!KF || j == 0 || kstride == 1), "%s %s k run broken at %d",
-                              c.name.c_str(), what, o + sl.k);
+                        CHECK(affine ? (ktab[(size_t)(o + sl.k + j)] == (int64_t)(o + sl.k + j) * kstride && (!KF || j == 0 || kstride == 1))
+                                     : (ktab[(size_t)(o + sl.k + j)] - ktab[(size_t)(o + sl.k)] == j),
+                              "%s %s k run broken at %d", c.name.c_str(), what, o + sl.k);
                 }
             }
     for(size_t i = 0; i < seen.size(); i++)
@@ -317,11 +358,12 @@ static void check_hk_operand(const char* what, const Case& c, const GemmView& v,
     }
 }
 
-static long check_hk_tile(const Case& c, const GemmView& v)
+template <int BQ>
+static long check_hk_tile(const Case& c, const GemmView& v, bool affine) // affine: the kernel multiplies a k stride (else it reads the tables)
 {
-    long      walked = 0;
-    const int K      = (int)v.K;
-    const int tiles_p = (int)((v.P + 255) / 256), tiles_q = (int)((v.Q + 255) / 256);
+    long       walked = 0;
+    const int  K      = (int)v.K;
+    const int  tiles_p = (int)((v.P + 255) / 256), tiles_q = (int)((v.Q + BQ - 1) / BQ);
     const int ktiles  = (K + 63) / 64;
     for(int want = 1; want <= 5; want++)
     {
@@ -340,18 +382,21 @@ static long check_hk_tile(const Case& c, const GemmView& v)
             // the tail tile is loaded from K - 64 and its last `tail` k-steps are multiplied
             for(int k = K - 16 * sl.tail; k < K; k++)
                 covered[(size_t)k]++;
-            int ko = sl.k00;
+            // one k stride: a running origin that stops at the slice's last tile; tables: the tile index, clamped to K - 64
+            int ko = sl.k00, tk = z * per * 64;
             for(int u = 0; u < sl.n_load + 8; u++)
             {
-                CHECK(ko >= 0 && ko <= K - 64, "%s origin %d out of range", c.name.c_str(), ko);
+                const int to = std::min(tk, sl.kmax);
+                CHECK(ko >= 0 && ko <= K - 64 && to >= 0 && to <= K - 64, "%s origin %d / %d out of range", c.name.c_str(), ko, to);
                 if(u < sl.nt)
-                    CHECK(ko == (z * per + u) * 64, "%s whole tile %d origin %d", c.name.c_str(), u, ko);
+                    CHECK(ko == (z * per + u) * 64 && to == ko, "%s whole tile %d origin %d / %d", c.name.c_str(), u, ko, to);
                 else if(sl.tail)
-                    CHECK(ko == K - 64, "%s tail tile origin %d", c.name.c_str(), ko);
+                    CHECK(ko == K - 64 && (u > sl.nt || to == K - 64), "%s tail tile origin %d / %d", c.name.c_str(), ko, to);
                 else
                     CHECK(ko == (z * per + sl.nt - 1) * 64, "%s tile %d beyond the slice at %d", c.name.c_str(), u, ko);
-                origins.push_back(ko);
+                origins.push_back(affine ? ko : to);
                 ko = hk_next_origin(ko, sl.klast);
+                tk += 64;
             }
         }
         for(int k = 0; k < K; k++)
@@ -361,18 +406,18 @@ static long check_hk_tile(const Case& c, const GemmView& v)
         for(int tp : {0, tiles_p / 2, tiles_p - 1})
             for(int tq : {0, tiles_q / 2, tiles_q - 1})
             {
-                const int p_own = tp * 256, q_own = tq * 256;
+                const int p_own = tp * 256, q_own = tq * BQ;
                 const int p0 = (v.shift_p && p_own + 256 > v.P) ? (int)v.P - 256 : p_own;
-                const int q0 = (v.shift_q && q_own + 256 > v.Q) ? (int)v.Q - 256 : q_own;
+                const int q0 = (v.shift_q && q_own + BQ > v.Q) ? (int)v.Q - BQ : q_own;
                 if(v.x_kfast)
-                    check_hk_operand<true, 256>("X", c, v, true, p0, origins);
+                    check_hk_operand<true, 256>("X", c, v, true, p0, origins, affine);
                 else
-                    check_hk_operand<false, 256>("X", c, v, true, p0, origins);
+                    check_hk_operand<false, 256>("X", c, v, true, p0, origins, affine);
                 if(v.y_kfast)
-                    check_hk_operand<true, 256>("Y", c, v, false, q0, origins);
+                    check_hk_operand<true, BQ>("Y", c, v, false, q0, origins, affine);
                 else
-                    check_hk_operand<false, 256>("Y", c, v, false, q0, origins);
-                walked += (long)origins.size() * 512 * 8;
+                    check_hk_operand<false, BQ>("Y", c, v, false, q0, origins, affine);
+                walked += (long)origins.size() * (256 + BQ) * 8;
             }
         if(want > 1 && split == 1)
             break;
@@ -596,7 +641,7 @@ int main()
         }
     }
     long walked = 0;
-    int  offered = 0, offered_hk = 0;
+    int  offered = 0, offered_hk = 0, offered_ring = 0, offered_ring_chunked = 0;
     for(const Case& c : cases)
     {
         ProblemIn in;
@@ -613,14 +658,15 @@ int main()
         CHECK(st == PlanStatus::OK, "%s: %s", c.name.c_str(), why.c_str());
         if(st != PlanStatus::OK)
             continue;
-        // is a direct-load tile offered for it?  (tile ids 9: 256 x 256, 10: 256 x 192; 11: 256 x 256 in K tiles of 64
-        // on 16 x 16 x 32 MFMAs)
-        for(int tile : {9, 10, 11})
+        // is a direct-load tile offered for it?  (tile ids 9: 256 x 256, 10: 256 x 192; on 16 x 16 x 32 MFMAs: 11: 256 x 256 in
+        // K tiles of 64, one k stride per operand; 12: 256 x 192 in K tiles of 32 through a ring of four stages, k offsets from tables)
+        for(int tile : {9, 10, 11, 12})
         {
             hiptk_problem_t p{};
             p.cls = v.cls, p.tile_id = tile, p.x_kfast = v.x_kfast, p.y_kfast = v.y_kfast, p.x_vec = v.x_vec, p.y_vec = v.y_vec;
             p.k_affine = v.k_affine, p.P = v.P, p.Q = v.Q, p.K = v.K, p.shift_p = v.shift_p, p.shift_q = v.shift_q;
             p.xy_aligned = v.xy_aligned, p.x_max_off = (int32_t)v.x_max_off, p.y_max_off = (int32_t)v.y_max_off;
+            p.x_rows_adjacent = v.x_rows_adjacent, p.y_rows_adjacent = v.y_rows_adjacent;
             const bool avail = hiptk_kernel_available(&p) != 0;
             std::printf("%-22s P %5lld Q %5lld K %5lld xkf %d ykf %d vec %d/%d kaff %d shift %d/%d aligned %d tile %2d: %s\n", c.name.c_str(),
                         (long long)v.P, (long long)v.Q, (long long)v.K, v.x_kfast, v.y_kfast, v.x_vec, v.y_vec, v.k_affine, v.shift_p, v.shift_q,
@@ -632,7 +678,14 @@ int main()
             {
                 CHECK(v.k_affine && v.K >= 64, "%s offered the K-tile-of-64 kernel outside its restrictions", c.name.c_str());
                 offered_hk++;
-                walked += check_hk_tile(c, v);
+                walked += check_hk_tile<256>(c, v, true);
+                continue;
+            }
+            if(tile == 12)
+            {
+                offered_ring++;
+                offered_ring_chunked += (v.x_kfast && v.x_rows_adjacent) || (v.y_kfast && v.y_rows_adjacent);
+                walked += check_tile_size<192>(c, v, true);
                 continue;
             }
             offered++;
@@ -640,7 +693,10 @@ int main()
         }
     }
     CHECK(offered >= 40, "only %d (case, tile) pairs were offered a direct-load kernel", offered);
-    CHECK(offered_hk >= 20, "only %d cases were offered the kernel with K tiles of 64", offered_hk);
+    CHECK(offered_hk >= 15, "only %d cases were offered the kernel with K tiles of 64", offered_hk);
+    CHECK(offered_ring >= 20, "only %d cases were offered the ring kernel", offered_ring);
+    CHECK(offered_ring_chunked >= 3, "only %d cases of the ring kernel stage an operand chunk-major", offered_ring_chunked);
+    std::printf("offered: %d (K tiles of 32), %d (K tiles of 64), %d (ring; %d chunk-major)\n", offered, offered_hk, offered_ring, offered_ring_chunked);
 
     // ---- 32/64-bit classes ----
     // benchmark configurations 1 (256^3), 3 (1920^2 x 768), 4 (1024^2 x 512) and a tensor of 2^32 bytes and more

@@ -111,6 +111,17 @@ def layouts(dtype, compute, big):
         if dtype == "f16":
             out.append(wl.config5(extents=(32, 2, 8, 24, 2, 16, 5, 8, 10)))
             out.append(wl.config5(extents=(32, 2, 8, 24, 2, 16, 4, 8, 10)))
+        if dtype in ("f16", "bf16"):
+            # k-contiguous operands in runs of one vector whose next row follows in memory (staged chunk-major by the
+            # kernel that loads K tiles of 32 into a ring): both operands, and one of them with the other's rows far apart
+            e6 = {0: 32, 1: 2, 2: 8, 10: 24, 11: 2, 12: 16, 20: 5, 21: 8, 22: 10}
+            mA, mB, mD = [0, 1, 2, 20, 21, 22], [10, 11, 12, 20, 21, 22], [0, 1, 2, 10, 11, 12]
+            for tag, oA, oB in (("both", [21, 0, 20, 2, 1, 22], [21, 12, 20, 10, 22, 11]),
+                                ("one", [21, 0, 20, 2, 1, 22], [21, 10, 12, 20, 22, 11])):
+                out.append(wl.make_workload(dtype, compute, mA, mB, mD, e6, a, b,
+                                            strideA=wl.storage_order_strides(mA, e6, oA),
+                                            strideB=wl.storage_order_strides(mB, e6, oB),
+                                            name=f"tiles_krun8_{tag}_{dtype}"))
     if not big and compute == cases.COMPUTE[dtype]:
         # The 32/64-bit kernels that load their operand tiles straight into LDS (operands in 16-byte vectors,
         # one K stride, K tiles of 8 or 16; a ring of 4 tiles):
@@ -191,7 +202,7 @@ def _tile_exists(cls, tile):
     class TileInfo(ctypes.Structure):
         _fields_ = [("tile_id", ctypes.c_int32), ("bp", ctypes.c_int32), ("bq", ctypes.c_int32),
                     ("bk", ctypes.c_int32), ("threads", ctypes.c_int32), ("lds_bytes", ctypes.c_int32),
-                    ("name", ctypes.c_char * 64), ("k_multiple", ctypes.c_int32)]
+                    ("name", ctypes.c_char * 64), ("k_multiple", ctypes.c_int32), ("mfma_k", ctypes.c_int32)]
 
     ti = TileInfo()
     return lib.hiptk_tile_info(cls, tile, ctypes.byref(ti)) == 0

@@ -139,6 +139,45 @@ def test_16x16x32_direct_load_loops_hold_no_wait_states(tmp_path, unit):
             assert len(ops) - 256 < 3 * 256 // 2, f"{symbol}: {len(ops) - 256} instructions beside 256 MFMAs"
 
 
+@pytest.mark.parametrize("unit", ["contract_f16_hr192_kx", "contract_f16_hr192_rx", "contract_bf16_hr192_kx", "contract_bf16_hr192_rx"])
+def test_ring_kernel_loops(tmp_path, unit):
+    """The 16-bit kernel on v_mfma_f32_16x16x32 that loads K tiles of 32 into a ring of four stages and reads its k
+    offsets from tables.  Its loads are issued without wait states too; its loop does hold vector ALU instructions
+    (they turn table entries into load offsets), so the check is that none of them writes a scalar register.  Every
+    barrier of the loop must directly follow the wait for the loads of the tile after next AND for the wave's own LDS
+    reads (the stage those reads came from is overwritten after the barrier)."""
+    lines = device_asm(unit, tmp_path)
+    symbols = [l.split(":")[0] for l in lines if re.match(r"^_ZN5hiptk18contract_hr_kernel.*EvNS_5KArgsE:", l)]
+    assert len(symbols) == 2, symbols
+    for symbol in symbols:
+        body = kernel_body(lines, symbol)
+        # four K tiles of 48 MFMAs: the period of the ring, the table slots and the offset sets
+        loops = [(a, b) for a, b in main_loops(body, 192) if len(opcodes(body, a, b)) < 1024]
+        assert len(loops) == 4, f"{symbol}: {len(loops)} main loops (one per wave position expected)"
+        for a, b in loops:
+            ops = opcodes(body, a, b)
+            assert sum(o.startswith("v_mfma_f32_16x16x32") for o in ops) == 192, symbol
+            valu = sorted({o for o in ops if o.startswith("v_") and not o.startswith("v_mfma")})
+            assert valu and all(o.startswith(("v_min_u32", "v_add_lshl_u32", "v_lshl_add_u32", "v_add_u32", "v_lshlrev_b32")) for o in valu), \
+                f"vector ALU instructions in the main loop of {symbol}: {valu}"
+            assert not any(o.startswith(("s_cbranch", "s_branch", "scratch_", "buffer_store", "global_store")) for o in ops), symbol
+            # (the compiler puts one s_nop 0 per K tile in front of the table request's first write of M0)
+            assert sum(o == "s_nop" for o in ops) <= 4, f"{symbol}: s_nop in the main loop"
+            # seven loads of 16 bytes a lane and two of table entries per K tile, each with its own write of M0
+            assert sum(o == "global_load_lds_dwordx4" for o in ops) == 28 and sum(o == "global_load_lds_dword" for o in ops) == 8, symbol
+            text = [l for l in body[a:b] if "m0" in l.split(";")[0]]
+            assert len(text) == 36 and all(l.strip().startswith("s_add_u32 m0,") for l in text), text[:5]
+            code = [l.split(";")[0].strip() for l in body[a:b]]
+            code = [l for l in code if l and not l.endswith(":") and not l.startswith(".")]
+            bars = [i for i, l in enumerate(code) if l.startswith("s_barrier")]
+            assert len(bars) == 4, symbol
+            for i in bars:
+                assert code[i - 1].startswith("s_waitcnt") and "vmcnt(20)" in code[i - 1] and "lgkmcnt(0)" in code[i - 1], \
+                    f"{symbol}: '{code[i - 1]}' in front of a barrier of the main loop"
+            # instructions beside the MFMAs: fewer than two per MFMA (a 16-cycle MFMA leaves the wave three issue slots)
+            assert len(ops) - 192 < 2 * 192, f"{symbol}: {len(ops) - 192} instructions beside 192 MFMAs"
+
+
 def test_direct_load_loops_leave_m0_alone(tmp_path):
     """The 32 x 32 x 16 direct-load kernel writes M0 one MFMA ahead of the load that reads it, in separate asm
     statements: nothing the compiler generates in between may touch M0."""
