@@ -45,6 +45,14 @@ MEASURED_TRAFFIC_KIB = {
     ("cfg2_f16_bilinear_4096", "TraitsF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (116540.0, 34591.0),
     ("cfg2_bf16_scale_4096", "TraitsBF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (98747.0, 32768.0),
     ("cfg2_bf16_bilinear_4096", "TraitsBF16_256x256x32_xfalse8_yfalse8_kafftrue_direct2x2"): (115910.0, 32770.0),
+    # profiles/contract_hk_kernel_4096cubed.md
+    ("cfg2_f16_scale_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue_direct2x2_m16x16x32"): (98748.1, 32768.1),
+    ("cfg2_f16_bilinear_4096", "TraitsF16_256x256x64_xfalse8_yfalse8_kafftrue_direct2x2_m16x16x32"): (115179.0, 32795.3),
+    ("cfg2_bf16_bilinear_4096", "TraitsBF16_256x256x64_xfalse8_yfalse8_kafftrue_direct2x2_m16x16x32"): (115209.0, 32786.7),
+    ("rowmajor_f16_bilinear_4096", "TraitsF16_256x256x64_xtrue8_ytrue8_kafftrue_direct2x2_m16x16x32"): (115171.0, 32794.3),
+    ("rowmajor_bf16_bilinear_4096", "TraitsBF16_256x256x64_xtrue8_ytrue8_kafftrue_direct2x2_m16x16x32"): (115184.0, 32779.5),
+    # profiles/contract_hr_kernel_rank6.md
+    ("cfg5_f16_bilinear_rank6_permuted", "TraitsF16_256x192x32_xfalse8_ytrue8_kafffalse_direct2x2_ring4_m16x16x32"): (325825.0, 103383.0),
     # profiles/contract_kernels_configs_1_3_4_5_counters.md (split-K: contraction kernel + reduction kernel)
     ("cfg1_f32_bilinear_256", "WTraitsF32_64x64x16_00"): (823.0 + 1187.5, 2048.0 + 256.0),
     ("cfg1_f32_bilinear_256", "WTraitsF32_32x32x16_direct4k4"): (979.0, 256.0),

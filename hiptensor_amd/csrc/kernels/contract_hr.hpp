@@ -109,9 +109,10 @@ namespace hiptk
         // loads a wavefront issues per step: two of table entries, then the tile's; and how many may be
         // outstanding when tile t + 1 must have landed: those of the two steps after the one that requested it
         constexpr int PER_STEP = NL + 2, NWAIT = 2 + (NS - 2) * PER_STEP;
-        // MFMA slots of a step: the table request's two loads (each with its M0 write one MFMA earlier)
-        constexpr int TRQ_X = NM - 5, TRQ_Y = NM - 3;
-        static_assert(hk_load_slot(3, NL - 1, SPM) + 1 < TRQ_X - 1 && 2 * NL + 8 <= NM, "a tile's loads and table work fit under its MFMAs");
+        // MFMA slots of a step: the table request's two loads (each with its M0 write one MFMA earlier), the first offset
+        constexpr int TRQ_X = NM - 5, TRQ_Y = NM - 3, TF0 = NM - 13;
+        static_assert(hk_load_slot(3, NL - 1, SPM) + 1 < TRQ_X - 1 && TF0 > 4 * (NBP - 1) + 1 && TF0 > 6 * (NBQ - 1) + 2 && TF0 + NL <= NM,
+                      "a tile's loads and table work fit under its MFMAs, the offsets behind the last operand read");
         static_assert(NS == 4, "stage, table slot and offset set indices share the period 4");
 
         extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
@@ -261,11 +262,13 @@ namespace hiptk
             __builtin_amdgcn_sched_barrier(0);
             hk_static_for<NM>([&](auto m_c) __attribute__((always_inline)) {
                 constexpr int m = decltype(m_c)::value;
-                // table work: one entry out of LDS in front of each of the first NL MFMAs; eight MFMAs later, one offset each
+                // table work: one entry out of LDS in front of each of the first NL MFMAs; one offset each from MFMA TF0 on, behind
+                // the step's last operand read (LDS reads return in order: the entries have long arrived; formed eight MFMAs
+                // behind their reads, the wait in front of each cost 37 cycles a step)
                 if constexpr(m < NL)
                     t_read(std::integral_constant<int, (T + 1) & 3>{}, m_c); // (tile t + 5: slot (t + 5) % 4)
-                if constexpr(m >= NL + 8 && m < 2 * NL + 8)
-                    t_form(std::integral_constant<int, (m >= NL + 8 && m < 2 * NL + 8) ? m - NL - 8 : 0>{}, std::integral_constant<int, (T + 1) & 1>{});
+                if constexpr(m >= TF0 && m < TF0 + NL)
+                    t_form(std::integral_constant<int, (m >= TF0 && m < TF0 + NL) ? m - TF0 : 0>{}, std::integral_constant<int, (T + 1) & 1>{});
                 // operand fetches of tile t + 1: all issued in the first three quarters of the step, so that the barrier
                 // of the next step does not wait for them
                 if constexpr(m % 4 == 1 && m / 4 < NBP)
