@@ -402,6 +402,8 @@ namespace hipta
 
         // ---- gather direction and vector width per operand ----
         const int maxv = class_max_vec(v.cls);
+        // f32 (4 elements in 16 bytes): the register-staged kernels also gather both operands in pairs
+        const bool half_vectors = v.cls == HIPTK_F32;
         auto pick = [&](bool use_x, const std::vector<Dim>& rows, int& kfast, int& vec, bool& ragged) {
             int  vk = 1, vr = 1;
             bool rr = false;
@@ -411,9 +413,9 @@ namespace hipta
                 vk = vector_width(v.kdims[0].len, v.kdims.size() == 1, maxv, &kr, 2 * maxv);
             if(!rows.empty() && (use_x ? rows[0].sx : rows[0].sy) == 1)
                 vr = vector_width(rows[0].len, rows.size() == 1, maxv, &rr);
-            // the wide classes are instantiated for full-width vectors and for scalars; the
-            // 16-bit classes also for 8- and 4-byte vectors (narrowed jointly below)
-            if(maxv != 8)
+            // the wide classes are instantiated for full-width vectors and for scalars; f32 also for
+            // 8-byte vectors and the 16-bit classes for 8- and 4-byte vectors (narrowed jointly below)
+            if(maxv != 8 && !half_vectors)
             {
                 if(vk < maxv)
                     vk = 1;
@@ -453,6 +455,28 @@ namespace hipta
                     xRagged   = false;
                 }
                 if(v.y_vec < 8)
+                {
+                    v.y_vec   = 1;
+                    v.y_kfast = 1;
+                    yRagged   = false;
+                }
+            }
+        }
+        if(half_vectors && !(v.x_vec == maxv && v.y_vec == maxv) && !(v.x_vec == 1 && v.y_vec == 1))
+        {
+            // f32 kernels exist for (4,4), (4,1), (1,4), (1,1) and (2,2) elements per vector of (X, Y)
+            if(v.x_vec >= 2 && v.y_vec >= 2)
+                v.x_vec = v.y_vec = 2;
+            else
+            {
+                // scalar gathers are staged k-fast
+                if(v.x_vec < maxv)
+                {
+                    v.x_vec   = 1;
+                    v.x_kfast = 1;
+                    xRagged   = false;
+                }
+                if(v.y_vec < maxv)
                 {
                     v.y_vec   = 1;
                     v.y_kfast = 1;

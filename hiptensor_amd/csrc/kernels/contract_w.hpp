@@ -29,9 +29,11 @@ namespace hiptk
 
     enum
     {
-        GATHER_MN_VEC = 0, // vectors of VMAX along the row index
-        GATHER_K_VEC  = 1, // vectors of VMAX along k
-        GATHER_SCALAR = 2
+        GATHER_MN_VEC  = 0, // vectors of VMAX along the row index
+        GATHER_K_VEC   = 1, // vectors of VMAX along k
+        GATHER_SCALAR  = 2,
+        GATHER_MN_HALF = 3, // vectors of VMAX / 2 along the row index (8 bytes of f32: runs that are a multiple of 2, not of 4)
+        GATHER_K_HALF  = 4 // ... along k
     };
 
     // ---- per-class traits -------------------------------------------------------
@@ -279,16 +281,18 @@ namespace hiptk
     {
         typedef typename Tr::E E;
         typedef typename Tr::S S;
-        static constexpr int   V     = MODE == GATHER_SCALAR ? 1 : Tr::VMAX;
+        static constexpr bool  MN    = MODE == GATHER_MN_VEC || MODE == GATHER_MN_HALF; // vectors along the row index
+        static constexpr bool  KV    = MODE == GATHER_K_VEC || MODE == GATHER_K_HALF; // vectors along k
+        static constexpr int   V     = MODE == GATHER_SCALAR ? 1 : (MODE == GATHER_MN_HALF || MODE == GATHER_K_HALF) ? Tr::VMAX / 2 : Tr::VMAX;
         static constexpr int   N     = BR * BK / NT; // elements per thread
         static constexpr int   NV    = N / V; // vectors per thread
         static constexpr int   PAD   = (sizeof(S) >= 8 ? 2 : 4);
         static constexpr int   PITCH = BR + PAD;
         static constexpr int   ELEMS = BK * PITCH;
         // threads along the fast direction of the mapping, and rows / k's covered per pass
-        static constexpr int PER  = MODE == GATHER_MN_VEC ? BR / V : (MODE == GATHER_K_VEC ? BK / V : BK);
+        static constexpr int PER  = MN ? BR / V : (KV ? BK / V : BK);
         static constexpr int STEP = NT / PER;
-        static_assert(BR * BK % NT == 0 && N % V == 0 && NV >= 1, "tile must split evenly over threads");
+        static_assert(BR * BK % NT == 0 && N % V == 0 && NV >= 1 && V >= 1, "tile must split evenly over threads");
         static_assert(NT % PER == 0, "thread mapping");
 
         struct alignas(sizeof(E) * V) PackE
@@ -301,15 +305,15 @@ namespace hiptk
         };
 
         PackE   data[NV];
-        int32_t roff[MODE == GATHER_MN_VEC ? 1 : NV]; // row-table offsets (loop invariant)
-        int32_t koff[MODE == GATHER_MN_VEC ? NV : 1]; // k-table offsets of the tile being fetched
+        int32_t roff[MN ? 1 : NV]; // row-table offsets (loop invariant)
+        int32_t koff[MN ? NV : 1]; // k-table offsets of the tile being fetched
         int     a, b;
 
         __device__ inline void init(const int32_t* rtab, int r0, int tid)
         {
             a = tid % PER;
             b = tid / PER;
-            if constexpr(MODE == GATHER_MN_VEC)
+            if constexpr(MN)
                 roff[0] = rtab[r0 + a * V];
             else
             {
@@ -321,7 +325,7 @@ namespace hiptk
 
         __device__ inline void load_koffs(const int32_t* ktab, int k0)
         {
-            if constexpr(MODE == GATHER_MN_VEC)
+            if constexpr(MN)
             {
 #pragma unroll
                 for(int i = 0; i < NV; i++)
@@ -338,13 +342,13 @@ namespace hiptk
 #pragma unroll
             for(int i = 0; i < NV; i++)
             {
-                const int  k  = MODE == GATHER_MN_VEC ? k0 + b + i * STEP : k0 + a * V;
+                const int  k  = MN ? k0 + b + i * STEP : k0 + a * V;
                 const bool ok = !TAIL || k < K;
                 // A k-fast vector that straddles K (K is then one contiguous run, not a multiple
                 // of the vector) is loaded V elements back from the end of the run, inside the
                 // tensor, and moved down in registers; that also clears the slots from K on.
-                const bool partial = MODE == GATHER_K_VEC && TAIL && V > 1 && k < K && k + V > K;
-                const uint32_t off = MODE == GATHER_MN_VEC ? (uint32_t)roff[0] + (uint32_t)koff[i]
+                const bool partial = KV && TAIL && V > 1 && k < K && k + V > K;
+                const uint32_t off = MN ? (uint32_t)roff[0] + (uint32_t)koff[i]
                                                             : (uint32_t)roff[i] + (uint32_t)koff[0] - (partial ? (uint32_t)(k + V - K) : 0u);
                 PackE v = *(const PackE*)(bp + off);
                 if(TAIL && !ok)
@@ -353,7 +357,7 @@ namespace hiptk
                     for(int j = 0; j < V; j++)
                         v.e[j] = E{};
                 }
-                if constexpr(MODE == GATHER_K_VEC && TAIL && V > 1)
+                if constexpr(KV && TAIL && V > 1)
                 {
                     const int r = K % V; // uniform; 0 when no vector straddles K
                     if(r != 0)
@@ -391,7 +395,7 @@ namespace hiptk
 #pragma unroll
             for(int i = 0; i < NV; i++)
             {
-                if constexpr(MODE == GATHER_MN_VEC)
+                if constexpr(MN)
                 {
                     PackS s;
 #pragma unroll
@@ -711,9 +715,10 @@ namespace hiptk
 // gather mode <-> (kfast, vec) as the registry describes it
 #define HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, XM, YM)                                      \
     {                                                                                          \
-        hiptk::TR::CLS, ID, (XM != hiptk::GATHER_MN_VEC), (YM != hiptk::GATHER_MN_VEC),        \
-            (XM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX),                                \
-            (YM == hiptk::GATHER_SCALAR ? 1 : hiptk::TR::VMAX), 0, BP, BQ, BK, WP *WQ * 64,      \
+        hiptk::TR::CLS, ID, (XM != hiptk::GATHER_MN_VEC && XM != hiptk::GATHER_MN_HALF),       \
+            (YM != hiptk::GATHER_MN_VEC && YM != hiptk::GATHER_MN_HALF),                       \
+            (XM == hiptk::GATHER_SCALAR ? 1 : XM >= hiptk::GATHER_MN_HALF ? hiptk::TR::VMAX / 2 : hiptk::TR::VMAX), \
+            (YM == hiptk::GATHER_SCALAR ? 1 : YM >= hiptk::GATHER_MN_HALF ? hiptk::TR::VMAX / 2 : hiptk::TR::VMAX), 0, BP, BQ, BK, WP *WQ * 64, \
             hiptk::lds_bytes_w<hiptk::TR, BP, BQ, BK>(), #TR "_" #BP "x" #BQ "x" #BK "_" #XM #YM, \
             &hiptk::launch_w<hiptk::TR, BP, BQ, BK, WP, WQ, XM, YM>                            \
     }
@@ -727,3 +732,7 @@ namespace hiptk
         HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 2, 0),                                       \
         HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 2, 1),                                       \
         HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 2, 2)
+// ... with both operands in vectors of VMAX / 2
+#define HIPTK_W_TILE_HALF(TR, ID, BP, BQ, BK, WP, WQ)                                          \
+    HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 3, 3), HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 3, 4), \
+        HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 4, 3), HIPTK_W_ENTRY(TR, ID, BP, BQ, BK, WP, WQ, 4, 4)

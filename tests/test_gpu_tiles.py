@@ -51,6 +51,19 @@ def layouts(dtype, compute, big):
                                         name=f"tiles_{tag}_kfast_{dtype}"))
             out.append(wl.make_workload(dtype, compute, [0, 1, 20, 21], [20, 21, 10, 11], [10, 11, 0, 1], ev, a, b,
                                         name=f"tiles_{tag}_mixed_{dtype}"))
+    if dtype == "f32" and compute == cases.COMPUTE[dtype]:
+        # f32 runs that are a multiple of 2 elements but not of 4: both operands in 8-byte vectors (row-fast,
+        # k-fast and mixed; K = 90 ends inside a K tile and inside no vector)
+        # (row and k modes interleaved in memory, so that no run is longer than its leading mode)
+        ev = {0: 10, 1: 9, 10: 10, 11: 13, 20: 10, 21: 9}
+        out.append(wl.make_workload(dtype, compute, [0, 20, 1, 21], [10, 20, 11, 21], [0, 10, 1, 11], ev, a, b,
+                                    name=f"tiles_v2_rowfast_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [20, 0, 21, 1], [20, 10, 21, 11], [10, 0, 11, 1], ev, a, None,
+                                    name=f"tiles_v2_kfast_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [0, 20, 1, 21], [20, 10, 21, 11], [10, 0, 11, 1], ev, a, b,
+                                    name=f"tiles_v2_mixed_{dtype}"))
+        out.append(wl.make_workload(dtype, compute, [20, 0, 21, 1], [10, 20, 11, 21], [0, 10, 1, 11], ev, a, None,
+                                    name=f"tiles_v2_mixed2_{dtype}"))
     # odd extents of 256 and more, each index one contiguous run: vectors stay, tiles that would
     # overhang are moved back (2 row tiles of 256, 3 of 128, 5 of 64; columns likewise)
     rg = {0: 15, 1: 19, 10: 17, 11: 21, 20: 16, 21: 9 if big else 5}
@@ -188,6 +201,8 @@ def test_every_tile_of_the_class(gpu_handle, oracle_mod, dtype, compute):
                     assert info["split_k"] == split
                     cases.assert_parity(w, cases.logical_view(w, got), exp, info["kernel_name"])
                     covered.setdefault(tile, set()).add(info["kernel_name"])
+                    if dtype == "f32" and w["name"].startswith("tiles_v2_"):
+                        assert (info["x_vec"], info["y_vec"]) == (2, 2), (w["name"], info["kernel_name"], info["x_vec"], info["y_vec"])
     finally:
         os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
     # every tile id that has a kernel at all must have run on at least one layout

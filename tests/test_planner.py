@@ -121,9 +121,18 @@ def test_vector_width_follows_runs_not_alignment(host_handle):
     w = wl.make_workload("f16", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
     info, _ = plan(host_handle, w)
     assert (info["x_vec"], info["y_vec"], info["x_kfast"], info["y_kfast"]) == (1, 1, 1, 1)
-    # the wide classes have full-width or scalar kernels only
+    # f32 kernels exist for (4,4), (4,1), (1,4), (1,1) and (2,2): a run of 30 elements beside one of 80 narrows both to 8 bytes
     ext = {0: 6, 1: 5, 10: 8, 11: 10, 20: 16, 21: 5}
     w = wl.make_workload("f32", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"]) == (2, 2)
+    ext[0] = 5  # ... an odd run is a scalar gather, and the other operand keeps 16 bytes
+    w = wl.make_workload("f32", api.HIPTENSOR_COMPUTE_32F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
+    info, _ = plan(host_handle, w)
+    assert (info["x_vec"], info["y_vec"]) == (4, 1)
+    # the other wide classes have full-width or scalar kernels only (f32 tensors contracted in 16-bit arithmetic: 4 or 1)
+    ext[0] = 6
+    w = wl.make_workload("f32", api.HIPTENSOR_COMPUTE_16F, [0, 1, 20, 21], [10, 11, 20, 21], [0, 1, 10, 11], ext, 1.0, None)
     info, _ = plan(host_handle, w)
     assert (info["x_vec"], info["y_vec"]) == (4, 1)
     # an odd row pitch (leading dimension padded by one element) does not narrow anything either
