@@ -183,7 +183,7 @@ namespace hiptk
         // loads a wavefront may have outstanding when tile t + 1 must have landed: those of a ring of
         // three that were issued behind it
         constexpr int NWAIT = (NSX == 3 ? NXL : 0) + (NSY == 3 ? NYL : 0);
-        static_assert(hk_load_slot(3, NL - 1, SPM) < KST * NM, "a tile's loads are issued within a tile");
+        static_assert(hk_load_slot(3, NL - 1, SPM) < NM, "a tile's loads are issued within the k-step behind the barrier");
 
         extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
 
@@ -302,13 +302,19 @@ namespace hiptk
         // NKS of the stages nx / ny) into the other set, X block i in front of MFMA NBQ i and Y block j in
         // front of MFMA NBP j + NBP / 2; and this wave's loads of the window slots G0 .. G0 + NM - 1.
         // sched_barrier(0) after every MFMA keeps the issue order as written.
-        auto kstep = [&](auto wv_c, auto ks_c, const uint16_t* nx, const uint16_t* ny, auto nks_c, auto g0_c) __attribute__((always_inline)) {
+        auto kstep = [&](auto wv_c, auto ks_c, const uint16_t* nx, const uint16_t* ny, auto nks_c, auto g0_c, auto sx_c, auto sy_c) __attribute__((always_inline)) {
             constexpr int KS   = decltype(ks_c)::value;
             constexpr int NKS  = decltype(nks_c)::value;
             constexpr int G0   = decltype(g0_c)::value;
             constexpr int slot = KS & 1;
             hk_static_for<NM>([&](auto m_c) __attribute__((always_inline)) {
                 constexpr int m = decltype(m_c)::value;
+                // k-step 0: where the next window's tiles lie and go (scalar arithmetic under the MFMAs instead of behind
+                // the barrier, where nothing covers it; this wave's loads of the window before have all been issued)
+                if constexpr(KS == 0 && m == 2)
+                    x_open(sx_c);
+                if constexpr(KS == 0 && m == 6)
+                    y_open(sy_c);
                 if constexpr(m % NBQ == 0)
                     xf[slot ^ 1][m / NBQ] = fx.load(nx, m / NBQ, NKS);
                 if constexpr(m % NBP == NBP / 2)
@@ -335,16 +341,14 @@ namespace hiptk
             const uint16_t* nx = lds + ((SX + 1) % NSX) * G::OPX;
             const uint16_t* ny = lds + G::YRING + ((SY + 1) % NSY) * G::OPY;
             // k-step 0 fetches k-step 1 (the window that opened in the last k-step of the tile before goes on)
-            kstep(wv_c, I0{}, cx, cy, I1{}, std::integral_constant<int, NM>{});
+            kstep(wv_c, I0{}, cx, cy, I1{}, std::integral_constant<int, NM>{}, sx_c, sy_c);
             // Every wave has issued its reads of tile t.  Tile t + 1 must have landed.
             __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(NWAIT));
             lds_barrier();
             __builtin_amdgcn_sched_barrier(0);
             // the stages of tile t are free: the window of tiles t + NSY (Y) and t + NSX (X) opens
-            x_open(sx_c);
-            y_open(sy_c);
             // k-step 1 fetches k-step 0 of tile t + 1 (beyond the last tile: stale data, not used)
-            kstep(wv_c, I1{}, nx, ny, I0{}, I0{});
+            kstep(wv_c, I1{}, nx, ny, I0{}, I0{}, sx_c, sy_c);
         };
 
         auto main_loop = [&](auto wv_c) __attribute__((always_inline)) {
