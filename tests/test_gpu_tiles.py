@@ -276,3 +276,86 @@ def test_direct_load_tiles_on_random_layouts(gpu_handle, oracle_mod, dtype):
         os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
     print("ran:", sorted(ran), flush=True)
     assert len({r[0] for r in ran}) == 3 and len({(r[1], r[2]) for r in ran}) >= (1 if dtype == "c64" else 3), sorted(ran)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_16bit_direct_load_tiles_on_random_storage_orders(gpu_handle, oracle_mod, dtype):
+    """The 16-bit kernels that load operand tiles straight into LDS (tile ids 9 - 12), on seeded random problems of
+    two or three modes per group whose tensors are stored in random mode orders: the fastest mode of A and of B is a
+    free mode or a contracted one (row- or k-contiguous operand), of extent 8 or a multiple (16-byte vectors); the
+    modes behind it come in any order, so the contracted modes fuse into one stride or do not (k offsets from
+    tables), and the vector after a k-contiguous one is the next row's or not (chunk-major staging or not); K is a
+    multiple of 16 that ends inside a K tile or not; D is packed in a random order; scale and bilinear.  Every problem
+    runs the default selection and each of the four tile ids, the table-driven one also with split-K 2, against
+    the oracle; a tile that is not offered for a problem is skipped, and every tile id must have run on both
+    kinds of first operand."""
+    rng = np.random.default_rng({"f16": 21, "bf16": 22}[dtype])
+    ran, chunked = set(), 0
+    try:
+        for n in range(16):
+            nm, nn, nk = (int(rng.integers(2, 4)) for _ in range(3))
+            ext = {}
+            for base, cnt, lead in ((0, nm, [16, 32, 64]), (10, nn, [16, 32, 64]), (20, nk, [8, 16])):
+                for i in range(cnt):
+                    ext[base + i] = int(rng.choice(lead)) if i == 0 else int(rng.choice([2, 3, 4, 5]))
+            ms, ns, ks = ([b + i for i in range(c)] for b, c in ((0, nm), (10, nn), (20, nk)))
+            K = int(np.prod([ext[k] for k in ks]))
+            if K % 16 != 0:
+                ext[ks[-1]] *= 2
+            mA, mB, mD = ms + ks, ns + ks, ms + ns
+            fused = n % 2 == 0  # the contracted modes stay together, in one order, in A and in B: one k stride per operand
+
+            def order(free, first_k):
+                if fused:
+                    rest = list(free[1:])
+                    rng.shuffle(rest)
+                    if first_k:
+                        return ks + [free[0]] + rest
+                    pos = int(rng.integers(0, len(rest) + 1))
+                    return [free[0]] + rest[:pos] + ks + rest[pos:]
+                rest = [m for m in free[1:]] + [k for k in ks[1:]]
+                rng.shuffle(rest)
+                lead, other = (ks[0], free[0]) if first_k else (free[0], ks[0])
+                # where the other group's leading mode goes (0: right behind the fastest; every fourth problem has it there)
+                pos = 0 if n % 4 == 1 else int(rng.integers(0, len(rest) + 1))
+                return [lead] + rest[:pos] + [other] + rest[pos:]
+
+            a_kfast, b_kfast = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+            oA, oB = order(ms, a_kfast), order(ns, b_kfast)
+            # (the planner folds the free modes in D's order: an operand's fastest free mode must be the first of its
+            # group in D too, or its rows have no runs)
+            oD = list(mD)
+            rng.shuffle(oD)
+            for grp in (ms, ns):
+                at = sorted(oD.index(m) for m in grp)
+                rest = [m for m in oD if m in grp and m != grp[0]]
+                for pos, m in zip(at, [grp[0]] + rest):
+                    oD[pos] = m
+            alpha, beta = float(rng.uniform(-2, 2)), (None if n % 3 == 0 else float(rng.uniform(-2, 2)))
+            sD = wl.storage_order_strides(mD, ext, oD)
+            w = wl.make_workload(dtype, cases.COMPUTE[dtype], mA, mB, mD, ext, alpha, beta,
+                                 strideA=wl.storage_order_strides(mA, ext, oA), strideB=wl.storage_order_strides(mB, ext, oB),
+                                 strideC=sD, strideD=sD, name=f"random16_{dtype}_{n}_{'k' if a_kfast else 'r'}{'k' if b_kfast else 'r'}")
+            chunked += (a_kfast and oA[1] == ms[0]) or (b_kfast and oB[1] == ns[0])
+            inp = wl.host_inputs(w)
+            exp = cases.logical_view(w, oracle_mod.contract(w, inp["A"], inp["B"], inp["C"]))
+            for force in (None, "9,1", "10,1", "11,1", "12,1", "12,2"):
+                if force:
+                    os.environ["HIPTENSOR_AMD_FORCE_KERNEL"] = force
+                else:
+                    os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
+                print(f"[case] {w['name']} ext={ext} oA={oA} oB={oB} oD={oD} force={force}", flush=True)
+                try:
+                    got, info = gpu_util.run_gpu(gpu_handle, w, inp, pref=api.HIPTENSOR_WORKSPACE_MAX, return_info=True)
+                except api.HiptensorError as e:
+                    assert force and e.status == api.HIPTENSOR_STATUS_EXECUTION_FAILED, e
+                    continue
+                cases.assert_parity(w, cases.logical_view(w, got), exp, info["kernel_name"])
+                if force and "direct" in info["kernel_name"]:
+                    ran.add((force.split(",")[0], info["x_kfast"], info["y_kfast"]))
+    finally:
+        os.environ.pop("HIPTENSOR_AMD_FORCE_KERNEL", None)
+    print("ran:", sorted(ran), "problems with a k-contiguous operand whose next vector is the next row's:", chunked, flush=True)
+    for tile in ("9", "10", "11", "12"):
+        assert {r[1] for r in ran if r[0] == tile} == {0, 1}, (tile, sorted(ran))
+    assert chunked >= 2
