@@ -106,8 +106,9 @@ namespace hiptk
         constexpr int TP = 4, TQ = BQ / 64, WP = 2, WQ = 2; // 32 x 32 blocks of a wave tile (what the epilogue walks)
         constexpr int NBP = 2 * TP, NBQ = 2 * TQ, NM = NBP * NBQ; // MFMA blocks, MFMAs per K tile
         constexpr int SPM = NM / NL >= 6 ? 6 : NM / NL; // MFMAs between two loads of a wave
-        // loads a wavefront issues per step: two of table entries, then the tile's; and how many may be
-        // outstanding when tile t + 1 must have landed: those of the two steps after the one that requested it
+        // loads a wavefront issues per step: the tile's, then two of table entries; and how many may be
+        // outstanding when tile t + 1 must have landed: the table entries requested right behind it and the loads
+        // of the two steps after that
         constexpr int PER_STEP = NL + 2, NWAIT = 2 + (NS - 2) * PER_STEP;
         // MFMA slots of a step: the table request's two loads (each with its M0 write one MFMA earlier), the first offset
         constexpr int TRQ_X = NM - 5, TRQ_Y = NM - 3, TF0 = NM - 13;
@@ -296,9 +297,9 @@ namespace hiptk
         };
 
         auto main_loop = [&](auto wv_c) __attribute__((always_inline)) {
-            // Prologue.  The table entries of tiles 0 .. 8 and the loads of tiles 0 .. 3, each after its offsets, in
-            // the order the loop would have issued them in (the entries of tile u + 5 right after the loads of tile u):
-            // the loop's wait counts the loads issued after those of the tile it needs.
+            // Prologue.  The table entries of tiles 0 .. 8 and the loads of tiles 0 .. 3, each after its offsets, issued so
+            // that as many loads follow those of tiles 2 and 3 as follow those of every later tile (20: the loop's wait
+            // counts the loads issued after those of the tile it needs; tiles 0 and 1 are waited for here).
             t_request(I0{});
             t_request(I1{});
             t_request(I2{});
