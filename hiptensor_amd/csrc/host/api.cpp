@@ -828,6 +828,8 @@ hiptensorStatus_t hiptensorInitContractionPlan(const hiptensorHandle_t*         
         p.dq_stride = (int32_t)v.dq_stride;
         p.cp_stride = (int32_t)v.cp_stride;
         p.cq_stride = (int32_t)v.cq_stride;
+        p.xp_stride = (int32_t)v.xp_stride;
+        p.yq_stride = (int32_t)v.yq_stride;
         p.shift_p   = v.shift_p;
         p.shift_q   = v.shift_q;
         p.xy_aligned = v.xy_aligned;

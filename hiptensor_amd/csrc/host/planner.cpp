@@ -395,9 +395,13 @@ namespace hipta
             v.cp_stride = v.pdims.empty() ? 0 : v.pdims[0].sc;
             v.dq_stride = v.qdims.empty() ? 0 : v.qdims[0].sd;
             v.cq_stride = v.qdims.empty() ? 0 : v.qdims[0].sc;
+            v.xp_stride = v.pdims.empty() ? 0 : v.pdims[0].sx;
+            v.yq_stride = v.qdims.empty() ? 0 : v.qdims[0].sy;
             for(int64_t st : {v.dp_stride, v.dq_stride, v.cp_stride, v.cq_stride})
                 if(st > 0x7FFFFFFFll)
                     v.cd_affine = 0;
+            if(v.xp_stride > 0x7FFFFFFFll || v.yq_stride > 0x7FFFFFFFll || !v.cd_affine)
+                v.xp_stride = v.yq_stride = 0;
         }
 
         // ---- gather direction and vector width per operand ----

@@ -67,6 +67,7 @@ namespace hipta
         // every 16-byte vector of X and Y starts a multiple of 16 bytes from its tensor's base
         int xy_aligned = 0;
         // largest element offset of X / Y that the tables address
+        int64_t xp_stride = 0, yq_stride = 0; // with cd_affine: element stride of the one row mode of X / column mode of Y
         int64_t x_max_off = 0, y_max_off = 0;
         // k-contiguous operand: the vectors of consecutive rows are neighbours in memory more often than consecutive
         // vectors of one row (a hint for the kernels' LDS layout)

@@ -215,13 +215,19 @@ namespace hiptk
         for(int i = 0; i < NXL; i++)
         {
             const HdSlot s = hk_stage_slot<XKF, BP>((wave * NXL + i) * 64 + lane);
-            xvoff[i]       = 2u * ((uint32_t)a.xp[p0 + s.row] + (uint32_t)s.k * (uint32_t)a.xk_stride);
+            // (one row mode: the offset is computed, which spares the prologue a round trip to the table; rows beyond P
+            // read row 0, as the table has them)
+            const int      pr  = p0 + s.row;
+            const uint32_t row = a.xp_stride ? (pr < a.P ? (uint32_t)pr * (uint32_t)a.xp_stride : 0u) : (uint32_t)a.xp[pr];
+            xvoff[i]           = 2u * (row + (uint32_t)s.k * (uint32_t)a.xk_stride);
         }
 #pragma unroll
         for(int i = 0; i < NYL; i++)
         {
             const HdSlot s = hk_stage_slot<YKF, BQ>((wave * NYL + i) * 64 + lane);
-            yvoff[i]       = 2u * ((uint32_t)a.yq[q0 + s.row] + (uint32_t)s.k * (uint32_t)a.yk_stride);
+            const int      qr  = q0 + s.row;
+            const uint32_t row = a.yq_stride ? (qr < a.Q ? (uint32_t)qr * (uint32_t)a.yq_stride : 0u) : (uint32_t)a.yq[qr];
+            yvoff[i]           = 2u * (row + (uint32_t)s.k * (uint32_t)a.yk_stride);
         }
         HkFrag<XKF, BP> fx;
         HkFrag<YKF, BQ> fy;

@@ -24,6 +24,7 @@ namespace hiptk
         int32_t xk_stride, yk_stride; // element stride of k when the K modes fused into one
         int32_t cd_affine; // 1: C / D offsets are p * stride + q * stride, no table lookups
         int32_t dp_stride, dq_stride, cp_stride, cq_stride;
+        int32_t xp_stride, yq_stride; // with cd_affine: xp[p] = p * xp_stride, yq[q] = q * yq_stride (0: look them up)
         int32_t cd_vec; // contiguous elements along q shared by C and D
         // 1: a tile that would overhang P (Q) is moved back so that it ends at P (Q); it still
         // stores only the rows (columns) of its own range.  Lets vectors run along a contiguous

@@ -373,6 +373,8 @@ extern "C" int hiptk_contract(const hiptk_problem_t* prob,
     a.dq_stride = prob->dq_stride;
     a.cp_stride = prob->cp_stride;
     a.cq_stride = prob->cq_stride;
+    a.xp_stride = prob->cd_affine ? prob->xp_stride : 0;
+    a.yq_stride = prob->cd_affine ? prob->yq_stride : 0;
     a.xk_stride = prob->xk_stride;
     a.yk_stride = prob->yk_stride;
     a.cd_vec    = prob->cd_vec;

@@ -93,6 +93,9 @@ typedef struct hiptk_problem
                           for a bilinear problem) for all p < P, q < Q: the epilogue then computes
                           offsets instead of reading the tables (which must still be valid)      */
     int32_t dp_stride, dq_stride, cp_stride, cq_stride;
+    int32_t xp_stride, yq_stride; /* with cd_affine = 1 also: xp[p] == p * xp_stride and yq[q] == q * yq_stride for p < P,
+                                     q < Q (the rows of X and the columns of Y are one mode each): kernels may then
+                                     compute their operands' row offsets as well (0: look them up)               */
     int32_t shift_p; /* 1: the rows are one contiguous run of P elements in every tensor that is read
                         or written in vectors along them, P need not be a multiple of the vector: a
                         tile that would overhang P is moved back to end at P (it recomputes some of

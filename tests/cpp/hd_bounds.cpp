@@ -641,7 +641,7 @@ int main()
         }
     }
     long walked = 0;
-    int  offered = 0, offered_hk = 0, offered_ring = 0, offered_ring_chunked = 0;
+    int  offered = 0, offered_hk = 0, offered_ring = 0, offered_ring_chunked = 0, computed_rows = 0;
     for(const Case& c : cases)
     {
         ProblemIn in;
@@ -676,6 +676,14 @@ int main()
             CHECK(v.x_vec == 8 && v.y_vec == 8 && v.K % 16 == 0 && v.K >= 32 && v.xy_aligned, "%s offered outside its restrictions", c.name.c_str());
             if(tile == 11)
             {
+                // this kernel computes its operands' row offsets where the planner says the rows are one mode each
+                if(v.cd_affine && v.xp_stride)
+                    for(int64_t r = 0; r < v.P; r++)
+                        CHECK(v.xp[(size_t)r] == r * v.xp_stride, "%s xp[%lld] is not %lld x the row stride", c.name.c_str(), (long long)r, (long long)r);
+                if(v.cd_affine && v.yq_stride)
+                    for(int64_t r = 0; r < v.Q; r++)
+                        CHECK(v.yq[(size_t)r] == r * v.yq_stride, "%s yq[%lld] is not %lld x the column stride", c.name.c_str(), (long long)r, (long long)r);
+                computed_rows += v.cd_affine && v.xp_stride && v.yq_stride;
                 CHECK(v.k_affine && v.K >= 64, "%s offered the K-tile-of-64 kernel outside its restrictions", c.name.c_str());
                 offered_hk++;
                 walked += check_hk_tile<256>(c, v, true);
@@ -694,6 +702,7 @@ int main()
     }
     CHECK(offered >= 40, "only %d (case, tile) pairs were offered a direct-load kernel", offered);
     CHECK(offered_hk >= 15, "only %d cases were offered the kernel with K tiles of 64", offered_hk);
+    CHECK(computed_rows >= 10, "only %d cases of the K-tile-of-64 kernel have computed row offsets", computed_rows);
     CHECK(offered_ring >= 20, "only %d cases were offered the ring kernel", offered_ring);
     CHECK(offered_ring_chunked >= 3, "only %d cases of the ring kernel stage an operand chunk-major", offered_ring_chunked);
     std::printf("offered: %d (K tiles of 32), %d (K tiles of 64), %d (ring; %d chunk-major)\n", offered, offered_hk, offered_ring, offered_ring_chunked);
