@@ -100,6 +100,21 @@ static TensorIn tensor(const Case& c, const std::vector<int32_t>& modes, std::ve
     return t;
 }
 
+// The kernels compute their operands' row offsets where the planner says the rows of X and the columns of Y are one mode
+// each: what they compute must be what the tables hold.
+static int check_computed_rows(const Case& c, const GemmView& v)
+{
+    if(!v.cd_affine)
+        return 0;
+    if(v.xp_stride)
+        for(int64_t r = 0; r < v.P; r++)
+            CHECK(v.xp[(size_t)r] == r * v.xp_stride, "%s xp[%lld] is not %lld x the row stride", c.name.c_str(), (long long)r, (long long)r);
+    if(v.yq_stride)
+        for(int64_t r = 0; r < v.Q; r++)
+            CHECK(v.yq[(size_t)r] == r * v.yq_stride, "%s yq[%lld] is not %lld x the column stride", c.name.c_str(), (long long)r, (long long)r);
+    return v.xp_stride && v.yq_stride;
+}
+
 template <bool KF, int BR>
 static void check_operand(const char* what, const Case& c, const GemmView& v, bool is_x, int r0, const std::vector<int>& origins,
                           bool affine, bool ring = false) // ring: the kernel on 16 x 16 x 32 MFMAs (contract_hr.hpp), table form only
@@ -676,14 +691,7 @@ int main()
             CHECK(v.x_vec == 8 && v.y_vec == 8 && v.K % 16 == 0 && v.K >= 32 && v.xy_aligned, "%s offered outside its restrictions", c.name.c_str());
             if(tile == 11)
             {
-                // this kernel computes its operands' row offsets where the planner says the rows are one mode each
-                if(v.cd_affine && v.xp_stride)
-                    for(int64_t r = 0; r < v.P; r++)
-                        CHECK(v.xp[(size_t)r] == r * v.xp_stride, "%s xp[%lld] is not %lld x the row stride", c.name.c_str(), (long long)r, (long long)r);
-                if(v.cd_affine && v.yq_stride)
-                    for(int64_t r = 0; r < v.Q; r++)
-                        CHECK(v.yq[(size_t)r] == r * v.yq_stride, "%s yq[%lld] is not %lld x the column stride", c.name.c_str(), (long long)r, (long long)r);
-                computed_rows += v.cd_affine && v.xp_stride && v.yq_stride;
+                computed_rows += check_computed_rows(c, v);
                 CHECK(v.k_affine && v.K >= 64, "%s offered the K-tile-of-64 kernel outside its restrictions", c.name.c_str());
                 offered_hk++;
                 walked += check_hk_tile<256>(c, v, true);
