@@ -219,7 +219,8 @@ namespace hiptk
             // read row 0, as the table has them)
             const int      pr  = p0 + s.row;
             const uint32_t row = a.xp_stride ? (pr < a.P ? (uint32_t)pr * (uint32_t)a.xp_stride : 0u) : (uint32_t)a.xp[pr];
-            xvoff[i]           = 2u * (row + (uint32_t)s.k * (uint32_t)a.xk_stride);
+            // (four loads share a write of M0: dma_lds.hpp)
+            xvoff[i]           = 2u * (row + (uint32_t)s.k * (uint32_t)a.xk_stride) + (uint32_t)(DMA_BIAS - (i % 4) * 1024);
         }
 #pragma unroll
         for(int i = 0; i < NYL; i++)
@@ -227,7 +228,7 @@ namespace hiptk
             const HdSlot s = hk_stage_slot<YKF, BQ>((wave * NYL + i) * 64 + lane);
             const int      qr  = q0 + s.row;
             const uint32_t row = a.yq_stride ? (qr < a.Q ? (uint32_t)qr * (uint32_t)a.yq_stride : 0u) : (uint32_t)a.yq[qr];
-            yvoff[i]           = 2u * (row + (uint32_t)s.k * (uint32_t)a.yk_stride);
+            yvoff[i]           = 2u * (row + (uint32_t)s.k * (uint32_t)a.yk_stride) + (uint32_t)(DMA_BIAS - (i % 4) * 1024);
         }
         HkFrag<XKF, BP> fx;
         HkFrag<YKF, BQ> fy;
@@ -243,13 +244,13 @@ namespace hiptk
         uint32_t       xdst = 0, ydst = 0;
         auto x_open = [&](auto s_c) __attribute__((always_inline)) {
             constexpr int S = decltype(s_c)::value;
-            xsrc            = (const char*)a.X + (uint64_t)((uint32_t)xko * xkb);
+            xsrc            = (const char*)a.X + (uint64_t)((uint32_t)xko * xkb) - DMA_BIAS;
             xdst            = wdstx + S * (G::OPX * 2);
             xko             = hk_next_origin(xko, klast);
         };
         auto y_open = [&](auto s_c) __attribute__((always_inline)) {
             constexpr int S = decltype(s_c)::value;
-            ysrc            = (const char*)a.Y + (uint64_t)((uint32_t)yko * ykb);
+            ysrc            = (const char*)a.Y + (uint64_t)((uint32_t)yko * ykb) - DMA_BIAS;
             ydst            = wdsty + S * (G::OPY * 2);
             yko             = hk_next_origin(yko, klast);
         };
@@ -258,16 +259,18 @@ namespace hiptk
             constexpr int  j   = decltype(j_c)::value;
             constexpr bool isy = YFIRST ? j < NYL : j >= NXL;
             constexpr int  i   = YFIRST ? (j < NYL ? j : j - NYL) : (j < NXL ? j : j - NXL);
-            dma_dst<i * 1024>(isy ? ydst : xdst);
+            // (the first of four loads into consecutive KiB writes M0 for all of them)
+            if constexpr(i % 4 == 0)
+                dma_dst<i * 1024>(isy ? ydst : xdst);
         };
         auto load = [&](auto j_c, auto bare_c) __attribute__((always_inline)) {
             constexpr int  j   = decltype(j_c)::value;
             constexpr bool isy = YFIRST ? j < NYL : j >= NXL;
             constexpr int  i   = YFIRST ? (j < NYL ? j : j - NYL) : (j < NXL ? j : j - NXL);
             if constexpr(decltype(bare_c)::value)
-                dma_load_in_loop(isy ? yvoff[i] : xvoff[i], isy ? ysrc : xsrc);
+                dma_load_in_loop_off<(i % 4) * 1024>(isy ? yvoff[i] : xvoff[i], isy ? ysrc : xsrc);
             else
-                dma_load(isy ? yvoff[i] : xvoff[i], isy ? ysrc : xsrc);
+                dma_load_off<(i % 4) * 1024>(isy ? yvoff[i] : xvoff[i], isy ? ysrc : xsrc);
         };
         // what wave WV does about its loads in front of the MFMA of window slot g: M0 for a load
         // that follows the next MFMA, and the load whose turn it is
@@ -370,8 +373,9 @@ namespace hiptk
                         y_open(std::integral_constant<int, (ty >= 0 ? ty : 0)>{});
                         hk_static_for<NYL>([&](auto i_c) __attribute__((always_inline)) {
                             constexpr int i = decltype(i_c)::value;
-                            dma_dst<i * 1024>(ydst);
-                            dma_load(yvoff[i], ysrc);
+                            if constexpr(i % 4 == 0)
+                                dma_dst<i * 1024>(ydst);
+                            dma_load_off<(i % 4) * 1024>(yvoff[i], ysrc);
                         });
                     }
                 };
@@ -381,8 +385,9 @@ namespace hiptk
                         x_open(std::integral_constant<int, (tx >= 0 ? tx : 0)>{});
                         hk_static_for<NXL>([&](auto i_c) __attribute__((always_inline)) {
                             constexpr int i = decltype(i_c)::value;
-                            dma_dst<i * 1024>(xdst);
-                            dma_load(xvoff[i], xsrc);
+                            if constexpr(i % 4 == 0)
+                                dma_dst<i * 1024>(xdst);
+                            dma_load_off<(i % 4) * 1024>(xvoff[i], xsrc);
                         });
                     }
                 };

@@ -52,6 +52,24 @@ namespace hiptk
     {
         asm volatile("global_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(hd_scalar(base)) : "memory");
     }
+    // The instruction's offset field moves the global address AND the LDS destination (found by a probe on the device: with
+    // offset:1024 lane l's 16 bytes came from base + voff + 1024 and landed at M0 + 1024 + 16 l).  So up to four loads into
+    // consecutive KiB of LDS share one write of M0 (the field is 13 bits, signed), when each lane's offset is lowered by the
+    // same amount beforehand: the callers keep voff + DMA_BIAS - OFF in their registers and base - DMA_BIAS in the scalars, so
+    // that no lane offset goes below zero.
+    constexpr int DMA_BIAS = 3072;
+    template <int OFF>
+    __device__ __forceinline__ void dma_load_off(uint32_t voff, const void* base)
+    {
+        static_assert(OFF >= 0 && OFF <= DMA_BIAS && OFF % 1024 == 0, "one of four consecutive KiB");
+        asm volatile("s_nop 4\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(hd_scalar(base)), "n"(OFF) : "memory");
+    }
+    template <int OFF>
+    __device__ __forceinline__ void dma_load_in_loop_off(uint32_t voff, const void* base)
+    {
+        static_assert(OFF >= 0 && OFF <= DMA_BIAS && OFF % 1024 == 0, "one of four consecutive KiB");
+        asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" : : "v"(voff), "s"(hd_scalar(base)), "n"(OFF) : "memory");
+    }
     // ... with a full address per lane (no scalar base): for loads some lanes of which must look elsewhere
     __device__ __forceinline__ void dma_load_at(const void* lane_address)
     {

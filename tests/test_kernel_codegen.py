@@ -133,9 +133,12 @@ def test_16x16x32_direct_load_loops_hold_no_wait_states(tmp_path, unit):
             # compiler adds an s_nop 0 of its own in front of the next write of M0)
             assert sum(o == "s_nop" for o in ops) <= 4, f"{symbol}: s_nop in the main loop"
             assert sum(o == "global_load_lds_dwordx4" for o in ops) == 32, symbol
-            # M0 is written by the load helpers' s_add_u32 only, once per load, in front of the MFMA before it
+            # M0 is written by the load helpers' s_add_u32 only, once per four loads (which reach consecutive KiB of LDS
+            # through their offset fields), in front of the MFMA before the first of them
             text = [l for l in body[a:b] if "m0" in l.split(";")[0]]
-            assert len(text) == 32 and all(l.strip().startswith("s_add_u32 m0,") for l in text), text[:5]
+            assert len(text) == 8 and all(l.strip().startswith("s_add_u32 m0,") for l in text), text[:5]
+            offs = sorted({int(m.group(1), 0) for l in body[a:b] for m in [re.search(r"global_load_lds_dwordx4 .*offset:(0x[0-9a-f]+|\d+)", l)] if m})
+            assert offs == [0, 1024, 2048, 3072], offs
             # instructions beside the MFMAs: fewer than three per MFMA on average
             assert len(ops) - 256 < 3 * 256 // 2, f"{symbol}: {len(ops) - 256} instructions beside 256 MFMAs"
 
