@@ -12,7 +12,9 @@ namespace hiptk
     //   dma_dst:  M0 <- LDS byte address lds_base + off (wave-uniform)
     //   dma_load: 16 bytes per lane from global memory (base + 32-bit byte offset voff) to LDS address
     //             M0 + 16 * lane (dma_load1: 4 bytes per lane to M0 + 4 * lane).  Counted by vmcnt.
-    // Nothing else in these kernels uses M0.
+    // Nothing else in these kernels uses M0.  M0 cannot be named in a clobber list (the compiler treats it as a reserved
+    // register and warns that clobbering it is undefined), so that nothing the compiler generates between the two halves
+    // touches M0 is checked in the device assembly instead (tests/test_kernel_codegen.py).
     // The compiler's hazard recognizer does not look inside inline assembly, so the wait states an
     // instruction needs are provided here: a VMEM instruction must not read an SGPR within 5 wait
     // states of a VALU instruction writing it (the compiler reloads spilled SGPRs with v_readlane,
