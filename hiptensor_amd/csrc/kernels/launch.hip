@@ -7,6 +7,7 @@
 
 #include "contract_h.hpp"
 #include "contract_w.hpp"
+#include "dma_lds.hpp"
 
 namespace hiptk
 {
@@ -205,7 +206,8 @@ namespace hiptk
                     {
                         const uint64_t eb   = (uint64_t)operand_bytes(p->cls);
                         const int32_t  most = p->x_max_off > p->y_max_off ? p->x_max_off : p->y_max_off;
-                        if(most < 0 || ((uint64_t)most + 16 / eb) * eb > 0xFFFFFFFFull)
+                        // (less the bias some of them keep in a lane's offset so that loads can share a write of M0)
+                        if(most < 0 || ((uint64_t)most + 16 / eb) * eb > 0xFFFFFFFFull - (uint64_t)DMA_BIAS)
                             continue;
                     }
                     if(e.k_affine && p->k_affine)

@@ -214,3 +214,35 @@ def test_workspace_preferences(host_handle):
         assert rec.info["workspace_bytes"] == rec.info["split_k"] * 256 * 256 * 4
     rec.close()
     mx.close()
+
+
+def test_direct_load_kernels_keep_32_bit_offsets_in_range(host_handle, monkeypatch):
+    """The kernels that load straight into LDS address an operand with 32-bit byte offsets, and some keep a bias of up
+    to 3 KiB in a lane's offset (loads that share one write of M0): an operand whose last vector ends within that of
+    4 GiB is not offered to them, one that ends a few KiB earlier is.  (A: 512 rows contiguous, 128 k at a stride that
+    puts the last vector where the case wants it.)"""
+    ext = {0: 512, 10: 512, 20: 128}
+    top = (2 ** 31 - 512 - 8) // 127 // 8 * 8  # largest k stride, a multiple of 8 elements, whose last vector ends below 4 GiB
+
+    def kernel(stride, force):
+        if force:
+            monkeypatch.setenv("HIPTENSOR_AMD_FORCE_KERNEL", force)
+        else:
+            monkeypatch.delenv("HIPTENSOR_AMD_FORCE_KERNEL", raising=False)
+        w = wl.make_workload("f16", cases.COMPUTE["f16"], [0, 20], [10, 20], [0, 10], ext, 1.0, None, strideA=[1, stride],
+                             name=f"a_ends_near_4GiB_{stride}")
+        try:
+            info, _ = plan(host_handle, w)
+        except api.HiptensorError as e:
+            assert e.status == api.HIPTENSOR_STATUS_EXECUTION_FAILED, e
+            return None
+        return info["kernel_name"]
+
+    for stride, offered in ((top, False), (top - 8, False), (top - 16, True)):
+        room = 2 ** 32 - (2 * (511 + 127 * stride) + 16)
+        assert (room > 3072) == offered, (stride, room)
+        for force in ("9,1", "10,1", "11,1", "12,1"):
+            name = kernel(stride, force)
+            assert (name is not None and "direct" in name) == offered, (stride, force, name)
+        name = kernel(stride, None)
+        assert name is not None and (offered or "direct" not in name), (stride, name)
