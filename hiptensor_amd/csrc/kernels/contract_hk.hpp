@@ -242,17 +242,29 @@ namespace hiptk
         int            xko = sl.k00, yko = sl.k00;
         const char *   xsrc = nullptr, *ysrc = nullptr;
         uint32_t       xdst = 0, ydst = 0;
-        auto x_open = [&](auto s_c) __attribute__((always_inline)) {
+        // (in two halves of three scalar instructions each, so that neither fills more than the three issue slots beside
+        // an MFMA of the loop)
+        const char* const xbase = (const char*)a.X - DMA_BIAS;
+        const char* const ybase = (const char*)a.Y - DMA_BIAS;
+        auto x_open_src = [&]() __attribute__((always_inline)) { xsrc = xbase + (uint64_t)((uint32_t)xko * xkb); };
+        auto x_open_dst = [&](auto s_c) __attribute__((always_inline)) {
             constexpr int S = decltype(s_c)::value;
-            xsrc            = (const char*)a.X + (uint64_t)((uint32_t)xko * xkb) - DMA_BIAS;
             xdst            = wdstx + S * (G::OPX * 2);
             xko             = hk_next_origin(xko, klast);
         };
-        auto y_open = [&](auto s_c) __attribute__((always_inline)) {
+        auto y_open_src = [&]() __attribute__((always_inline)) { ysrc = ybase + (uint64_t)((uint32_t)yko * ykb); };
+        auto y_open_dst = [&](auto s_c) __attribute__((always_inline)) {
             constexpr int S = decltype(s_c)::value;
-            ysrc            = (const char*)a.Y + (uint64_t)((uint32_t)yko * ykb) - DMA_BIAS;
             ydst            = wdsty + S * (G::OPY * 2);
             yko             = hk_next_origin(yko, klast);
+        };
+        auto x_open = [&](auto s_c) __attribute__((always_inline)) {
+            x_open_src();
+            x_open_dst(s_c);
+        };
+        auto y_open = [&](auto s_c) __attribute__((always_inline)) {
+            y_open_src();
+            y_open_dst(s_c);
         };
         // load j of a tile's window: the first NYL (NXL) are Y's (X's) when Y (X) goes first
         auto set_m0 = [&](auto j_c) __attribute__((always_inline)) {
@@ -284,11 +296,11 @@ namespace hiptk
                     set_m0(j_c);
                 if constexpr(ls == g)
                 {
-                    // (first slot of a window: no earlier MFMA in it to separate the write of M0 from the load,
-                    // so this one keeps its wait states)
-                    if constexpr(g == 0)
+                    // (first slot of a window: inside the loop M0 is written in front of the last MFMA of the k-step
+                    // before, see kstep; the prologue writes it here and keeps the load's wait states)
+                    if constexpr(g == 0 && !decltype(bare_c)::value)
                         set_m0(j_c);
-                    load(j_c, std::integral_constant<bool, (g != 0) && decltype(bare_c)::value>{});
+                    load(j_c, bare_c);
                 }
             });
         };
@@ -321,14 +333,25 @@ namespace hiptk
                 // k-step 0: where the next window's tiles lie and go (scalar arithmetic under the MFMAs instead of behind
                 // the barrier, where nothing covers it; this wave's loads of the window before have all been issued)
                 if constexpr(KS == 0 && m == 2)
-                    x_open(sx_c);
+                    x_open_src();
+                if constexpr(KS == 0 && m == 3)
+                    x_open_dst(sx_c);
                 if constexpr(KS == 0 && m == 6)
-                    y_open(sy_c);
+                    y_open_src();
+                if constexpr(KS == 0 && m == 7)
+                    y_open_dst(sy_c);
                 if constexpr(m % NBQ == 0)
                     xf[slot ^ 1][m / NBQ] = fx.load(nx, m / NBQ, NKS);
                 if constexpr(m % NBP == NBP / 2)
                     yf[slot ^ 1][m / NBP] = fy.load(ny, m / NBP, NKS);
                 window_slot(wv_c, std::integral_constant<int, G0 + m>{}, std::true_type{});
+                // M0 for the load in the first slot of the window that opens behind this k-step's barrier (an s_nop between
+                // the two there would hold up the MFMAs of the wave that every other wave then waits for at the next barrier)
+                if constexpr(KS == 0 && m == NM - 1)
+                    hk_static_for<NL>([&](auto j_c) __attribute__((always_inline)) {
+                        if constexpr(hk_load_slot(decltype(wv_c)::value, decltype(j_c)::value, SPM) == 0)
+                            set_m0(j_c);
+                    });
                 {
                     constexpr int bi = hk_block_i(m, NBQ), bj = hk_block_j(m, NBQ);
                     hk_mfma16_acc(Tr{}, acc[bi][bj], xf[slot][bi], yf[slot][bj]);

@@ -141,6 +141,20 @@ def test_16x16x32_direct_load_loops_hold_no_wait_states(tmp_path, unit):
             assert offs == [0, 1024, 2048, 3072], offs
             # instructions beside the MFMAs: fewer than three per MFMA on average
             assert len(ops) - 256 < 3 * 256 // 2, f"{symbol}: {len(ops) - 256} instructions beside 256 MFMAs"
+            # ... and no more than three between two MFMAs (a fourth delays the MFMA behind it): the scalar arithmetic that
+            # opens a tile's window of loads is spread over four MFMAs, and M0 for the load right behind a barrier is written
+            # in front of the barrier, for that.  (The first MFMA of the period may have four in front of it, and the two
+            # behind a barrier, which wait anyway, five, the wait and the barrier included.)
+            gaps, run = [], []
+            for o in ops:
+                if o.startswith("v_mfma"):
+                    gaps.append(run)
+                    run = []
+                else:
+                    run.append(o)
+            plain = [len(g) for g in gaps if "s_barrier" not in g]
+            assert max(plain) <= 4 and sum(n == 4 for n in plain) <= 1, (symbol, [g for g in gaps if len(g) > 3])
+            assert all(len(g) <= 5 for g in gaps), (symbol, [g for g in gaps if len(g) > 5])
 
 
 @pytest.mark.parametrize("unit", ["contract_f16_hr192_kx", "contract_f16_hr192_rx", "contract_bf16_hr192_kx", "contract_bf16_hr192_rx"])
