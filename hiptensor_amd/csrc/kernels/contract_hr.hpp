@@ -98,6 +98,21 @@ namespace hiptk
         }
     };
 
+    // The MFMA of a step in front of which the j-th table entry is read from LDS: from the fourth on, leaving out those that
+    // hold an operand fetch (X's at m % 4 == 1, Y's at m % 6 == 2), so that with a direct load and a write of M0 no MFMA has
+    // more than three instructions in front of it.
+    constexpr int hr_table_read_slot(int j)
+    {
+        int m = 2;
+        for(int n = -1; n < j;)
+        {
+            m++;
+            if(m % 4 != 1 && m % 6 != 2)
+                n++;
+        }
+        return m;
+    }
+
     template <typename Tr, bool XKF, bool YKF, int BQ>
     __global__ void __launch_bounds__(256, 1) contract_hr_kernel(const KArgs a)
     {
@@ -111,8 +126,9 @@ namespace hiptk
         // of the two steps after that
         constexpr int PER_STEP = NL + 2, NWAIT = 2 + (NS - 2) * PER_STEP;
         // MFMA slots of a step: the table request's two loads (each with its M0 write one MFMA earlier), the first offset
-        constexpr int TRQ_X = NM - 5, TRQ_Y = NM - 3, TF0 = NM - 13;
-        static_assert(hk_load_slot(3, NL - 1, SPM) + 1 < TRQ_X - 1 && TF0 > 4 * (NBP - 1) + 1 && TF0 > 6 * (NBQ - 1) + 2 && TF0 + NL <= NM,
+        constexpr int TRQ0 = NM - 6, TF0 = NM - 13;
+        static_assert(hk_load_slot(3, NL - 1, SPM) + 1 < TRQ0 && TF0 > 4 * (NBP - 1) + 1 && TF0 > 6 * (NBQ - 1) + 2 && TF0 + NL <= TRQ0
+                          && hr_table_read_slot(NL - 1) < TF0,
                       "a tile's loads and table work fit under its MFMAs, the offsets behind the last operand read");
         static_assert(NS == 4, "stage, table slot and offset set indices share the period 4");
 
@@ -173,8 +189,8 @@ namespace hiptk
         // tail tile again, one beyond the slice a tile of the next slice: harmless, its stage is free)
         int      tk = kt_begin * HD_BK;
         uint64_t tofs = 0;
-        // phase 0: the tile's (clamped) position in the tables and the destination of X's entries; 1: X's entries;
-        // 2: the destination of Y's; 3: Y's entries
+        // phase 0: the tile's (clamped) position in the tables; 1: the destination of X's entries; 2: X's entries; 3: the
+        // destination of Y's; 4: Y's entries (no phase holds more than the three instructions an MFMA leaves room for)
         auto t_request_part = [&](auto slot_c, auto phase_c, auto bare_c) __attribute__((always_inline)) {
             constexpr int S = decltype(slot_c)::value, PH = decltype(phase_c)::value;
             if constexpr(PH == 0)
@@ -182,13 +198,14 @@ namespace hiptk
                 const int kc = tk < kmax ? tk : kmax;
                 tofs         = 4ull * (uint64_t)(uint32_t)kc;
                 tk += HD_BK;
-                dma_dst<S * 512>(wtab);
             }
-            if constexpr(PH == 2)
+            if constexpr(PH == 1)
+                dma_dst<S * 512>(wtab);
+            if constexpr(PH == 3)
                 dma_dst<S * 512 + 256>(wtab);
-            if constexpr(PH == 1 || PH == 3)
+            if constexpr(PH == 2 || PH == 4)
             {
-                const char* src = (const char*)(PH == 1 ? (const void*)a.xk : (const void*)a.yk) + tofs;
+                const char* src = (const char*)(PH == 2 ? (const void*)a.xk : (const void*)a.yk) + tofs;
                 if constexpr(decltype(bare_c)::value)
                     dma_load1_bare(tlane, src);
                 else
@@ -196,7 +213,7 @@ namespace hiptk
             }
         };
         auto t_request = [&](auto slot_c) __attribute__((always_inline)) {
-            hk_static_for<4>([&](auto ph_c) __attribute__((always_inline)) { t_request_part(slot_c, ph_c, std::false_type{}); });
+            hk_static_for<5>([&](auto ph_c) __attribute__((always_inline)) { t_request_part(slot_c, ph_c, std::false_type{}); });
         };
         auto t_read = [&](auto slot_c, auto j_c) __attribute__((always_inline)) {
             constexpr int S = decltype(slot_c)::value, j = decltype(j_c)::value;
@@ -266,8 +283,10 @@ namespace hiptk
                 // table work: one entry out of LDS in front of each of the first NL MFMAs; one offset each from MFMA TF0 on, behind
                 // the step's last operand read (LDS reads return in order: the entries have long arrived; formed eight MFMAs
                 // behind their reads, the wait in front of each cost 37 cycles a step)
-                if constexpr(m < NL)
-                    t_read(std::integral_constant<int, (T + 1) & 3>{}, m_c); // (tile t + 5: slot (t + 5) % 4)
+                hk_static_for<NL>([&](auto j_c) __attribute__((always_inline)) {
+                    if constexpr(hr_table_read_slot(decltype(j_c)::value) == m)
+                        t_read(std::integral_constant<int, (T + 1) & 3>{}, j_c); // (tile t + 5: slot (t + 5) % 4)
+                });
                 if constexpr(m >= TF0 && m < TF0 + NL)
                     t_form(std::integral_constant<int, (m >= TF0 && m < TF0 + NL) ? m - TF0 : 0>{}, std::integral_constant<int, (T + 1) & 1>{});
                 // operand fetches of tile t + 1: all issued in the first three quarters of the step, so that the barrier
@@ -286,8 +305,8 @@ namespace hiptk
                         load(j_c, std::integral_constant<int, T & 1>{}, std::true_type{});
                 });
                 // the table entries of tile t + 9 (slot (t + 9) % 4: the entries read from it above have been used)
-                if constexpr(m >= TRQ_X - 1 && m <= TRQ_Y)
-                    t_request_part(std::integral_constant<int, (T + 1) & 3>{}, std::integral_constant<int, (m >= TRQ_X - 1 && m <= TRQ_Y) ? m - (TRQ_X - 1) : 0>{}, std::true_type{});
+                if constexpr(m >= TRQ0 && m < TRQ0 + 5)
+                    t_request_part(std::integral_constant<int, (T + 1) & 3>{}, std::integral_constant<int, (m >= TRQ0 && m < TRQ0 + 5) ? m - TRQ0 : 0>{}, std::true_type{});
                 {
                     constexpr int bi = hk_block_i(m, NBQ), bj = hk_block_j(m, NBQ);
                     hk_mfma16_acc(Tr{}, acc[bi][bj], xf[T & 1][bi], yf[T & 1][bj]);
