@@ -120,7 +120,7 @@ namespace hiptk
         constexpr int BP = G::BP, NS = G::NS, NXL = G::NXL, NYL = G::NYL, NL = NXL + NYL;
         constexpr int TP = 4, TQ = BQ / 64, WP = 2, WQ = 2; // 32 x 32 blocks of a wave tile (what the epilogue walks)
         constexpr int NBP = 2 * TP, NBQ = 2 * TQ, NM = NBP * NBQ; // MFMA blocks, MFMAs per K tile
-        constexpr int SPM = NM / NL >= 6 ? 6 : NM / NL; // MFMAs between two loads of a wave
+        constexpr int SPM = NM / NL >= 5 ? 5 : NM / NL; // MFMAs between two loads of a wave (the last one in front of the first offset)
         // loads a wavefront issues per step: the tile's, then two of table entries; and how many may be
         // outstanding when tile t + 1 must have landed: the table entries requested right behind it and the loads
         // of the two steps after that

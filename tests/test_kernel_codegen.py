@@ -194,6 +194,15 @@ def test_ring_kernel_loops(tmp_path, unit):
                     f"{symbol}: '{code[i - 1]}' in front of a barrier of the main loop"
             # instructions beside the MFMAs: fewer than two per MFMA (a 16-cycle MFMA leaves the wave three issue slots)
             assert len(ops) - 192 < 2 * 192, f"{symbol}: {len(ops) - 192} instructions beside 192 MFMAs"
+            # ... and never more than three in front of one MFMA (four where the period begins: the loop's own bookkeeping)
+            gaps, run = [], []
+            for o in ops:
+                if o.startswith("v_mfma"):
+                    gaps.append(run)
+                    run = []
+                else:
+                    run.append(o)
+            assert sum(len(g) > 3 for g in gaps) <= 1 and max(len(g) for g in gaps) <= 4, (symbol, [g for g in gaps if len(g) > 3])
 
 
 def test_direct_load_loops_leave_m0_alone(tmp_path):
