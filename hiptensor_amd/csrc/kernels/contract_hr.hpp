@@ -280,7 +280,7 @@ namespace hiptk
             __builtin_amdgcn_sched_barrier(0);
             hk_static_for<NM>([&](auto m_c) __attribute__((always_inline)) {
                 constexpr int m = decltype(m_c)::value;
-                // table work: one entry out of LDS in front of each of the first NL MFMAs; one offset each from MFMA TF0 on, behind
+                // table work: one entry out of LDS in front of each of NL early MFMAs (hr_table_read_slot); one offset each from MFMA TF0 on, behind
                 // the step's last operand read (LDS reads return in order: the entries have long arrived; formed eight MFMAs
                 // behind their reads, the wait in front of each cost 37 cycles a step)
                 hk_static_for<NL>([&](auto j_c) __attribute__((always_inline)) {
