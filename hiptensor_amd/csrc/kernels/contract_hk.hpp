@@ -184,6 +184,7 @@ namespace hiptk
         // three that were issued behind it
         constexpr int NWAIT = (NSX == 3 ? NXL : 0) + (NSY == 3 ? NYL : 0);
         static_assert(hk_load_slot(3, NL - 1, SPM) < NM, "a tile's loads are issued within the k-step behind the barrier");
+        static_assert(6 * (NBP - 1) < NM && 6 * (NBQ - 1) + 3 < NM, "the operand fetches of a k-step fit under its MFMAs");
 
         extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
 
@@ -320,8 +321,8 @@ namespace hiptk
         u32x4_t xf[2][NBP], yf[2][NBQ];
 
         // One k-step: NM MFMAs out of register set KS % 2; the operand fetches of the next k-step (k-step
-        // NKS of the stages nx / ny) into the other set, X block i in front of MFMA NBQ i and Y block j in
-        // front of MFMA NBP j + NBP / 2; and this wave's loads of the window slots G0 .. G0 + NM - 1.
+        // NKS of the stages nx / ny) into the other set, X block i in front of MFMA 6 i and Y block j in
+        // front of MFMA 6 j + 3; and this wave's loads of the window slots G0 .. G0 + NM - 1.
         // sched_barrier(0) after every MFMA keeps the issue order as written.
         auto kstep = [&](auto wv_c, auto ks_c, const uint16_t* nx, const uint16_t* ny, auto nks_c, auto g0_c, auto sx_c, auto sy_c) __attribute__((always_inline)) {
             constexpr int KS   = decltype(ks_c)::value;
@@ -332,18 +333,20 @@ namespace hiptk
                 constexpr int m = decltype(m_c)::value;
                 // k-step 0: where the next window's tiles lie and go (scalar arithmetic under the MFMAs instead of behind
                 // the barrier, where nothing covers it; this wave's loads of the window before have all been issued)
-                if constexpr(KS == 0 && m == 2)
+                if constexpr(KS == 0 && m == 10)
                     x_open_src();
-                if constexpr(KS == 0 && m == 3)
+                if constexpr(KS == 0 && m == 11)
                     x_open_dst(sx_c);
-                if constexpr(KS == 0 && m == 6)
+                if constexpr(KS == 0 && m == 14)
                     y_open_src();
-                if constexpr(KS == 0 && m == 7)
+                if constexpr(KS == 0 && m == 16)
                     y_open_dst(sy_c);
-                if constexpr(m % NBQ == 0)
-                    xf[slot ^ 1][m / NBQ] = fx.load(nx, m / NBQ, NKS);
-                if constexpr(m % NBP == NBP / 2)
-                    yf[slot ^ 1][m / NBP] = fy.load(ny, m / NBP, NKS);
+                // (all issued in the first three quarters of the k-step: the wait in front of the barrier that follows
+                // k-step 0 is also a wait for this wave's own LDS reads, and a read issued four MFMAs before it had not returned)
+                if constexpr(m % 6 == 0 && m / 6 < NBP)
+                    xf[slot ^ 1][m / 6] = fx.load(nx, m / 6, NKS);
+                if constexpr(m % 6 == 3 && m / 6 < NBQ)
+                    yf[slot ^ 1][m / 6] = fy.load(ny, m / 6, NKS);
                 window_slot(wv_c, std::integral_constant<int, G0 + m>{}, std::true_type{});
                 // M0 for the load in the first slot of the window that opens behind this k-step's barrier (an s_nop between
                 // the two there would hold up the MFMAs of the wave that every other wave then waits for at the next barrier)
