@@ -19,10 +19,20 @@ KDIR = os.path.join(ROOT, "hiptensor_amd", "csrc", "kernels")
 
 _ASM = {}
 
+# every translation unit a test of this file looks at: the first request compiles them all, side by side
+UNITS = ["contract_f64", "contract_c32", "contract_f16_hd", "contract_f32", "contract_c64",
+         "contract_f16_hk_kx", "contract_f16_hk_rx", "contract_bf16_hk_kx", "contract_bf16_hk_rx",
+         "contract_f16_hr192_kx", "contract_f16_hr192_rx", "contract_bf16_hr192_kx", "contract_bf16_hr192_rx"]
+
 
 def device_asm(unit, tmp_path):
     if unit not in _ASM:
-        _ASM[unit] = _compile(unit, tmp_path)
+        from concurrent.futures import ThreadPoolExecutor
+
+        todo = [u for u in dict.fromkeys([unit] + UNITS) if u not in _ASM]
+        with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+            for u, lines in zip(todo, pool.map(lambda u: _compile(u, tmp_path), todo)):
+                _ASM[u] = lines
     return _ASM[unit]
 
 
